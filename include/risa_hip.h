@@ -1,0 +1,153 @@
+/*
+ * C ABI of the gfx950 (MI355X) implementation of RISA's quantized attention path.
+ *
+ * This header replaces the nanobind module `risa_attention._C`
+ * (reference csrc/bindings.cpp:642-673) and the launcher interface behind it
+ * (reference csrc/launchers.h:8-64).  Conventions shared by every entry point:
+ *
+ *   - All pointers are device pointers on the current HIP device unless stated
+ *     otherwise.  The caller allocates and owns every buffer; the library
+ *     borrows them for the duration of the asynchronous launch, never
+ *     allocates, never synchronises and keeps no pointer after returning.
+ *   - `stream` is a hipStream_t passed as void* (PyTorch-ROCm:
+ *     torch.cuda.current_stream().cuda_stream).  Work is enqueued on it only.
+ *   - Strides are in elements, as int64_t.
+ *   - dtype codes: 0 = float32, 1 = float16, 2 = bfloat16, 3 = bool/uint8
+ *     (masks only).  Output dtype codes: 1 or 2.
+ *   - Return value 0 means success.  Any other value means the call was
+ *     rejected or a launch failed; risa_last_error() returns the message for
+ *     the calling host thread (the reference throws std::runtime_error with
+ *     the same wording).
+ */
+#ifndef RISA_HIP_H
+#define RISA_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Message of the last failed call on this host thread ("" if none). */
+const char* risa_last_error(void);
+
+/* Library/ABI version, bumped when a signature or a packed layout changes. */
+int risa_abi_version(void);
+
+/*
+ * Q/K preparation: anchor detection, rotation, per-group INT8 codes and scales.
+ * Replaces launch_quantize_qk (reference csrc/launchers.h:13-19, implemented in
+ * csrc/kernels/quantize_qk_impl.cuh:660-826) as called from risa_sdpa_quantize
+ * (csrc/bindings.cpp:254-258).
+ *   q [B,Hq,Lq,D], k [B,Hkv,Lk,D] with the given batch/head/token strides, last
+ *   dim contiguous, D in {64,128,256}, base and strides 4-element aligned.
+ *   q_int8 [B,Hq,Lq,D], k_int8 [B,Hkv,Lk,D] contiguous.
+ *   q_scale [B,Hq,ceil(Lq/128)*(D==256?64:32)], k_scale [B,Hkv,ceil(Lk/cta_k)*4].
+ *   anchor_indices int32 [B,Hkv]: receives the anchor row or -1.
+ */
+int risa_quantize_qk(const void* q, void* q_int8, float* q_scale, const void* k, void* k_int8,
+                     float* k_scale, int batch, int q_heads, int q_len, int kv_heads, int k_len,
+                     int head_dim, int cta_k, int64_t q_stride_b, int64_t q_stride_h,
+                     int64_t q_stride_n, int64_t k_stride_b, int64_t k_stride_h,
+                     int64_t k_stride_n, int input_dtype, int32_t* anchor_indices, void* stream);
+
+/*
+ * V preparation.  Replaces launch_quantize_v (reference csrc/launchers.h:30-34,
+ * csrc/kernels/quantize_v_impl.cuh:314-409).
+ *   v [B,Hkv,L,D] strided (16-byte aligned rows), out int8 [B*Hkv*D, padded] in
+ *   the packed order documented at risa_unpack_order, scale/center [B*Hkv*D],
+ *   tile_sum int32 [B*Hkv, padded/cta_k, D] (sum of the codes of each key tile,
+ *   the zero-point term of the signed P*V product; no reference counterpart),
+ *   workspace of risa_quantize_v_workspace_bytes(...) bytes.
+ */
+size_t risa_quantize_v_workspace_bytes(int batch, int heads, int length, int head_dim,
+                                       int midpoint_affine);
+int risa_quantize_v(const void* v, void* out, float* scale, float* center, int32_t* tile_sum,
+                    void* workspace, size_t workspace_bytes, int batch, int heads, int length,
+                    int head_dim, int padded_length, int cta_k, int64_t stride_b,
+                    int64_t stride_h, int64_t stride_n, int input_dtype, int midpoint_affine,
+                    void* stream);
+
+/*
+ * Tile sums of an already packed V matrix (for callers that build packed V
+ * themselves, as reference tests/cuda/test_large_offsets.py:35-36 does).
+ */
+int risa_value_tile_sums(const void* v_int8, int32_t* tile_sum, int batch_heads, int head_dim,
+                         int padded_length, int cta_k, void* stream);
+
+/*
+ * Writes into order[0..31] the token (0..31) stored at each byte position of a
+ * 32-token group of packed V: order[16*h + 4*b + r] = 8*b + 4*h + r.  Host
+ * call.  The reference's 16-token order (csrc/kernels/quantize_v_impl.cuh:47-52)
+ * follows the NVIDIA mma fragment; this one follows the 32x32x32 INT8 MFMA.
+ */
+void risa_unpack_order(int32_t* order);
+
+/*
+ * Fused attention over prepared tensors: dense, sparse-support, block-mass
+ * capture, custom / key-only masks, causal, optional LSE.  Replaces
+ * launch_attention (reference csrc/launchers.h:44-55,
+ * csrc/kernels/attention_dispatch.cu:113-296) as called from
+ * risa_sdpa_prequantized (csrc/bindings.cpp:277-461).
+ *   q_int8/k_int8 contiguous [B,H,L,D]; v_int8 [B*Hkv*D, padded];
+ *   out [B,Hq,Lq,D] fp16/bf16 with the given batch/token/head strides (last
+ *   dim contiguous); mask (nullable) expanded to [B,Hq,Lq,Lk] with its strides,
+ *   query stride 0 selecting the key-only path; sparse_row_offsets int32
+ *   [B*Hq*ceil(Lq/128)+1] and sparse_block_indices int32 (both or neither);
+ *   block_mass (nullable) float32 workspace laid out as mass
+ *   [B*Hq*ceil(Lq/128), tiles] ++ per-row full-tile stats [rows, tiles-1, 2]
+ *   (u32 sum of U8 probabilities, f32 tile maximum) ++ last-tile stats
+ *   [rows, 2] (f32, f32) ++ state [rows, 2] (m, d), rows = B*Hq*Lq
+ *   (reference attention_int8.cuh:51-143, 871-898); lse (nullable) float32
+ *   [B,Hq,Lq]; key_mask_tiles (nullable) int32 [B,Hq,tiles+1] from
+ *   risa_prepare_key_mask_tiles.
+ */
+int risa_attention(const void* q_int8, const void* k_int8, const void* v_int8, void* out,
+                   const float* q_scale, const float* k_scale, const float* v_scale,
+                   const float* v_center, const int32_t* v_tile_sum, const void* mask,
+                   int64_t mask_stride_b, int64_t mask_stride_h, int64_t mask_stride_q,
+                   int64_t mask_stride_k, int mask_dtype, int cta_k, int batch, int q_len,
+                   int k_len, int q_heads, int kv_heads, int head_dim, int64_t out_stride_b,
+                   int64_t out_stride_n, int64_t out_stride_h, float sm_scale, int out_dtype,
+                   const int32_t* sparse_row_offsets, const int32_t* sparse_block_indices,
+                   float* block_mass, int is_causal, float* lse, const int32_t* key_mask_tiles,
+                   void* stream);
+
+/*
+ * Retained-mass selection over masses already sorted in descending order.
+ * Replaces launch_select_retained_mass and retained_mass_selector_workspace_size
+ * (reference csrc/launchers.h:56-63, csrc/kernels/sparse_selection.cu:129-159).
+ * The scan needs no workspace here; the size query is kept for callers that
+ * allocate one and always returns 0.
+ */
+size_t risa_selector_workspace_size(int row_count);
+int risa_select_retained_mass(const float* sorted_mass, const int64_t* descending_indices,
+                              int32_t* counts, uint8_t* support, double* row_totals,
+                              int32_t* row_offsets, int32_t* block_indices, double* summary,
+                              int row_count, int key_blocks, double theta, void* stream);
+
+/*
+ * Active key tiles of a broadcast key mask.  Replaces
+ * launch_prepare_key_mask_tiles (reference csrc/launchers.h:39-43,
+ * csrc/kernels/key_mask_tiles.cu:45-61).
+ */
+int risa_prepare_key_mask_tiles(const void* mask, int32_t* tiles, int batch, int q_heads,
+                                int key_length, int tile_size, int64_t stride_b, int64_t stride_h,
+                                int64_t stride_k, int mask_dtype, void* stream);
+
+/*
+ * LSE anchor correction out[b,h,i] = scale * <q[b,h,i], k[b,h/G,anchor[b,h/G]]>.
+ * Replaces launch_correct_lse (reference csrc/launchers.h:9-12,
+ * csrc/kernels/lse_correction.cu:30-44).
+ */
+int risa_lse_shift(const void* q, const void* k, const int32_t* anchors, float* out, int batch,
+                   int q_heads, int kv_heads, int q_len, int head_dim, int64_t q_stride_b,
+                   int64_t q_stride_h, int64_t q_stride_n, int64_t k_stride_b, int64_t k_stride_h,
+                   int64_t k_stride_n, float scale, int dtype, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* RISA_HIP_H */

@@ -1,0 +1,57 @@
+// Per-head-dim instantiation of the attention kernel (one translation unit per
+// head dim so the variants compile in parallel).
+#pragma once
+
+#include "attention_kernel.hpp"
+
+namespace risa {
+
+template <int D> int launch_attention_variant(const KernelParams& p, int cta_k, bool fast,
+                                              bool indexed, bool capture, hipStream_t stream);
+
+template <int D, int CTA_K, bool FAST, bool INDEXED, bool CAPTURE>
+int launch_one(const KernelParams& p, hipStream_t stream) {
+  using Shape = TileShape<D, CTA_K>;
+  auto kernel = attention_kernel<D, CTA_K, FAST, INDEXED, CAPTURE>;
+  // The dynamic LDS limit is a per-device property of the function; setting it
+  // again is cheap and keeps the launcher free of host-side caches.
+  static thread_local int configured_device = -1;
+  int device = -1;
+  if (hipGetDevice(&device) != hipSuccess) return fail("risa_attention: hipGetDevice failed");
+  if (device != configured_device) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                            hipFuncAttributeMaxDynamicSharedMemorySize,
+                            Shape::kLdsBytes) != hipSuccess) {
+      return fail("risa_attention: cannot reserve " + std::to_string(Shape::kLdsBytes) +
+                  " bytes of LDS");
+    }
+    configured_device = device;
+  }
+  const dim3 grid(static_cast<unsigned>(p.n_qb) * p.q_heads * p.batch);
+  kernel<<<grid, 256, Shape::kLdsBytes, stream>>>(p);
+  return 0;
+}
+
+template <int D, int CTA_K>
+int launch_tile(const KernelParams& p, bool fast, bool indexed, bool capture, hipStream_t stream) {
+  if (fast) {
+    if (capture) return launch_one<D, CTA_K, true, false, true>(p, stream);
+    if (indexed) return launch_one<D, CTA_K, true, true, false>(p, stream);
+    return launch_one<D, CTA_K, true, false, false>(p, stream);
+  }
+  if (capture) return launch_one<D, CTA_K, false, false, true>(p, stream);
+  if (indexed) return launch_one<D, CTA_K, false, true, false>(p, stream);
+  return launch_one<D, CTA_K, false, false, false>(p, stream);
+}
+
+#define RISA_DEFINE_ATTENTION_VARIANT(DIM)                                                        \
+  template <>                                                                                     \
+  int launch_attention_variant<DIM>(const KernelParams& p, int cta_k, bool fast, bool indexed,    \
+                                    bool capture, hipStream_t stream) {                           \
+    if constexpr (DIM != 64) {                                                                    \
+      if (cta_k == 128) return launch_tile<DIM, 128>(p, fast, indexed, capture, stream);          \
+    }                                                                                             \
+    return launch_tile<DIM, 64>(p, fast, indexed, capture, stream);                               \
+  }
+
+}  // namespace risa

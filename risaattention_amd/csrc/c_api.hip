@@ -1,0 +1,231 @@
+// extern "C" entry points declared in include/risa_hip.h: argument checks that
+// the reference performs in csrc/bindings.cpp and the launchers, then dispatch.
+
+#include "../../include/risa_hip.h"
+
+#include "common.hpp"
+#include "launchers.hpp"
+
+namespace {
+
+bool aligned(const void* pointer, size_t bytes) {
+  return reinterpret_cast<uintptr_t>(pointer) % bytes == 0;
+}
+
+// A stride is irrelevant when the extent is below two.
+bool stride_multiple(int64_t stride, int extent, int64_t multiple) {
+  return extent < 2 || (stride > 0 && stride % multiple == 0);
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* risa_last_error(void) { return risa::last_error_storage().c_str(); }
+
+int risa_abi_version(void) { return 1; }
+
+int risa_quantize_qk(const void* q, void* q_int8, float* q_scale, const void* k, void* k_int8,
+                     float* k_scale, int batch, int q_heads, int q_len, int kv_heads, int k_len,
+                     int head_dim, int cta_k, int64_t q_stride_b, int64_t q_stride_h,
+                     int64_t q_stride_n, int64_t k_stride_b, int64_t k_stride_h,
+                     int64_t k_stride_n, int input_dtype, int32_t* anchor_indices, void* stream) {
+  using risa::fail;
+  if (head_dim != 64 && head_dim != 128 && head_dim != 256)
+    return fail("risa_quantize_qk: padded head_dim must be 64, 128, or 256");
+  if ((cta_k != 64 && cta_k != 128) || (head_dim == 64 && cta_k != 64))
+    return fail("risa_quantize_qk: unsupported key tile for this head_dim");
+  if (input_dtype < 0 || input_dtype > 2)
+    return fail("risa_quantize_qk: input dtype code must be 0 (fp32), 1 (fp16), or 2 (bf16)");
+  if (anchor_indices == nullptr) return fail("risa_quantize_qk: anchor_indices scratch is required");
+  if (batch <= 0 || q_heads <= 0 || kv_heads <= 0 || q_len <= 0 || k_len <= 0)
+    return fail("risa_quantize_qk: extents must be positive");
+  const size_t vector_bytes = 4 * (input_dtype == 0 ? 4 : 2);
+  const bool q_ok = aligned(q, vector_bytes) && stride_multiple(q_stride_b, batch, 4) &&
+                    stride_multiple(q_stride_h, q_heads, 4) && stride_multiple(q_stride_n, q_len, 4);
+  const bool k_ok = aligned(k, vector_bytes) && stride_multiple(k_stride_b, batch, 4) &&
+                    stride_multiple(k_stride_h, kv_heads, 4) && stride_multiple(k_stride_n, k_len, 4);
+  if (!q_ok || !k_ok)
+    return fail("risa_quantize_qk: Q/K base pointers and batch/head/sequence strides must "
+                "preserve 4-element alignment");
+  risa::QkArgs a{};
+  a.q = q;
+  a.q_codes = static_cast<int8_t*>(q_int8);
+  a.q_scale = q_scale;
+  a.k = k;
+  a.k_codes = static_cast<int8_t*>(k_int8);
+  a.k_scale = k_scale;
+  a.anchors = anchor_indices;
+  a.batch = batch;
+  a.q_heads = q_heads;
+  a.q_len = q_len;
+  a.kv_heads = kv_heads;
+  a.k_len = k_len;
+  a.head_dim = head_dim;
+  a.cta_k = cta_k;
+  a.dtype = input_dtype;
+  a.q_stride_b = q_stride_b;
+  a.q_stride_h = q_stride_h;
+  a.q_stride_n = q_stride_n;
+  a.k_stride_b = k_stride_b;
+  a.k_stride_h = k_stride_h;
+  a.k_stride_n = k_stride_n;
+  return risa::launch_quantize_qk(a, static_cast<hipStream_t>(stream));
+}
+
+size_t risa_quantize_v_workspace_bytes(int batch, int heads, int length, int head_dim,
+                                       int midpoint_affine) {
+  return risa::value_workspace_bytes(batch, heads, length, head_dim, midpoint_affine != 0);
+}
+
+int risa_quantize_v(const void* v, void* out, float* scale, float* center, int32_t* tile_sum,
+                    void* workspace, size_t workspace_bytes, int batch, int heads, int length,
+                    int head_dim, int padded_length, int cta_k, int64_t stride_b,
+                    int64_t stride_h, int64_t stride_n, int input_dtype, int midpoint_affine,
+                    void* stream) {
+  using risa::fail;
+  if (head_dim != 64 && head_dim != 128 && head_dim != 256)
+    return fail("risa_quantize_v: padded head_dim must be 64, 128, or 256");
+  if (cta_k != 64 && cta_k != 128) return fail("risa_quantize_v: cta_k must be 64 or 128");
+  if (input_dtype < 0 || input_dtype > 2) return fail("risa_quantize_v: unsupported input dtype");
+  if (batch <= 0 || heads <= 0 || length <= 0) return fail("risa_quantize_v: extents must be positive");
+  if (padded_length != (length + cta_k - 1) / cta_k * cta_k)
+    return fail("risa_quantize_v: padded length must round the sequence up to the key tile");
+  const int64_t per_16_bytes = input_dtype == 0 ? 4 : 8;
+  if (!aligned(v, 16) || !stride_multiple(stride_b, batch, per_16_bytes) ||
+      !stride_multiple(stride_h, heads, per_16_bytes) ||
+      !stride_multiple(stride_n, length, per_16_bytes))
+    return fail("risa_quantize_v: V base pointer and batch/head/sequence strides must be "
+                "16-byte aligned");
+  if (tile_sum == nullptr || workspace == nullptr)
+    return fail("risa_quantize_v: tile sums and workspace are required");
+  risa::ValueArgs a{};
+  a.v = v;
+  a.codes = static_cast<int8_t*>(out);
+  a.scale = scale;
+  a.center = center;
+  a.tile_sum = tile_sum;
+  a.workspace = workspace;
+  a.workspace_bytes = workspace_bytes;
+  a.batch = batch;
+  a.heads = heads;
+  a.length = length;
+  a.head_dim = head_dim;
+  a.padded = padded_length;
+  a.cta_k = cta_k;
+  a.dtype = input_dtype;
+  a.stride_b = stride_b;
+  a.stride_h = stride_h;
+  a.stride_n = stride_n;
+  a.midpoint_affine = midpoint_affine != 0;
+  return risa::launch_quantize_v(a, static_cast<hipStream_t>(stream));
+}
+
+int risa_value_tile_sums(const void* v_int8, int32_t* tile_sum, int batch_heads, int head_dim,
+                         int padded_length, int cta_k, void* stream) {
+  if ((cta_k != 64 && cta_k != 128) || padded_length % cta_k != 0 || head_dim <= 0)
+    return risa::fail("risa_value_tile_sums: unsupported tile or padding");
+  return risa::launch_value_tile_sums(static_cast<const int8_t*>(v_int8), tile_sum, batch_heads,
+                                      head_dim, padded_length, cta_k,
+                                      static_cast<hipStream_t>(stream));
+}
+
+void risa_unpack_order(int32_t* order) {
+  for (int token = 0; token < 32; ++token) order[risa::packed_value_position(token)] = token;
+}
+
+int risa_attention(const void* q_int8, const void* k_int8, const void* v_int8, void* out,
+                   const float* q_scale, const float* k_scale, const float* v_scale,
+                   const float* v_center, const int32_t* v_tile_sum, const void* mask,
+                   int64_t mask_stride_b, int64_t mask_stride_h, int64_t mask_stride_q,
+                   int64_t mask_stride_k, int mask_dtype, int cta_k, int batch, int q_len,
+                   int k_len, int q_heads, int kv_heads, int head_dim, int64_t out_stride_b,
+                   int64_t out_stride_n, int64_t out_stride_h, float sm_scale, int out_dtype,
+                   const int32_t* sparse_row_offsets, const int32_t* sparse_block_indices,
+                   float* block_mass, int is_causal, float* lse, const int32_t* key_mask_tiles,
+                   void* stream) {
+  using risa::fail;
+  if (out_dtype != 1 && out_dtype != 2)
+    return fail("risa_attention: output dtype code must be 1 (fp16) or 2 (bf16)");
+  if (mask != nullptr && (mask_dtype < 0 || mask_dtype > 3))
+    return fail("risa_attention: attention mask must be bool, float16, bfloat16, or float32");
+  if (batch <= 0 || q_heads <= 0 || kv_heads <= 0 || q_len <= 0 || k_len <= 0)
+    return fail("risa_attention: extents must be positive");
+  if (out_stride_n % 4 != 0 || out_stride_h % 4 != 0 || out_stride_b % 4 != 0 || !aligned(out, 8))
+    return fail("risa_attention: output rows must be 8-byte aligned");
+  risa::AttentionArgs a{};
+  a.q = static_cast<const int8_t*>(q_int8);
+  a.k = static_cast<const int8_t*>(k_int8);
+  a.v = static_cast<const int8_t*>(v_int8);
+  a.out = out;
+  a.q_scale = q_scale;
+  a.k_scale = k_scale;
+  a.v_scale = v_scale;
+  a.v_center = v_center;
+  a.v_tile_sum = v_tile_sum;
+  a.mask = mask;
+  a.mask_stride_b = mask_stride_b;
+  a.mask_stride_h = mask_stride_h;
+  a.mask_stride_q = mask_stride_q;
+  a.mask_stride_k = mask_stride_k;
+  a.mask_dtype = mask_dtype;
+  a.cta_k = cta_k;
+  a.batch = batch;
+  a.q_len = q_len;
+  a.k_len = k_len;
+  a.q_heads = q_heads;
+  a.kv_heads = kv_heads;
+  a.head_dim = head_dim;
+  a.out_stride_b = out_stride_b;
+  a.out_stride_n = out_stride_n;
+  a.out_stride_h = out_stride_h;
+  a.sm_scale = sm_scale;
+  a.out_dtype = out_dtype;
+  a.sparse_row_offsets = sparse_row_offsets;
+  a.sparse_block_indices = sparse_block_indices;
+  a.block_mass = block_mass;
+  a.is_causal = is_causal != 0;
+  a.lse = lse;
+  a.key_mask_tiles = key_mask_tiles;
+  return risa::launch_attention(a, static_cast<hipStream_t>(stream));
+}
+
+size_t risa_selector_workspace_size(int) { return 0; }
+
+int risa_select_retained_mass(const float* sorted_mass, const int64_t* descending_indices,
+                              int32_t* counts, uint8_t* support, double* row_totals,
+                              int32_t* row_offsets, int32_t* block_indices, double* summary,
+                              int row_count, int key_blocks, double theta, void* stream) {
+  if (row_count <= 0 || key_blocks <= 0)
+    return risa::fail("risa_select_retained_mass: invalid shape, dtype, or stride");
+  if (static_cast<int64_t>(row_count) * key_blocks > INT32_MAX)
+    return risa::fail("risa_select_retained_mass: matrix is too large");
+  risa::SelectArgs a{sorted_mass, descending_indices, counts,   support,    row_totals, row_offsets,
+                     block_indices, summary,          row_count, key_blocks, theta};
+  return risa::launch_select_retained_mass(a, static_cast<hipStream_t>(stream));
+}
+
+int risa_prepare_key_mask_tiles(const void* mask, int32_t* tiles, int batch, int q_heads,
+                                int key_length, int tile_size, int64_t stride_b, int64_t stride_h,
+                                int64_t stride_k, int mask_dtype, void* stream) {
+  if (tile_size != 64 && tile_size != 128)
+    return risa::fail("risa_prepare_key_mask_tiles requires an expanded broadcast key mask");
+  if (mask_dtype < 0 || mask_dtype > 3)
+    return risa::fail("risa_prepare_key_mask_tiles requires a supported mask dtype");
+  return risa::launch_key_mask_tiles(mask, tiles, batch, q_heads, key_length, tile_size, stride_b,
+                                     stride_h, stride_k, mask_dtype,
+                                     static_cast<hipStream_t>(stream));
+}
+
+int risa_lse_shift(const void* q, const void* k, const int32_t* anchors, float* out, int batch,
+                   int q_heads, int kv_heads, int q_len, int head_dim, int64_t q_stride_b,
+                   int64_t q_stride_h, int64_t q_stride_n, int64_t k_stride_b, int64_t k_stride_h,
+                   int64_t k_stride_n, float scale, int dtype, void* stream) {
+  if (dtype < 0 || dtype > 2) return risa::fail("risa_lse_shift: unsupported dtype");
+  risa::LseShiftArgs a{q,          k,          anchors,    out,        batch,      q_heads,
+                       kv_heads,   q_len,      head_dim,   dtype,      q_stride_b, q_stride_h,
+                       q_stride_n, k_stride_b, k_stride_h, k_stride_n, scale};
+  return risa::launch_lse_shift(a, static_cast<hipStream_t>(stream));
+}
+
+}  // extern "C"

@@ -1,0 +1,150 @@
+// Shared device/host helpers for the gfx950 kernels of the quantized attention path.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+#include <cstdio>
+#include <cstring>
+#include <string>
+
+namespace risa {
+
+// ---------------------------------------------------------------------------
+// Error reporting across the C boundary: entry points return 0 on success and
+// a non-zero code otherwise; the message is kept per host thread.
+// ---------------------------------------------------------------------------
+inline std::string& last_error_storage() {
+  static thread_local std::string message;
+  return message;
+}
+
+inline int fail(const std::string& message) {
+  last_error_storage() = message;
+  return 1;
+}
+
+inline int check_launch(const char* what) {
+  const hipError_t error = hipGetLastError();
+  if (error != hipSuccess) {
+    return fail(std::string(what) + " launch failed: " + hipGetErrorString(error));
+  }
+  return 0;
+}
+
+// dtype codes shared with the Python side: 0 = float32, 1 = float16,
+// 2 = bfloat16, 3 = bool/uint8 (masks only).
+constexpr int kF32 = 0;
+constexpr int kF16 = 1;
+constexpr int kBF16 = 2;
+constexpr int kBool = 3;
+
+constexpr int kWave = 64;
+
+// ---------------------------------------------------------------------------
+// Typed loads that widen to binary32 exactly.
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ float bf16_bits_to_float(uint32_t bits16) {
+  return __uint_as_float(bits16 << 16);
+}
+
+__device__ __forceinline__ float f16_bits_to_float(uint32_t bits16) {
+  const _Float16 value = __builtin_bit_cast(_Float16, static_cast<uint16_t>(bits16));
+  return static_cast<float>(value);
+}
+
+template <int DT> struct Element;
+template <> struct Element<kF32> {
+  using type = float;
+  static constexpr int bytes = 4;
+};
+template <> struct Element<kF16> {
+  using type = uint16_t;
+  static constexpr int bytes = 2;
+};
+template <> struct Element<kBF16> {
+  using type = uint16_t;
+  static constexpr int bytes = 2;
+};
+
+// Four consecutive elements starting at element offset `offset` (which the
+// callers keep a multiple of four elements and 4-element aligned in memory).
+template <int DT>
+__device__ __forceinline__ void load4(const void* base, int64_t offset, float out[4]) {
+  if constexpr (DT == kF32) {
+    const float4 raw = *reinterpret_cast<const float4*>(static_cast<const float*>(base) + offset);
+    out[0] = raw.x;
+    out[1] = raw.y;
+    out[2] = raw.z;
+    out[3] = raw.w;
+  } else {
+    const uint2 raw = *reinterpret_cast<const uint2*>(static_cast<const uint16_t*>(base) + offset);
+    if constexpr (DT == kBF16) {
+      out[0] = bf16_bits_to_float(raw.x & 0xffffu);
+      out[1] = bf16_bits_to_float(raw.x >> 16);
+      out[2] = bf16_bits_to_float(raw.y & 0xffffu);
+      out[3] = bf16_bits_to_float(raw.y >> 16);
+    } else {
+      out[0] = f16_bits_to_float(raw.x & 0xffffu);
+      out[1] = f16_bits_to_float(raw.x >> 16);
+      out[2] = f16_bits_to_float(raw.y & 0xffffu);
+      out[3] = f16_bits_to_float(raw.y >> 16);
+    }
+  }
+}
+
+// Eight consecutive elements (16-byte aligned for 16-bit types, 32 for fp32).
+template <int DT>
+__device__ __forceinline__ void load8(const void* base, int64_t offset, float out[8]) {
+  if constexpr (DT == kF32) {
+    load4<DT>(base, offset, out);
+    load4<DT>(base, offset + 4, out + 4);
+  } else {
+    const uint4 raw = *reinterpret_cast<const uint4*>(static_cast<const uint16_t*>(base) + offset);
+    const uint32_t words[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      if constexpr (DT == kBF16) {
+        out[2 * i] = bf16_bits_to_float(words[i] & 0xffffu);
+        out[2 * i + 1] = bf16_bits_to_float(words[i] >> 16);
+      } else {
+        out[2 * i] = f16_bits_to_float(words[i] & 0xffffu);
+        out[2 * i + 1] = f16_bits_to_float(words[i] >> 16);
+      }
+    }
+  }
+}
+
+template <int DT>
+__device__ __forceinline__ float load1(const void* base, int64_t offset) {
+  if constexpr (DT == kF32) {
+    return static_cast<const float*>(base)[offset];
+  } else if constexpr (DT == kBF16) {
+    return bf16_bits_to_float(static_cast<const uint16_t*>(base)[offset]);
+  } else {
+    return f16_bits_to_float(static_cast<const uint16_t*>(base)[offset]);
+  }
+}
+
+// Round to nearest even, saturate to the signed 8-bit range, NaN -> 0.
+__device__ __forceinline__ int quantize_s8(float value) {
+  float rounded = __builtin_rintf(value);
+  rounded = rounded != rounded ? 0.0f : rounded;
+  rounded = __builtin_fminf(__builtin_fmaxf(rounded, -128.0f), 127.0f);
+  return static_cast<int>(rounded);
+}
+
+__device__ __forceinline__ uint32_t pack_s8x4(int a, int b, int c, int d) {
+  return (static_cast<uint32_t>(a) & 0xffu) | ((static_cast<uint32_t>(b) & 0xffu) << 8) |
+         ((static_cast<uint32_t>(c) & 0xffu) << 16) | ((static_cast<uint32_t>(d) & 0xffu) << 24);
+}
+
+// Position of token `t` (0..31) inside its 32-token group of the packed V
+// matrix.  Byte p = 16*h + 4*b + r holds token 8*b + 4*h + r, so the sixteen
+// bytes a lane of half h feeds to the 32x32x32 INT8 MFMA are the sixteen keys
+// the same lane holds in the accumulator of the transposed score tile.
+__host__ __device__ __forceinline__ int packed_value_position(int t) {
+  return ((t >> 2) & 1) * 16 + (t >> 3) * 4 + (t & 3);
+}
+
+}  // namespace risa

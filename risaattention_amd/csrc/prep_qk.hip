@@ -1,0 +1,428 @@
+// Q/K preparation for gfx950: K anchor detection, sign-diagonal + Walsh-Hadamard
+// rotation and per-group signed INT8 quantisation.
+//
+// Numerical contract (bit-exact): reference csrc/kernels/quantize_qk_impl.cuh
+//   detect_k_anchor :442-577, rotations :69-147, process_q :153-269,
+//   process_k :278-426, dispatch by (head_dim, key_length) :769-811.
+// The reference assigns one scale group to a 32-lane warp in which every lane
+// owns four adjacent channels.  Here one 32-lane half of a 64-wide wavefront
+// plays that role, so a wavefront quantises two scale groups at once and the
+// butterfly order (4-point local stage, then lane bits 1, 2, 4, 8, 16) is the
+// reference's.  All arithmetic is IEEE binary32 without contraction.
+
+#include "common.hpp"
+#include "launchers.hpp"
+
+namespace risa {
+namespace {
+
+constexpr int kRot4 = 4;
+constexpr int kRot64 = 64;
+constexpr int kRot128Signed = 128;
+constexpr int kRot128Plain = 129;
+
+__device__ __forceinline__ void rotate4(float* v) {
+  const float a0 = v[0] + v[1];
+  const float a1 = v[0] - v[1];
+  const float a2 = v[2] + v[3];
+  const float a3 = v[2] - v[3];
+  v[0] = (a0 + a2) * 0.5f;
+  v[1] = (a1 + a3) * 0.5f;
+  v[2] = (a0 - a2) * 0.5f;
+  v[3] = (a1 - a3) * 0.5f;
+}
+
+// Channel c keeps its sign when bit c%32 of word c/32 is set and is negated
+// otherwise; `sub` is the lane inside the 32-lane half, owning channels 4*sub..
+__device__ __forceinline__ void apply_sign_diagonal(float* v, int sub) {
+  const uint32_t words[4] = {0x1035997bu, 0x8087f5eeu, 0xee2e4e1au, 0x71132418u};
+  const uint32_t word = words[sub >> 3];
+  const int shift = (sub & 7) * 4;
+#pragma unroll
+  for (int c = 0; c < 4; ++c) {
+    const uint32_t flip = ((word >> (shift + c)) & 1u) ^ 1u;
+    v[c] = __uint_as_float(__float_as_uint(v[c]) ^ (flip << 31));
+  }
+}
+
+template <int LANES> __device__ __forceinline__ void lane_butterflies(float* v, int sub) {
+#pragma unroll
+  for (int bit = 1; bit < LANES; bit <<= 1) {
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      const float other = __shfl_xor(v[c], bit);
+      v[c] = (sub & bit) ? other - v[c] : v[c] + other;
+    }
+  }
+}
+
+template <int ROT> __device__ __forceinline__ void rotate(float* v, int sub) {
+  if constexpr (ROT == kRot128Signed) {
+    apply_sign_diagonal(v, sub);
+  }
+  rotate4(v);
+  if constexpr (ROT == kRot64) {
+    lane_butterflies<16>(v, sub & 15);
+#pragma unroll
+    for (int c = 0; c < 4; ++c) v[c] *= 0.25f;
+  } else if constexpr (ROT == kRot128Signed || ROT == kRot128Plain) {
+    lane_butterflies<32>(v, sub);
+#pragma unroll
+    for (int c = 0; c < 4; ++c) v[c] *= 0.1767766952966369f;
+  }
+}
+
+__device__ __forceinline__ float half_wave_max(float value) {
+#pragma unroll
+  for (int offset = 16; offset > 0; offset >>= 1) {
+    value = __builtin_fmaxf(value, __shfl_xor(value, offset));
+  }
+  return value;
+}
+
+// One scale group handled by one 32-lane half: NTOK tokens x DK channels.
+// `token_of(i)` gives the i-th token of the group.
+template <int DT, int DK, int ROT, int NTOK, typename TokenOf>
+__device__ __forceinline__ void quantize_group(const void* in, int64_t in_base, int64_t stride_n,
+                                               int8_t* out, float* scale_slot, int length, int sub,
+                                               const float* bias, TokenOf token_of) {
+  constexpr int CT = DK == 256 ? 2 : 1;
+  float v[CT][NTOK][4];
+#pragma unroll
+  for (int tile = 0; tile < CT; ++tile) {
+    const int ch = tile * 128 + sub * 4;
+#pragma unroll
+    for (int i = 0; i < NTOK; ++i) {
+      const int n = token_of(i);
+      v[tile][i][0] = v[tile][i][1] = v[tile][i][2] = v[tile][i][3] = 0.0f;
+      if (ch < DK && n < length) {
+        load4<DT>(in, in_base + static_cast<int64_t>(n) * stride_n + ch, v[tile][i]);
+        if (bias != nullptr) {
+#pragma unroll
+          for (int c = 0; c < 4; ++c) v[tile][i][c] -= bias[tile * 4 + c];
+        }
+      }
+    }
+  }
+  float mx = 0.0f;
+#pragma unroll
+  for (int tile = 0; tile < CT; ++tile) {
+#pragma unroll
+    for (int i = 0; i < NTOK; ++i) {
+      rotate<ROT>(v[tile][i], sub);
+#pragma unroll
+      for (int c = 0; c < 4; ++c) mx = __builtin_fmaxf(mx, __builtin_fabsf(v[tile][i][c]));
+    }
+  }
+  mx = half_wave_max(mx);
+  const float scale = mx / 127.0f + 1e-7f;
+  const float inverse = 1.0f / scale;
+  if (sub == 0) *scale_slot = scale;
+#pragma unroll
+  for (int tile = 0; tile < CT; ++tile) {
+    const int ch = tile * 128 + sub * 4;
+#pragma unroll
+    for (int i = 0; i < NTOK; ++i) {
+      const int n = token_of(i);
+      if (ch < DK && n < length) {
+        const uint32_t packed =
+            pack_s8x4(quantize_s8(v[tile][i][0] * inverse), quantize_s8(v[tile][i][1] * inverse),
+                      quantize_s8(v[tile][i][2] * inverse), quantize_s8(v[tile][i][3] * inverse));
+        *reinterpret_cast<uint32_t*>(out + static_cast<int64_t>(n) * DK + ch) = packed;
+      }
+    }
+  }
+}
+
+// grid (slices, Hq, B), 256 threads: eight 32-lane halves = the eight scale
+// groups (token index mod 8) of one W-row slice, W = 32 (16 for head_dim 256).
+template <int DT, int DK, int ROT>
+__global__ __launch_bounds__(256) void quantize_q_kernel(const void* __restrict__ q,
+                                                         int8_t* __restrict__ codes,
+                                                         float* __restrict__ scales, int length,
+                                                         int heads, int scales_per_head,
+                                                         int64_t stride_b, int64_t stride_h,
+                                                         int64_t stride_n) {
+  constexpr int W = DK == 256 ? 16 : 32;
+  constexpr int NR = W / 8;
+  const int slice = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+  const int sub = threadIdx.x & 31;
+  const int group = threadIdx.x >> 5;
+  const int base = slice * W + group;
+  const int64_t in_base = static_cast<int64_t>(b) * stride_b + static_cast<int64_t>(h) * stride_h;
+  const int64_t bh = static_cast<int64_t>(b) * heads + h;
+  quantize_group<DT, DK, ROT, NR>(q, in_base, stride_n, codes + bh * length * DK,
+                                  scales + bh * scales_per_head + slice * 8 + group, length, sub,
+                                  nullptr, [base](int i) { return base + i * 8; });
+}
+
+// grid (key tiles, Hkv, B), 128 threads: four 32-lane halves = the four scale
+// groups ((token mod 8) / 2) of one key tile of CTA_K tokens.
+template <int DT, int DK, int CTA_K, int ROT>
+__global__ __launch_bounds__(128) void quantize_k_kernel(const void* __restrict__ k,
+                                                         int8_t* __restrict__ codes,
+                                                         float* __restrict__ scales,
+                                                         const int* __restrict__ anchors, int length,
+                                                         int heads, int scales_per_head,
+                                                         int64_t stride_b, int64_t stride_h,
+                                                         int64_t stride_n) {
+  constexpr int CT = DK == 256 ? 2 : 1;
+  constexpr int NTOK = CTA_K / 4;
+  const int tile = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+  const int sub = threadIdx.x & 31;
+  const int group = threadIdx.x >> 5;
+  const int64_t in_base = static_cast<int64_t>(b) * stride_b + static_cast<int64_t>(h) * stride_h;
+  const int64_t bh = static_cast<int64_t>(b) * heads + h;
+  const int anchor = anchors[b * heads + h];
+  float bias[CT * 4];
+#pragma unroll
+  for (int t = 0; t < CT; ++t) {
+    const int ch = t * 128 + sub * 4;
+    bias[t * 4] = bias[t * 4 + 1] = bias[t * 4 + 2] = bias[t * 4 + 3] = 0.0f;
+    if (anchor >= 0 && ch < DK) {
+      load4<DT>(k, in_base + static_cast<int64_t>(anchor) * stride_n + ch, bias + t * 4);
+    }
+  }
+  const int first = tile * CTA_K + group * 2;
+  quantize_group<DT, DK, ROT, NTOK>(k, in_base, stride_n, codes + bh * length * DK,
+                                    scales + bh * scales_per_head + tile * 4 + group, length, sub,
+                                    anchor >= 0 ? bias : nullptr,
+                                    [first](int i) { return first + (i >> 1) * 8 + (i & 1); });
+}
+
+// ---------------------------------------------------------------------------
+// Anchor detector: grid (Hkv, B), 128 threads.  Thread t owns channels t and
+// t+128; partial sums are combined by a 32-lane shuffle-down tree and then the
+// four 32-lane segments are added in order, which is the reference's order.
+// ---------------------------------------------------------------------------
+constexpr int kSamples = 9;
+
+__device__ __forceinline__ float segment_down_sum(float value) {
+#pragma unroll
+  for (int offset = 16; offset > 0; offset >>= 1) value += __shfl_down(value, offset, 32);
+  return value;
+}
+__device__ __forceinline__ float segment_down_max(float value) {
+#pragma unroll
+  for (int offset = 16; offset > 0; offset >>= 1)
+    value = __builtin_fmaxf(value, __shfl_down(value, offset, 32));
+  return value;
+}
+
+template <int DT>
+__global__ __launch_bounds__(128) void detect_anchor_kernel(const void* __restrict__ k,
+                                                            int* __restrict__ anchors, int length,
+                                                            int dim, int heads, int64_t stride_b,
+                                                            int64_t stride_h, int64_t stride_n) {
+  __shared__ float samples[kSamples * 256];
+  __shared__ float seg_energy[4], seg_max[4], seg_dist[kSamples][4], seg_best_energy[4],
+      seg_best_max[4];
+  __shared__ int chosen;
+  const int h = blockIdx.x, b = blockIdx.y;
+  const int tid = threadIdx.x, sub = tid & 31, seg = tid >> 5;
+  const int64_t base = static_cast<int64_t>(b) * stride_b + static_cast<int64_t>(h) * stride_h;
+  for (int index = tid; index < kSamples * dim; index += 128) {
+    const int s = index / dim;
+    const int c = index - s * dim;
+    const int64_t row = static_cast<int64_t>(s) * (length - 1) / (kSamples - 1);
+    samples[index] = load1<DT>(k, base + row * stride_n + c);
+  }
+  __syncthreads();
+
+  float energy = 0.0f, peak = 0.0f, dist[kSamples];
+#pragma unroll
+  for (int c = 0; c < kSamples; ++c) dist[c] = 0.0f;
+  for (int channel = tid; channel < dim; channel += 128) {
+    float sum = 0.0f;
+#pragma unroll
+    for (int s = 0; s < kSamples; ++s) {
+      const float value = samples[s * dim + channel];
+      energy = __builtin_fmaf(value, value, energy);
+      peak = __builtin_fmaxf(peak, __builtin_fabsf(value));
+      sum += value;
+    }
+#pragma unroll
+    for (int c = 0; c < kSamples; ++c) {
+      const float d = 9.0f * samples[c * dim + channel] - sum;
+      dist[c] = __builtin_fmaf(d, d, dist[c]);
+    }
+  }
+  energy = segment_down_sum(energy);
+  peak = segment_down_max(peak);
+#pragma unroll
+  for (int c = 0; c < kSamples; ++c) dist[c] = segment_down_sum(dist[c]);
+  if (sub == 0) {
+    seg_energy[seg] = energy;
+    seg_max[seg] = peak;
+#pragma unroll
+    for (int c = 0; c < kSamples; ++c) seg_dist[c][seg] = dist[c];
+  }
+  __syncthreads();
+  if (tid == 0) {
+    int best = 0;
+    float best_distance = 3.402823466e+38f;
+    for (int c = 0; c < kSamples; ++c) {
+      float total = 0.0f;
+      for (int w = 0; w < 4; ++w) total += seg_dist[c][w];
+      if (total < best_distance) {
+        best = c;
+        best_distance = total;
+      }
+    }
+    chosen = best;
+  }
+  __syncthreads();
+  const int best = chosen;
+  float best_energy = 0.0f, best_peak = 0.0f;
+  for (int channel = tid; channel < dim; channel += 128) {
+    const float anchor = samples[best * dim + channel];
+#pragma unroll
+    for (int s = 0; s < kSamples; ++s) {
+      const float residual = samples[s * dim + channel] - anchor;
+      best_energy = __builtin_fmaf(residual, residual, best_energy);
+      best_peak = __builtin_fmaxf(best_peak, __builtin_fabsf(residual));
+    }
+  }
+  best_energy = segment_down_sum(best_energy);
+  best_peak = segment_down_max(best_peak);
+  if (sub == 0) {
+    seg_best_energy[seg] = best_energy;
+    seg_best_max[seg] = best_peak;
+  }
+  __syncthreads();
+  if (tid == 0) {
+    float e0 = 0.0f, m0 = 0.0f, e1 = 0.0f, m1 = 0.0f;
+    for (int w = 0; w < 4; ++w) {
+      e0 += seg_energy[w];
+      m0 = __builtin_fmaxf(m0, seg_max[w]);
+      e1 += seg_best_energy[w];
+      m1 = __builtin_fmaxf(m1, seg_best_max[w]);
+    }
+    const bool improves = e1 < e0 && m1 <= m0 * 1.125f;
+    anchors[b * heads + h] =
+        improves ? static_cast<int>(static_cast<int64_t>(best) * (length - 1) / (kSamples - 1)) : -1;
+  }
+}
+
+template <int DT, int DK, int ROT>
+void launch_q(const QkArgs& a, hipStream_t stream) {
+  constexpr int W = DK == 256 ? 16 : 32;
+  const int slices = (a.q_len + 127) / 128 * (128 / W);
+  dim3 grid(slices, a.q_heads, a.batch);
+  quantize_q_kernel<DT, DK, ROT><<<grid, 256, 0, stream>>>(a.q, a.q_codes, a.q_scale, a.q_len,
+                                                           a.q_heads, slices * 8, a.q_stride_b,
+                                                           a.q_stride_h, a.q_stride_n);
+}
+
+template <int DT, int DK, int CTA_K, int ROT>
+void launch_k(const QkArgs& a, hipStream_t stream) {
+  const int tiles = (a.k_len + CTA_K - 1) / CTA_K;
+  dim3 grid(tiles, a.kv_heads, a.batch);
+  quantize_k_kernel<DT, DK, CTA_K, ROT><<<grid, 128, 0, stream>>>(
+      a.k, a.k_codes, a.k_scale, a.anchors, a.k_len, a.kv_heads, tiles * 4, a.k_stride_b,
+      a.k_stride_h, a.k_stride_n);
+}
+
+template <int DT, int DK, int ROT>
+void launch_qk_rot(const QkArgs& a, hipStream_t stream) {
+  launch_q<DT, DK, ROT>(a, stream);
+  if constexpr (DK == 64) {
+    launch_k<DT, DK, 64, ROT>(a, stream);
+  } else {
+    if (a.cta_k == 128)
+      launch_k<DT, DK, 128, ROT>(a, stream);
+    else
+      launch_k<DT, DK, 64, ROT>(a, stream);
+  }
+}
+
+template <int DT> void launch_qk_dtype(const QkArgs& a, hipStream_t stream) {
+  dim3 grid(a.kv_heads, a.batch);
+  detect_anchor_kernel<DT><<<grid, 128, 0, stream>>>(a.k, a.anchors, a.k_len, a.head_dim,
+                                                     a.kv_heads, a.k_stride_b, a.k_stride_h,
+                                                     a.k_stride_n);
+  const bool short_keys = a.k_len <= 256;
+  if (a.head_dim == 64) {
+    if (short_keys)
+      launch_qk_rot<DT, 64, kRot4>(a, stream);
+    else
+      launch_qk_rot<DT, 64, kRot64>(a, stream);
+  } else if (a.head_dim == 128) {
+    if (short_keys)
+      launch_qk_rot<DT, 128, kRot4>(a, stream);
+    else
+      launch_qk_rot<DT, 128, kRot128Signed>(a, stream);
+  } else {
+    if (short_keys)
+      launch_qk_rot<DT, 256, kRot4>(a, stream);
+    else
+      launch_qk_rot<DT, 256, kRot128Plain>(a, stream);
+  }
+}
+
+}  // namespace
+
+int launch_quantize_qk(const QkArgs& a, hipStream_t stream) {
+  if (a.dtype == kF32)
+    launch_qk_dtype<kF32>(a, stream);
+  else if (a.dtype == kF16)
+    launch_qk_dtype<kF16>(a, stream);
+  else
+    launch_qk_dtype<kBF16>(a, stream);
+  return check_launch("risa_quantize_qk");
+}
+
+// ---------------------------------------------------------------------------
+// LSE anchor correction: out[b,h,i] = scale * <q[b,h,i], k[b,h/G,anchor]>,
+// products and sums kept separate, lanes stride 32 over channels, shuffle-down
+// tree (reference csrc/kernels/lse_correction.cu:4-28).
+// grid (ceil(Lq/8), Hq, B), 256 threads: one 32-lane half per query row.
+// ---------------------------------------------------------------------------
+namespace {
+template <int DT>
+__global__ __launch_bounds__(256) void lse_shift_kernel(const void* __restrict__ q,
+                                                        const void* __restrict__ k,
+                                                        const int* __restrict__ anchors,
+                                                        float* __restrict__ out, int q_heads,
+                                                        int kv_heads, int q_len, int dim,
+                                                        int64_t qb, int64_t qh, int64_t qn,
+                                                        int64_t kb, int64_t kh, int64_t kn,
+                                                        float scale) {
+  const int sub = threadIdx.x & 31;
+  const int row = blockIdx.x * 8 + (threadIdx.x >> 5);
+  const int head = blockIdx.y, batch = blockIdx.z;
+  if (row >= q_len) return;
+  const int kv_head = head / (q_heads / kv_heads);
+  const int anchor = anchors[batch * kv_heads + kv_head];
+  float sum = 0.0f;
+  if (anchor >= 0) {
+    const int64_t q_base = batch * qb + head * qh + static_cast<int64_t>(row) * qn;
+    const int64_t k_base = batch * kb + kv_head * kh + static_cast<int64_t>(anchor) * kn;
+    for (int d = sub; d < dim; d += 32) {
+      const float product = load1<DT>(q, q_base + d) * load1<DT>(k, k_base + d);
+      sum = sum + product;
+    }
+    sum = segment_down_sum(sum);
+  }
+  if (sub == 0) out[(static_cast<int64_t>(batch) * q_heads + head) * q_len + row] = sum * scale;
+}
+}  // namespace
+
+int launch_lse_shift(const LseShiftArgs& a, hipStream_t stream) {
+  dim3 grid((a.q_len + 7) / 8, a.q_heads, a.batch);
+#define RISA_LSE(DTV)                                                                             \
+  lse_shift_kernel<DTV><<<grid, 256, 0, stream>>>(a.q, a.k, a.anchors, a.out, a.q_heads,           \
+                                                  a.kv_heads, a.q_len, a.head_dim, a.q_stride_b,   \
+                                                  a.q_stride_h, a.q_stride_n, a.k_stride_b,        \
+                                                  a.k_stride_h, a.k_stride_n, a.scale)
+  if (a.dtype == kF32)
+    RISA_LSE(kF32);
+  else if (a.dtype == kF16)
+    RISA_LSE(kF16);
+  else
+    RISA_LSE(kBF16);
+#undef RISA_LSE
+  return check_launch("risa_lse_shift");
+}
+
+}  // namespace risa

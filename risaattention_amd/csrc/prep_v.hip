@@ -1,0 +1,365 @@
+// V preparation for gfx950: per-channel range, signed INT8 codes in the packed
+// MFMA order, per-tile code sums (zero-point term of the signed P·V product) and
+// the residual-corrected centre of the midpoint_affine mode.
+//
+// Numerical contract (bit-exact): reference csrc/kernels/quantize_v_impl.cuh:83-292
+// (range :104-186, codes :203-246, residual centre :248-275) and the schedule
+// choice of launch_quantize_v :356-401 (512 summation threads, 128 when L <= 256).
+//
+// The reference runs one block per (batch, head, 8 channels) that walks the whole
+// sequence twice; at 32K tokens and four KV heads that is 64 blocks.  Here the
+// sequence axis is split across the grid:
+//   1. value_range_kernel     partial min/max per (1024-token chunk, channel)
+//   2. value_params_kernel    scale, midpoint and reciprocal per channel
+//   3. value_codes_kernel     codes + packed transposed store + tile sums
+//   4. value_residual_kernel  (affine) per-summation-thread residual sums in the
+//                             reference's order: thread t adds tokens L-1-t-k*T
+//   5. value_center_kernel    (affine) xor-tree per 32 threads, warps in order
+// min/max are order independent, so 1-3 are exact for any split; 4-5 keep the
+// floating-point summation order explicitly.
+
+#include "common.hpp"
+#include "launchers.hpp"
+
+#include <cfloat>
+
+namespace risa {
+namespace {
+
+constexpr int kChunk = 1024;  // tokens per block of the range pass
+
+__host__ __device__ inline int summation_threads(int length) { return length <= 256 ? 128 : 512; }
+
+// Tokens held by the four consecutive packed positions starting at p0 (multiple of 4).
+__device__ __forceinline__ int first_token_of_positions(int p0) {
+  const int pos = p0 & 31;
+  const int h = pos >> 4;
+  const int b = (pos & 15) >> 2;
+  return (p0 & ~31) + 8 * b + 4 * h;
+}
+
+template <int DT, bool AFFINE>
+__global__ __launch_bounds__(256) void value_range_kernel(const void* __restrict__ v,
+                                                          float* __restrict__ part_max,
+                                                          float* __restrict__ part_min, int length,
+                                                          int dim, int heads, int chunks,
+                                                          int64_t stride_b, int64_t stride_h,
+                                                          int64_t stride_n) {
+  const int chunk = blockIdx.x, bh = blockIdx.y;
+  const int b = bh / heads, h = bh - b * heads;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int64_t base = static_cast<int64_t>(b) * stride_b + static_cast<int64_t>(h) * stride_h;
+  const int octets = dim / 8;
+  for (int octet = wave; octet < octets; octet += 4) {
+    float mx[8], mn[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      mx[i] = AFFINE ? -FLT_MAX : 0.0f;
+      mn[i] = FLT_MAX;
+    }
+    for (int pass = 0; pass < kChunk / 256; ++pass) {
+      const int n0 = chunk * kChunk + pass * 256 + lane * 4;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int n = n0 + r;
+        if (n < length) {
+          float x[8];
+          load8<DT>(v, base + static_cast<int64_t>(n) * stride_n + octet * 8, x);
+#pragma unroll
+          for (int i = 0; i < 8; ++i) {
+            if constexpr (AFFINE) {
+              mx[i] = __builtin_fmaxf(mx[i], x[i]);
+              mn[i] = __builtin_fminf(mn[i], x[i]);
+            } else {
+              mx[i] = __builtin_fmaxf(mx[i], __builtin_fabsf(x[i]));
+            }
+          }
+        }
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+#pragma unroll
+      for (int offset = 32; offset > 0; offset >>= 1) {
+        mx[i] = __builtin_fmaxf(mx[i], __shfl_xor(mx[i], offset));
+        if constexpr (AFFINE) mn[i] = __builtin_fminf(mn[i], __shfl_xor(mn[i], offset));
+      }
+    }
+    if (lane == 0) {
+      const int64_t slot = (static_cast<int64_t>(bh) * chunks + chunk) * dim + octet * 8;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        part_max[slot + i] = mx[i];
+        if constexpr (AFFINE) part_min[slot + i] = mn[i];
+      }
+    }
+  }
+}
+
+template <bool AFFINE>
+__global__ void value_params_kernel(const float* __restrict__ part_max,
+                                    const float* __restrict__ part_min, float* __restrict__ scale,
+                                    float* __restrict__ center, float* __restrict__ inverse,
+                                    float* __restrict__ midpoint, int dim, int chunks, int rows) {
+  const int row = blockIdx.x * blockDim.x + threadIdx.x;  // (b*H + h)*D + c
+  if (row >= rows) return;
+  const int bh = row / dim, c = row - bh * dim;
+  float mx = AFFINE ? -FLT_MAX : 0.0f, mn = FLT_MAX;
+  for (int chunk = 0; chunk < chunks; ++chunk) {
+    const int64_t slot = (static_cast<int64_t>(bh) * chunks + chunk) * dim + c;
+    mx = __builtin_fmaxf(mx, part_max[slot]);
+    if constexpr (AFFINE) mn = __builtin_fminf(mn, part_min[slot]);
+  }
+  const float mid = AFFINE ? 0.5f * (mn + mx) : 0.0f;
+  const float radius = AFFINE ? 0.5f * (mx - mn) : mx;
+  const float sc = __builtin_fmaxf(radius * (1.0f / 127.0f), 1e-12f);
+  scale[row] = sc;
+  inverse[row] = 1.0f / sc;
+  midpoint[row] = mid;
+  if constexpr (!AFFINE) center[row] = 0.0f;
+}
+
+// grid (ceil(padded/256), B*H), 256 threads.  Lane l of every wave owns the four
+// packed positions 256*blockIdx.x + 4*l .. +3 (four consecutive tokens) and the
+// wave iterates over groups of eight channels.
+template <int DT, int CTA_K>
+__global__ __launch_bounds__(256) void value_codes_kernel(const void* __restrict__ v,
+                                                          int8_t* __restrict__ codes,
+                                                          int32_t* __restrict__ tile_sum,
+                                                          const float* __restrict__ inverse,
+                                                          const float* __restrict__ midpoint,
+                                                          int length, int padded, int dim, int heads,
+                                                          int64_t stride_b, int64_t stride_h,
+                                                          int64_t stride_n) {
+  const int bh = blockIdx.y;
+  const int b = bh / heads, h = bh - b * heads;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int p0 = blockIdx.x * 256 + lane * 4;
+  const int n0 = first_token_of_positions(p0);
+  const int64_t base = static_cast<int64_t>(b) * stride_b + static_cast<int64_t>(h) * stride_h;
+  const int octets = dim / 8;
+  const int tiles = padded / CTA_K;
+  for (int octet = wave; octet < octets; octet += 4) {
+    const int64_t row0 = static_cast<int64_t>(bh) * dim + octet * 8;
+    float inv[8], mid[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      inv[i] = inverse[row0 + i];
+      mid[i] = midpoint[row0 + i];
+    }
+    int q[8][4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int n = n0 + r;
+      if (n < length) {
+        float x[8];
+        load8<DT>(v, base + static_cast<int64_t>(n) * stride_n + octet * 8, x);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) q[i][r] = quantize_s8((x[i] - mid[i]) * inv[i]);
+      } else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) q[i][r] = 0;
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      if (p0 < padded) {
+        *reinterpret_cast<uint32_t*>(codes + (row0 + i) * padded + p0) =
+            pack_s8x4(q[i][0], q[i][1], q[i][2], q[i][3]);
+      }
+      int sum = q[i][0] + q[i][1] + q[i][2] + q[i][3];
+#pragma unroll
+      for (int offset = CTA_K / 8; offset > 0; offset >>= 1) sum += __shfl_xor(sum, offset);
+      if ((lane & (CTA_K / 4 - 1)) == 0 && p0 < padded) {
+        tile_sum[(static_cast<int64_t>(bh) * tiles + p0 / CTA_K) * dim + octet * 8 + i] = sum;
+      }
+    }
+  }
+}
+
+// grid (T / (256/octets), B*H), 256 threads: thread = (summation thread t, octet).
+template <int DT>
+__global__ __launch_bounds__(256) void value_residual_kernel(const void* __restrict__ v,
+                                                             float* __restrict__ partial,
+                                                             const float* __restrict__ inverse,
+                                                             const float* __restrict__ midpoint,
+                                                             int length, int dim, int heads,
+                                                             int threads, int64_t stride_b,
+                                                             int64_t stride_h, int64_t stride_n) {
+  const int bh = blockIdx.y;
+  const int b = bh / heads, h = bh - b * heads;
+  const int octets = dim / 8;
+  const int octet = threadIdx.x % octets;
+  const int t = blockIdx.x * (256 / octets) + threadIdx.x / octets;
+  const int64_t base = static_cast<int64_t>(b) * stride_b + static_cast<int64_t>(h) * stride_h;
+  const int64_t row0 = static_cast<int64_t>(bh) * dim + octet * 8;
+  float inv[8], mid[8], residual[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    inv[i] = inverse[row0 + i];
+    mid[i] = midpoint[row0 + i];
+    residual[i] = 0.0f;
+  }
+  for (int src = length - 1 - t; src >= 0; src -= threads) {
+    float x[8];
+    load8<DT>(v, base + static_cast<int64_t>(src) * stride_n + octet * 8, x);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const float normalized = (x[i] - mid[i]) * inv[i];
+      const float code = static_cast<float>(quantize_s8(normalized));
+      residual[i] += normalized - code;
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < 8; ++i) partial[(row0 + i) * threads + t] = residual[i];
+}
+
+__global__ void value_center_kernel(const float* __restrict__ partial,
+                                    const float* __restrict__ inverse,
+                                    const float* __restrict__ midpoint, float* __restrict__ center,
+                                    int rows, int threads, int length) {
+  const int row = blockIdx.x * blockDim.x + threadIdx.x;
+  if (row >= rows) return;
+  const float* p = partial + static_cast<int64_t>(row) * threads;
+  float total = 0.0f;
+  for (int w = 0; w < threads / 32; ++w) {
+    float t[32];
+#pragma unroll
+    for (int i = 0; i < 32; ++i) t[i] = p[w * 32 + i];
+#pragma unroll
+    for (int offset = 16; offset > 0; offset >>= 1) {
+#pragma unroll
+      for (int i = 0; i < offset; ++i) t[i] = t[i] + t[i + offset];
+    }
+    total += t[0];
+  }
+  const float scale = 1.0f / inverse[row];
+  const float mean = total / static_cast<float>(length);
+  const float correction = scale * mean;
+  center[row] = midpoint[row] + correction;
+}
+
+// grid (ceil(padded/256), rows_bh), 256 threads: tile sums of already packed codes.
+template <int CTA_K>
+__global__ __launch_bounds__(256) void value_tile_sum_kernel(const int8_t* __restrict__ codes,
+                                                             int32_t* __restrict__ tile_sum, int dim,
+                                                             int padded) {
+  const int bh = blockIdx.y;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int p0 = blockIdx.x * 256 + lane * 4;
+  const int tiles = padded / CTA_K;
+  for (int c = wave; c < dim; c += 4) {
+    int sum = 0;
+    if (p0 < padded) {
+      const uint32_t word =
+          *reinterpret_cast<const uint32_t*>(codes + (static_cast<int64_t>(bh) * dim + c) * padded + p0);
+      sum = static_cast<int8_t>(word & 0xff) + static_cast<int8_t>((word >> 8) & 0xff) +
+            static_cast<int8_t>((word >> 16) & 0xff) + static_cast<int8_t>(word >> 24);
+    }
+#pragma unroll
+    for (int offset = CTA_K / 8; offset > 0; offset >>= 1) sum += __shfl_xor(sum, offset);
+    if ((lane & (CTA_K / 4 - 1)) == 0 && p0 < padded) {
+      tile_sum[(static_cast<int64_t>(bh) * tiles + p0 / CTA_K) * dim + c] = sum;
+    }
+  }
+}
+
+struct Workspace {
+  float* part_max;
+  float* part_min;
+  float* inverse;
+  float* midpoint;
+  float* partial;
+  size_t bytes;
+};
+
+Workspace carve(void* base, int batch, int heads, int length, int dim, bool affine) {
+  const size_t bh = static_cast<size_t>(batch) * heads;
+  const size_t chunks = (length + kChunk - 1) / kChunk;
+  const size_t rows = bh * dim;
+  float* p = static_cast<float*>(base);
+  Workspace w{};
+  size_t offset = 0;
+  w.part_max = p + offset;
+  offset += bh * chunks * dim;
+  w.part_min = p + offset;
+  offset += affine ? bh * chunks * dim : 0;
+  w.inverse = p + offset;
+  offset += rows;
+  w.midpoint = p + offset;
+  offset += rows;
+  w.partial = p + offset;
+  offset += affine ? rows * summation_threads(length) : 0;
+  w.bytes = offset * sizeof(float);
+  return w;
+}
+
+template <int DT> int run(const ValueArgs& a, hipStream_t stream) {
+  const Workspace w = carve(a.workspace, a.batch, a.heads, a.length, a.head_dim, a.midpoint_affine);
+  const int bh = a.batch * a.heads;
+  const int chunks = (a.length + kChunk - 1) / kChunk;
+  const int rows = bh * a.head_dim;
+  dim3 range_grid(chunks, bh);
+  if (a.midpoint_affine) {
+    value_range_kernel<DT, true><<<range_grid, 256, 0, stream>>>(
+        a.v, w.part_max, w.part_min, a.length, a.head_dim, a.heads, chunks, a.stride_b, a.stride_h,
+        a.stride_n);
+    value_params_kernel<true><<<(rows + 255) / 256, 256, 0, stream>>>(
+        w.part_max, w.part_min, a.scale, a.center, w.inverse, w.midpoint, a.head_dim, chunks, rows);
+  } else {
+    value_range_kernel<DT, false><<<range_grid, 256, 0, stream>>>(
+        a.v, w.part_max, w.part_min, a.length, a.head_dim, a.heads, chunks, a.stride_b, a.stride_h,
+        a.stride_n);
+    value_params_kernel<false><<<(rows + 255) / 256, 256, 0, stream>>>(
+        w.part_max, w.part_min, a.scale, a.center, w.inverse, w.midpoint, a.head_dim, chunks, rows);
+  }
+  dim3 code_grid((a.padded + 255) / 256, bh);
+  if (a.cta_k == 128) {
+    value_codes_kernel<DT, 128><<<code_grid, 256, 0, stream>>>(
+        a.v, a.codes, a.tile_sum, w.inverse, w.midpoint, a.length, a.padded, a.head_dim, a.heads,
+        a.stride_b, a.stride_h, a.stride_n);
+  } else {
+    value_codes_kernel<DT, 64><<<code_grid, 256, 0, stream>>>(
+        a.v, a.codes, a.tile_sum, w.inverse, w.midpoint, a.length, a.padded, a.head_dim, a.heads,
+        a.stride_b, a.stride_h, a.stride_n);
+  }
+  if (a.midpoint_affine) {
+    const int threads = summation_threads(a.length);
+    const int per_block = 256 / (a.head_dim / 8);
+    dim3 residual_grid(threads / per_block, bh);
+    value_residual_kernel<DT><<<residual_grid, 256, 0, stream>>>(
+        a.v, w.partial, w.inverse, w.midpoint, a.length, a.head_dim, a.heads, threads, a.stride_b,
+        a.stride_h, a.stride_n);
+    value_center_kernel<<<(rows + 63) / 64, 64, 0, stream>>>(w.partial, w.inverse, w.midpoint,
+                                                             a.center, rows, threads, a.length);
+  }
+  return check_launch("risa_quantize_v");
+}
+
+}  // namespace
+
+size_t value_workspace_bytes(int batch, int heads, int length, int head_dim, bool midpoint_affine) {
+  return carve(nullptr, batch, heads, length, head_dim, midpoint_affine).bytes;
+}
+
+int launch_quantize_v(const ValueArgs& a, hipStream_t stream) {
+  if (a.workspace_bytes <
+      value_workspace_bytes(a.batch, a.heads, a.length, a.head_dim, a.midpoint_affine)) {
+    return fail("risa_quantize_v: workspace is too small");
+  }
+  if (a.dtype == kF32) return run<kF32>(a, stream);
+  if (a.dtype == kF16) return run<kF16>(a, stream);
+  return run<kBF16>(a, stream);
+}
+
+int launch_value_tile_sums(const int8_t* codes, int32_t* tile_sum, int rows_bh, int head_dim,
+                           int padded, int cta_k, hipStream_t stream) {
+  dim3 grid((padded + 255) / 256, rows_bh);
+  if (cta_k == 128)
+    value_tile_sum_kernel<128><<<grid, 256, 0, stream>>>(codes, tile_sum, head_dim, padded);
+  else
+    value_tile_sum_kernel<64><<<grid, 256, 0, stream>>>(codes, tile_sum, head_dim, padded);
+  return check_launch("risa_value_tile_sums");
+}
+
+}  // namespace risa

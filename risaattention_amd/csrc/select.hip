@@ -1,0 +1,217 @@
+// Retained-mass tile selection and broadcast key-mask tile metadata for gfx950.
+//
+// Contract: reference csrc/kernels/sparse_selection.cu:9-159 (FP64 total and
+// prefix over masses already sorted in descending order, shortest prefix whose
+// mass reaches theta * total, CSR compaction in ascending tile order, summary)
+// and csrc/kernels/key_mask_tiles.cu:10-43.
+
+#include "common.hpp"
+#include "launchers.hpp"
+
+namespace risa {
+namespace {
+
+// One 32-lane half of a wavefront per row, so that lane-strided sums and the
+// 32-wide inclusive scans associate exactly as in the contract.
+__global__ __launch_bounds__(64) void select_rows_kernel(const float* __restrict__ sorted_mass,
+                                                         const int64_t* __restrict__ order,
+                                                         int32_t* __restrict__ counts,
+                                                         uint8_t* __restrict__ support,
+                                                         double* __restrict__ row_totals, int rows,
+                                                         int tiles, double theta) {
+  const int sub = threadIdx.x & 31;
+  const int row = blockIdx.x * 2 + (threadIdx.x >> 5);
+  if (row >= rows) return;
+  const int64_t base = static_cast<int64_t>(row) * tiles;
+  double lane_total = 0.0;
+  for (int rank = sub; rank < tiles; rank += 32) {
+    lane_total += static_cast<double>(sorted_mass[base + rank]);
+    support[base + rank] = 0;
+  }
+  double total = lane_total;
+#pragma unroll
+  for (int offset = 16; offset > 0; offset >>= 1) total += __shfl_down(total, offset, 32);
+  total = __shfl(total, 0, 32);
+
+  const double target = theta * total;
+  double cumulative = 0.0;
+  double selected = total;
+  int count = tiles;
+  for (int chunk = 0; chunk < tiles; chunk += 32) {
+    const int rank = chunk + sub;
+    double prefix = rank < tiles ? static_cast<double>(sorted_mass[base + rank]) : 0.0;
+#pragma unroll
+    for (int offset = 1; offset < 32; offset <<= 1) {
+      const double previous = __shfl_up(prefix, offset, 32);
+      if (sub >= offset) prefix += previous;
+    }
+    const bool reaches = rank < tiles && cumulative + prefix >= target;
+    const uint64_t ballot = __ballot(reaches);
+    const uint32_t votes = static_cast<uint32_t>(ballot >> (threadIdx.x & 32));
+    if (votes != 0) {
+      const int first = __builtin_ctz(votes);
+      count = chunk + first + 1;
+      selected = cumulative + __shfl(prefix, first, 32);
+      break;
+    }
+    cumulative += __shfl(prefix, 31, 32);
+  }
+  // The support bytes of this row were cleared by these same 32 lanes above.
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  for (int rank = sub; rank < count; rank += 32) {
+    support[base + static_cast<int>(order[base + rank])] = 1;
+  }
+  if (sub == 0) {
+    counts[row] = count;
+    row_totals[row * 2] = selected;
+    row_totals[row * 2 + 1] = total;
+  }
+}
+
+// Single workgroup: exclusive scan of the per-row counts and the FP64 summary
+// (pairwise tree over 256 partial sums, as in the contract).
+__global__ __launch_bounds__(256) void offsets_summary_kernel(const int32_t* __restrict__ counts,
+                                                              const double* __restrict__ row_totals,
+                                                              int32_t* __restrict__ row_offsets,
+                                                              double* __restrict__ summary, int rows) {
+  __shared__ double selected_sums[256];
+  __shared__ double total_sums[256];
+  __shared__ int scan[256];
+  __shared__ int carry;
+  const int tid = threadIdx.x;
+  double selected = 0.0, total = 0.0;
+  for (int row = tid; row < rows; row += 256) {
+    selected += row_totals[row * 2];
+    total += row_totals[row * 2 + 1];
+  }
+  selected_sums[tid] = selected;
+  total_sums[tid] = total;
+  if (tid == 0) carry = 0;
+  __syncthreads();
+  for (int stride = 128; stride > 0; stride >>= 1) {
+    if (tid < stride) {
+      selected_sums[tid] += selected_sums[tid + stride];
+      total_sums[tid] += total_sums[tid + stride];
+    }
+    __syncthreads();
+  }
+  for (int base = 0; base < rows; base += 256) {
+    const int row = base + tid;
+    const int value = row < rows ? counts[row] : 0;
+    scan[tid] = value;
+    __syncthreads();
+    for (int offset = 1; offset < 256; offset <<= 1) {
+      const int add = tid >= offset ? scan[tid - offset] : 0;
+      __syncthreads();
+      scan[tid] += add;
+      __syncthreads();
+    }
+    if (row < rows) row_offsets[row] = carry + scan[tid] - value;
+    __syncthreads();
+    if (tid == 255) carry += scan[255];
+    __syncthreads();
+  }
+  if (tid == 0) {
+    row_offsets[rows] = carry;
+    summary[0] = selected_sums[0];
+    summary[1] = total_sums[0];
+    summary[2] = static_cast<double>(carry);
+  }
+}
+
+// One wavefront per row: ordered compaction of the support bytes.
+__global__ __launch_bounds__(256) void compact_rows_kernel(const uint8_t* __restrict__ support,
+                                                           const int32_t* __restrict__ row_offsets,
+                                                           int32_t* __restrict__ block_indices,
+                                                           int rows, int tiles) {
+  const int lane = threadIdx.x & 63;
+  const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const int64_t base = static_cast<int64_t>(row) * tiles;
+  int written = row_offsets[row];
+  for (int chunk = 0; chunk < tiles; chunk += 64) {
+    const int tile = chunk + lane;
+    const bool keep = tile < tiles && support[base + tile] != 0;
+    const uint64_t votes = __ballot(keep);
+    if (keep) {
+      const uint64_t lower = lane == 0 ? 0ull : (votes & ((1ull << lane) - 1ull));
+      block_indices[written + __builtin_popcountll(lower)] = tile;
+    }
+    written += __builtin_popcountll(votes);
+  }
+}
+
+__device__ __forceinline__ bool key_visible(const void* mask, int64_t index, int dtype) {
+  if (dtype == kBool) return static_cast<const uint8_t*>(mask)[index] != 0;
+  const float bias = dtype == kF32   ? load1<kF32>(mask, index)
+                     : dtype == kF16 ? load1<kF16>(mask, index)
+                                     : load1<kBF16>(mask, index);
+  return __builtin_isfinite(bias);
+}
+
+// One workgroup per (batch, head): flag tiles with any visible key, then one
+// wavefront compacts the active tile ids in ascending order and appends the count.
+__global__ __launch_bounds__(256) void key_mask_tiles_kernel(const void* __restrict__ mask,
+                                                             int32_t* __restrict__ output, int heads,
+                                                             int length, int tile_size,
+                                                             int64_t stride_b, int64_t stride_h,
+                                                             int64_t stride_k, int dtype) {
+  const int tiles = (length + tile_size - 1) / tile_size;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int64_t row = static_cast<int64_t>(blockIdx.x) * heads + blockIdx.y;
+  const int64_t mask_row = blockIdx.x * stride_b + blockIdx.y * stride_h;
+  int32_t* out = output + row * (tiles + 1);
+  extern __shared__ int active_flags[];
+  for (int tile = wave; tile < tiles; tile += 4) {
+    bool visible = false;
+    for (int offset = lane; offset < tile_size; offset += 64) {
+      const int key = tile * tile_size + offset;
+      if (key < length) visible |= key_visible(mask, mask_row + key * stride_k, dtype);
+    }
+    const bool any = __ballot(visible) != 0;
+    if (lane == 0) active_flags[tile] = any ? 1 : 0;
+  }
+  __syncthreads();
+  if (wave == 0) {
+    int count = 0;
+    for (int base = 0; base < tiles; base += 64) {
+      const int tile = base + lane;
+      const bool active = tile < tiles && active_flags[tile] != 0;
+      const uint64_t votes = __ballot(active);
+      if (active) {
+        const uint64_t lower = lane == 0 ? 0ull : (votes & ((1ull << lane) - 1ull));
+        out[count + __builtin_popcountll(lower)] = tile;
+      }
+      count += __builtin_popcountll(votes);
+    }
+    // Slots behind the active ids are never read by the attention kernel.
+    for (int slot = count + lane; slot < tiles; slot += 64) out[slot] = -1;
+    if (lane == 0) out[tiles] = count;
+  }
+}
+
+}  // namespace
+
+int launch_select_retained_mass(const SelectArgs& a, hipStream_t stream) {
+  select_rows_kernel<<<(a.rows + 1) / 2, 64, 0, stream>>>(a.sorted_mass, a.descending_indices,
+                                                          a.counts, a.support, a.row_totals, a.rows,
+                                                          a.tiles, a.theta);
+  offsets_summary_kernel<<<1, 256, 0, stream>>>(a.counts, a.row_totals, a.row_offsets, a.summary,
+                                                a.rows);
+  compact_rows_kernel<<<(a.rows + 3) / 4, 256, 0, stream>>>(a.support, a.row_offsets,
+                                                            a.block_indices, a.rows, a.tiles);
+  return check_launch("risa_select_retained_mass");
+}
+
+int launch_key_mask_tiles(const void* mask, int32_t* tiles, int batch, int heads, int length,
+                          int tile_size, int64_t stride_b, int64_t stride_h, int64_t stride_k,
+                          int dtype, hipStream_t stream) {
+  const int count = (length + tile_size - 1) / tile_size;
+  const dim3 grid(batch, heads);
+  key_mask_tiles_kernel<<<grid, 256, count * sizeof(int), stream>>>(
+      mask, tiles, heads, length, tile_size, stride_b, stride_h, stride_k, dtype);
+  return check_launch("risa_prepare_key_mask_tiles");
+}
+
+}  // namespace risa

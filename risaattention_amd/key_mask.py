@@ -1,0 +1,38 @@
+"""Tile lists that let broadcast key masks skip fully hidden key tiles.
+
+Counterpart of reference src/risa_attention/_key_mask.py:9-28.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from . import native
+from .policy import MASK_DTYPE_CODES
+
+
+def prepare_key_mask_tiles(mask, key_block_size, query_length, scale, is_causal):
+    """int32 [B,Hq,tiles+1] (active tile ids, then the count) or None.
+
+    Built only for masks without a query extent (stride 0), more than 1024
+    keys, at least 256 queries, a positive scale and no causal flag.
+    """
+    if (
+        mask is None
+        or mask.stride(-2) != 0
+        or mask.shape[-1] <= 1024
+        or query_length < 256
+        or scale <= 0
+        or is_causal
+    ):
+        return None
+    batch, heads, _, length = mask.shape
+    tiles = torch.empty((batch, heads, -(-length // key_block_size) + 1), device=mask.device, dtype=torch.int32)
+    native.check(
+        native.library().risa_prepare_key_mask_tiles(
+            mask.data_ptr(), tiles.data_ptr(), batch, heads, length, key_block_size,
+            mask.stride(0), mask.stride(1), mask.stride(3), MASK_DTYPE_CODES[mask.dtype],
+            native.current_stream(mask.device),
+        )
+    )
+    return tiles

@@ -1,0 +1,51 @@
+"""Shared helpers for the parity tests (oracle on CPU vs HIP kernels on the GPU)."""
+
+from __future__ import annotations
+
+import numpy as np
+import torch
+
+from oracle import pipeline as oracle_pipeline
+
+DTYPE_NAMES = {torch.float32: "float32", torch.float16: "float16", torch.bfloat16: "bfloat16"}
+
+
+def to_numpy(tensor: torch.Tensor) -> np.ndarray:
+    if tensor.dtype == torch.bool:
+        return tensor.detach().cpu().numpy()
+    return tensor.detach().float().cpu().numpy()
+
+
+def mask_to_numpy(mask: torch.Tensor | None):
+    """Keep a key-only mask's query extent at 1 so the oracle sees it as key-only."""
+    if mask is None:
+        return None
+    while mask.ndim < 4:
+        mask = mask[None]
+    if mask.dtype == torch.bool:
+        return mask.detach().cpu().numpy()
+    return mask.detach().float().cpu().numpy()
+
+
+def oracle_prequantize(q, k, v, *, attn_mask=None, **kwargs):
+    return oracle_pipeline.prequantize(
+        to_numpy(q), to_numpy(k), to_numpy(v), mask=mask_to_numpy(attn_mask),
+        dtype_name=DTYPE_NAMES[q.dtype], **kwargs,
+    )
+
+
+def relative_l2(actual, expected) -> float:
+    actual = np.asarray(actual, dtype=np.float64)
+    expected = np.asarray(expected, dtype=np.float64)
+    finite = np.isfinite(expected)
+    assert np.array_equal(np.isfinite(actual), finite), "finite patterns differ"
+    if not finite.any():
+        return 0.0
+    denominator = np.sqrt((expected[finite] ** 2).sum())
+    return float(np.sqrt(((actual[finite] - expected[finite]) ** 2).sum()) / max(denominator, 1e-30))
+
+
+def seeded(shape, dtype, seed, device="cuda", offset=0.0, scale=1.0):
+    generator = torch.Generator(device="cpu").manual_seed(seed)
+    values = torch.randn(shape, generator=generator, dtype=torch.float32) * scale + offset
+    return values.to(dtype).to(device)

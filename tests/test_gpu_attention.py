@@ -1,0 +1,199 @@
+"""Parity of the HIP attention kernel with the oracle: outputs and LSE within 1e-3
+relative L2 (the tolerance the task states for floating-point results), plus the
+closed-form contracts of the reference's own CUDA tests."""
+
+from dataclasses import replace
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import pipeline as oracle_pipeline
+from tests.helpers import oracle_prequantize, relative_l2, seeded, to_numpy
+
+pytestmark = pytest.mark.gpu
+
+TOLERANCE = 1e-3
+
+
+def mask_variants(q_len, k_len, device="cuda"):
+    key_bias = torch.linspace(-2, 0, k_len, device=device)[None, None, None, :]
+    row_mask = torch.ones(q_len, k_len, device=device, dtype=torch.bool)
+    row_mask[0] = False
+    row_mask[1:, 7::9] = False
+    return {"none": None, "key_bias": key_bias, "row_mask": row_mask}
+
+
+@pytest.mark.parametrize("mode", ["absmax", "midpoint_affine"])
+@pytest.mark.parametrize("dim", [64, 128, 256])
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("mask_name", ["none", "key_bias", "row_mask"])
+def test_dense_matches_oracle(risa, mode, dim, causal, mask_name):
+    q = seeded((1, 2, 137, dim), torch.float16, 17)
+    k = seeded((1, 1, 263, dim), torch.float16, 18)
+    v = seeded((1, 1, 263, dim), torch.float16, 19, offset=2.0)
+    mask = mask_variants(137, 263)[mask_name]
+    out, lse = risa.int8_attention(q, k, v, attn_mask=mask, is_causal=causal, v_quantization=mode,
+                                   return_lse=True)
+    prepared = oracle_prequantize(q, k, v, attn_mask=mask, is_causal=causal, v_quantization=mode,
+                                  return_lse=True)
+    expected, expected_lse, _ = oracle_pipeline.attend(prepared, return_lse=True)
+    assert relative_l2(to_numpy(out), expected) < TOLERANCE
+    assert relative_l2(to_numpy(lse), expected_lse) < TOLERANCE
+    # FP32 SDPA bound of reference tests/cuda/test_risa_attention.py:118-132
+    from risaattention_amd.policy import apply_score_mask
+
+    scores = q.float() @ k.float().repeat_interleave(2, 1).transpose(-1, -2) / dim**0.5
+    expanded = None if mask is None else torch.broadcast_to(mask, scores.shape)
+    scores = apply_score_mask(scores, expanded, causal, 0)
+    reference = scores.softmax(-1).nan_to_num(nan=0) @ v.float().repeat_interleave(2, 1)
+    torch.testing.assert_close(out.float(), reference, atol=0.10, rtol=0.03)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("k_len", [1153, 2304])
+def test_large_tile_dense_and_scale_signs(risa, dtype, k_len):
+    q = seeded((1, 4, 300, 128), dtype, 5)
+    k = seeded((1, 2, k_len, 128), dtype, 6)
+    v = seeded((1, 2, k_len, 128), dtype, 7)
+    for scale in (None, 0.0, -0.125):
+        out, lse = risa.int8_attention(q, k, v, scale=scale, return_lse=True)
+        prepared = oracle_prequantize(q, k, v, scale=scale, return_lse=True)
+        assert prepared.cta_k == 128
+        expected, expected_lse, _ = oracle_pipeline.attend(prepared, return_lse=True)
+        assert relative_l2(to_numpy(out), expected) < TOLERANCE
+        assert relative_l2(to_numpy(lse), expected_lse) < TOLERANCE
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("dim", [64, 128, 256])
+@pytest.mark.parametrize("k_len", [512, 1025])
+@pytest.mark.parametrize("scale", [None, 0.0, -0.125])
+@pytest.mark.parametrize("mode", ["absmax", "midpoint_affine"])
+def test_constant_values_preserve_probability_mass(risa, dtype, dim, k_len, scale, mode):
+    """reference tests/cuda/test_probability_mass.py:21-34."""
+    torch.manual_seed(41)
+    q = torch.randn(1, 4, 129, dim, device="cuda", dtype=dtype)
+    k = torch.randn(1, 2, k_len, dim, device="cuda", dtype=dtype)
+    values = torch.linspace(-3, 5, dim, device="cuda", dtype=dtype)
+    v = values.expand_as(k).contiguous()
+    out = risa.int8_attention(q, k, v, scale=scale, v_quantization=mode)
+    torch.testing.assert_close(out, values.expand_as(out), atol=0, rtol=0)
+
+
+@pytest.mark.parametrize("k_len", [512, 1025])
+@pytest.mark.parametrize("scale", [0.0, -0.125])
+@pytest.mark.parametrize("mode", ["absmax", "midpoint_affine"])
+def test_signed_scale_tail_masks_and_lse(risa, k_len, scale, mode):
+    """reference tests/cuda/test_probability_mass.py:37-70."""
+    torch.manual_seed(43)
+    q = torch.randn(1, 4, 129, 128, device="cuda", dtype=torch.bfloat16)
+    k = torch.randn(1, 2, k_len, 128, device="cuda", dtype=q.dtype)
+    v = torch.full_like(k, 3)
+    mask = torch.ones(129, k_len, device="cuda", dtype=torch.bool)
+    mask[0] = False
+    mask[1:, 7::9] = False
+    out, lse = risa.int8_attention(q, k, v, scale=scale, attn_mask=mask, is_causal=True,
+                                   v_quantization=mode, return_lse=True)
+    torch.testing.assert_close(out[:, :, 1:], torch.full_like(out[:, :, 1:], 3), atol=0, rtol=0)
+    assert torch.count_nonzero(out[:, :, 0]) == 0
+    assert torch.isneginf(lse[:, :, 0]).all()
+    assert torch.isfinite(lse[:, :, 1:]).all()
+    if scale == 0:
+        visible = mask & (torch.arange(k_len, device="cuda")[None, :] <= torch.arange(129, device="cuda")[:, None])
+        expected = visible.sum(-1).float().log().expand_as(lse)
+        torch.testing.assert_close(lse, expected, atol=2e-5, rtol=0)
+
+
+def test_residual_center_preserves_uniform_attention_mean(risa):
+    """reference tests/cuda/test_probability_mass.py:148-155."""
+    torch.manual_seed(3)
+    q = torch.zeros(1, 2, 129, 128, device="cuda", dtype=torch.bfloat16)
+    k = torch.zeros(1, 1, 512, 128, device="cuda", dtype=q.dtype)
+    v = torch.randn_like(k) + 3
+    v[..., ::53, :] += 12
+    out = risa.int8_attention(q, k, v, v_quantization="midpoint_affine")
+    expected = v.float().mean(-2, keepdim=True).to(v.dtype).expand_as(out)
+    torch.testing.assert_close(out, expected, atol=0, rtol=0)
+
+
+@pytest.mark.parametrize("mode", ["midpoint_affine", "absmax"])
+@pytest.mark.parametrize("dim", [64, 128, 256])
+@pytest.mark.parametrize("length", [63, 65, 193, 1153])
+def test_capture_tile_max_known_answer(risa, mode, dim, length):
+    """reference tests/cuda/test_risa_attention.py:20-92: packed Q=1, K=+3/-2 per tile."""
+    q = torch.zeros(1, 2, 137, dim, device="cuda", dtype=torch.float16)
+    k = torch.zeros(1, 1, length, dim, device="cuda", dtype=torch.float16)
+    torch.manual_seed(length)
+    packed = risa.prequantize_int8_attention(q, k, torch.randn_like(k) + 2, scale=1 / 128, v_quantization=mode)
+    packed.q.fill_(1)
+    packed.q_scale.fill_(1)
+    packed.k_scale.fill_(1)
+    blocks = (length + packed.cta_k - 1) // packed.cta_k
+    levels = torch.tensor([3 if i % 2 == 0 else -2 for i in range(blocks)], dtype=torch.int8, device="cuda")
+    for i in range(blocks):
+        packed.k[:, :, i * packed.cta_k : (i + 1) * packed.cta_k].fill_(3 if i % 2 == 0 else -2)
+    batch, heads, queries, _ = packed.q.shape
+    mass_elements = batch * heads * ((queries + 127) // 128) * blocks
+    rows = batch * heads * queries
+    workspace = torch.empty(mass_elements + rows * (blocks * 2 + 2), device="cuda", dtype=torch.float32)
+    plain = risa.int8_attention_from_prequantized(packed)
+    captured = risa.int8_attention_from_prequantized(packed, _block_mass=workspace)
+    assert torch.equal(plain.view(torch.int16), captured.view(torch.int16))
+    if blocks > 1:
+        full_stats = workspace[mass_elements : mass_elements + rows * (blocks - 1) * 2]
+        maxima = full_stats.reshape(rows, blocks - 1, 2)[..., 1]
+        scale = torch.tensor(1.44269504088896340736, device="cuda", dtype=torch.float32) / 128
+        offset = torch.tensor(7.9943534, device="cuda", dtype=torch.float32)
+        expected = (levels[:-1].double() * dim * scale.double() - offset.double()).float()
+        assert torch.equal(maxima, expected.expand_as(maxima))
+    masses = workspace[:mass_elements].view(-1, blocks)
+    per_block = torch.tensor([128.0, 9.0] * heads, device="cuda")
+    torch.testing.assert_close(masses.sum(-1), per_block, atol=2e-4, rtol=0)
+    hidden = torch.zeros(batch, heads, queries, length, device="cuda", dtype=torch.bool)
+    empty = risa.int8_attention_from_prequantized(replace(packed, attn_mask=hidden))
+    assert torch.count_nonzero(empty) == 0
+
+
+def test_causal_future_values_are_invisible(risa):
+    """reference tests/cuda/test_risa_attention.py:151-165."""
+    q = torch.zeros(1, 1, 193, 64, device="cuda", dtype=torch.float16)
+    v = torch.zeros_like(q)
+    v[:, :, 128:] = 100
+    for mode in ("midpoint_affine", "absmax"):
+        out, pattern = risa.construct_sparse_int8_attention(q, q, v, is_causal=True, theta=1.0, v_quantization=mode)
+        sparse = risa.sparse_int8_attention(q, q, v, pattern, is_causal=True, v_quantization=mode)
+        torch.testing.assert_close(out[:, :, :128], torch.zeros_like(out[:, :, :128]), atol=0.01, rtol=0)
+        torch.testing.assert_close(sparse, out, atol=0.05, rtol=0.01)
+
+
+def test_key_bias_large_tile_and_lse(risa):
+    """reference tests/cuda/test_risa_attention.py:167-179."""
+    q = torch.zeros(1, 2, 17, 128, device="cuda", dtype=torch.float16)
+    k = torch.zeros(1, 1, 1153, 128, device="cuda", dtype=torch.float16)
+    v = torch.ones_like(k) * 3
+    mask = torch.linspace(-3, 0, 1153, device="cuda")[None, None, None, :]
+    for mode in ("midpoint_affine", "absmax"):
+        packed = risa.prequantize_int8_attention(q, k, v, attn_mask=mask, return_lse=True, v_quantization=mode)
+        assert packed.cta_k == 128
+        out, lse = risa.int8_attention_from_prequantized(packed, return_lse=True)
+        torch.testing.assert_close(out, torch.full_like(out, 3), atol=0.03, rtol=0)
+        torch.testing.assert_close(lse, mask.logsumexp(-1).expand(1, 2, 17), atol=0.01, rtol=0)
+
+
+def test_lse_restores_shifted_keys_and_empty_rows(risa):
+    """reference tests/cuda/test_risa_attention.py:181-193."""
+    from risaattention_amd.policy import apply_score_mask
+
+    torch.manual_seed(29)
+    q = torch.randn(1, 2, 19, 128, device="cuda", dtype=torch.float16)
+    k = torch.randn(1, 1, 257, 128, device="cuda", dtype=torch.float16) * 0.1 + 4
+    v = torch.randn_like(k)
+    mask = torch.ones(19, 257, dtype=torch.bool, device="cuda")
+    mask[0] = False
+    out, lse = risa.int8_attention(q, k, v, attn_mask=mask, is_causal=True, return_lse=True)
+    scores = q.float() @ k.float().transpose(-1, -2) / 128**0.5
+    expected = apply_score_mask(scores, mask, True, 0).logsumexp(-1)
+    assert torch.isneginf(lse[:, :, 0]).all()
+    assert out[:, :, 0].count_nonzero().item() == 0
+    torch.testing.assert_close(lse[:, :, 1:], expected[:, :, 1:], atol=0.15, rtol=0.02)

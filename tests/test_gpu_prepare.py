@@ -1,0 +1,109 @@
+"""Bit-exact parity of the HIP preparation kernels with the oracle (through the C ABI)."""
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import prepare as oracle_prepare
+from tests.helpers import oracle_prequantize, seeded, to_numpy
+
+pytestmark = pytest.mark.gpu
+
+CASES = [
+    # (dtype, head_dim, Lq, Lk, Hq, Hkv, mode, key offset)
+    (torch.bfloat16, 128, 257, 1153, 4, 2, "absmax", 0.0),
+    (torch.float16, 128, 137, 263, 2, 1, "midpoint_affine", 0.0),
+    (torch.float32, 128, 64, 200, 2, 2, "midpoint_affine", 0.0),
+    (torch.bfloat16, 64, 193, 700, 2, 1, "absmax", 0.0),
+    (torch.float16, 64, 33, 129, 2, 2, "midpoint_affine", 0.0),
+    (torch.bfloat16, 256, 130, 1100, 2, 1, "midpoint_affine", 0.0),
+    (torch.float16, 256, 40, 250, 2, 2, "absmax", 0.0),
+    (torch.bfloat16, 80, 100, 300, 2, 2, "absmax", 0.0),  # padded head dim
+    (torch.float16, 128, 19, 257, 2, 1, "absmax", 4.0),  # anchor fires
+    (torch.bfloat16, 128, 300, 2049, 4, 1, "midpoint_affine", 0.0),
+]
+
+
+@pytest.mark.parametrize("dtype,dim,q_len,k_len,q_heads,kv_heads,mode,offset", CASES)
+def test_prepared_tensors_match_oracle_bit_for_bit(risa, dtype, dim, q_len, k_len, q_heads, kv_heads, mode, offset):
+    from risaattention_amd.layout import unpack_values
+
+    q = seeded((2, q_heads, q_len, dim), dtype, 1)
+    k = seeded((2, kv_heads, k_len, dim), dtype, 2, offset=offset, scale=0.1 if offset else 1.0)
+    v = seeded((2, kv_heads, k_len, dim), dtype, 3, offset=1.5)
+    packed = risa.prequantize_int8_attention(q, k, v, v_quantization=mode, return_lse=True)
+    expected = oracle_prequantize(q, k, v, v_quantization=mode, return_lse=True)
+    assert packed.cta_k == expected.cta_k
+    if offset:
+        assert (expected.anchor >= 0).all(), "test input should trigger the anchor"
+    np.testing.assert_array_equal(packed.q.cpu().numpy(), expected.q)
+    np.testing.assert_array_equal(packed.q_scale.cpu().numpy(), expected.q_scale)
+    np.testing.assert_array_equal(packed.k.cpu().numpy(), expected.k)
+    np.testing.assert_array_equal(packed.k_scale.cpu().numpy(), expected.k_scale)
+    np.testing.assert_array_equal(unpack_values(packed.v).cpu().numpy(), expected.v)
+    np.testing.assert_array_equal(packed.v_scale.cpu().numpy(), expected.v_scale)
+    np.testing.assert_array_equal(packed.v_center.cpu().numpy(), expected.v_center)
+    sums = oracle_prepare.value_tile_sums(expected.v, expected.cta_k)
+    rows = expected.v.shape[0]
+    kernel_dim = packed.q.shape[-1]
+    got = packed.v_tile_sum.cpu().numpy().transpose(0, 2, 1).reshape(rows, -1)
+    np.testing.assert_array_equal(got, sums)
+    np.testing.assert_array_equal(to_numpy(packed.lse_shift), expected.lse_shift)
+    assert kernel_dim in (64, 128, 256)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("layout", ["hnd", "nhd", "interleaved"])
+@pytest.mark.parametrize("length", [1025, 2048, 2049, 4097])
+def test_absmax_values_known_answer(risa, dtype, layout, length):
+    """Power-of-two scales make codes and scales exact (reference
+    tests/cuda/test_value_quantization.py:18-52, modulo the packed order)."""
+    from risaattention_amd.layout import unpack_values
+
+    batch, heads, channels = 2, 3, 128
+    tokens = torch.arange(length, device="cuda")[None, None, :, None]
+    head_offsets = torch.arange(batch * heads, device="cuda").reshape(batch, heads, 1, 1)
+    codes = ((tokens + head_offsets) % 255 - 127).expand(batch, heads, length, channels)
+    scales = 2.0 ** ((torch.arange(channels, device="cuda") % 4).float() - 2)
+    v = (codes * scales).to(dtype)
+    if layout == "nhd":
+        v = v.transpose(1, 2).contiguous().transpose(1, 2)
+    elif layout == "interleaved":
+        storage = torch.empty(batch, length, 3, heads, channels, device="cuda", dtype=dtype)
+        v = storage[:, :, 1].transpose(1, 2).copy_(v)
+    q = torch.zeros(batch, heads * 2, 3, channels, device="cuda", dtype=dtype)
+    k = torch.zeros_like(v)
+    packed = risa.prequantize_int8_attention(q, k, v, v_quantization="absmax")
+    padded = packed.v.shape[-1]
+    expected = torch.zeros(batch, heads, channels, padded, device="cuda", dtype=torch.int8)
+    expected[..., :length] = codes.transpose(2, 3).to(torch.int8)
+    logical = unpack_values(packed.v).reshape(batch, heads, channels, padded)
+    assert torch.equal(logical, expected)
+    assert torch.equal(packed.v_scale.reshape(batch, heads, channels), scales.expand(batch, heads, channels))
+    assert torch.count_nonzero(packed.v_center) == 0
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("dim", [64, 128, 256])
+def test_lse_shift_closed_form(risa, dtype, dim):
+    """reference tests/cuda/test_lse_correction.py:9-31 through the C ABI."""
+    from risaattention_amd import native
+
+    torch.manual_seed(35)
+    q = torch.randn(2, 17, 4, dim, device="cuda", dtype=dtype).transpose(1, 2)
+    k = torch.randn(2, 9, 2, dim, device="cuda", dtype=dtype).transpose(1, 2)
+    anchors = torch.tensor([[-1, 0], [3, 2]], device="cuda", dtype=torch.int32)
+    out = torch.empty(2, 4, 17, device="cuda")
+    code = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}[dtype]
+    native.check(
+        native.library().risa_lse_shift(
+            q.data_ptr(), k.data_ptr(), anchors.data_ptr(), out.data_ptr(), 2, 4, 2, 17, dim,
+            q.stride(0), q.stride(1), q.stride(2), k.stride(0), k.stride(1), k.stride(2),
+            dim**-0.5, code, torch.cuda.current_stream().cuda_stream,
+        )
+    )
+    selected = k.gather(2, anchors.clamp_min(0).long()[..., None, None].expand(2, 2, 1, dim))
+    selected = selected.float() * (anchors >= 0)[..., None, None]
+    reference = (q.float() * selected.repeat_interleave(2, 1)).sum(-1) * dim**-0.5
+    torch.testing.assert_close(out, reference, rtol=2e-5, atol=5e-6)
+    assert torch.count_nonzero(out[0, :2]) == 0
