@@ -1,0 +1,252 @@
+"""CPU tests of the host side: C-ABI exports, input contracts, tile policy, dataclasses,
+operator registration (in the spirit of reference tests/contracts/test_risa_attention.py:29-67)."""
+
+import ctypes
+import re
+from pathlib import Path
+from unittest.mock import patch
+
+import pytest
+import torch
+
+import risaattention_amd as risa
+from risaattention_amd import attend, dense, fp32_patterns, layout, native, policy, types
+
+ROOT = Path(__file__).resolve().parents[1]
+
+
+def test_library_exports_every_declared_symbol():
+    header = (ROOT / "include" / "risa_hip.h").read_text()
+    declared = set(re.findall(r"^(?:int|size_t|void|const char\*)\s+(risa_[a-z0-9_]+)\(", header, re.M))
+    assert declared == set(native.SIGNATURES), declared ^ set(native.SIGNATURES)
+    library = ctypes.CDLL(str(native.library_path()))
+    for name in declared:
+        assert hasattr(library, name), name
+    assert native.library().risa_abi_version() == 1
+    assert native.library().risa_last_error() == b""
+
+
+def test_host_only_entry_points():
+    assert native.unpack_order() == layout.position_to_token()
+    assert sorted(native.unpack_order()) == list(range(32))
+    lib = native.library()
+    assert lib.risa_selector_workspace_size(4096) == 0
+    small = lib.risa_quantize_v_workspace_bytes(1, 4, 32768, 128, 0)
+    large = lib.risa_quantize_v_workspace_bytes(1, 4, 32768, 128, 1)
+    assert 0 < small < large
+    # rejected calls report through risa_last_error and launch nothing
+    assert lib.risa_quantize_qk(None, None, None, None, None, None, 1, 1, 1, 1, 1, 96, 64,
+                                0, 0, 0, 0, 0, 0, 2, None, None) != 0
+    assert b"head_dim" in lib.risa_last_error()
+    with pytest.raises(RuntimeError, match="head_dim"):
+        native.check(1)
+
+
+def test_availability_gate_requires_rocm_gfx950():
+    assert not risa.int8_attention_is_available("cpu")
+
+    class Props:
+        gcnArchName = "gfx950:sramecc+:xnack-"
+
+    with patch.object(torch.version, "hip", "7.0"), patch.object(torch.cuda, "is_available", return_value=True), \
+            patch.object(torch.cuda, "get_device_properties", return_value=Props()):
+        assert native.is_available()
+        Props.gcnArchName = "gfx942:sramecc+:xnack-"
+        assert not native.is_available()
+    with patch.object(torch.version, "hip", None):
+        assert not native.is_available()
+
+
+def test_missing_library_fails_loudly(tmp_path, monkeypatch):
+    monkeypatch.setenv("RISA_HIP_LIBRARY", str(tmp_path / "absent.so"))
+    monkeypatch.setattr(native, "_LIBRARY", None)
+    monkeypatch.setattr(native, "_LOAD_ERROR", None)
+    with pytest.raises(RuntimeError, match="not available"):
+        native.library()
+    assert not native.is_available()
+    monkeypatch.setattr(native, "_LOAD_ERROR", None)
+
+
+def test_public_names_match_reference_surface():
+    assert set(risa.__all__) == {
+        "KVPermutation", "prepare_kv_permutation", "PrequantizedInt8Attention", "RetainedMassPattern",
+        "build_retained_mass_pattern", "construct_sparse_int8_attention",
+        "construct_sparse_int8_attention_from_prequantized", "int8_attention",
+        "int8_attention_from_prequantized", "int8_attention_is_available", "measure_pattern_recall",
+        "prequantize_int8_attention", "sparse_int8_attention",
+    }
+    fields = [f for f in types.PrequantizedInt8Attention.__dataclass_fields__]
+    assert fields[:16] == ["q", "k", "v", "q_scale", "k_scale", "v_scale", "v_center", "original_head_dim",
+                           "input_dtype", "attention_scale", "cta_k", "attn_mask", "v_quantization",
+                           "is_causal", "lse_shift", "kv_permuted"]
+
+
+def test_tile_policy_and_constants():
+    assert policy.select_key_block_size(128, 1025, has_mask=False) == 128
+    assert policy.select_key_block_size(128, 1024, has_mask=False) == 64
+    assert policy.select_key_block_size(256, 5000, has_mask=True) == 64
+    assert policy.select_key_block_size(64, 5000, has_mask=False) == 64
+    assert policy.pad_key_length(1153, 128) == 1280 and policy.pad_key_length(64) == 64
+    assert policy.MIN_PATTERN_SPARSITY == 0.05 and policy.QUERY_BLOCK_SIZE == 128
+    assert policy.DTYPE_CODES == {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}
+
+
+def test_invalid_v_mode_and_input_errors():
+    q = torch.empty(1)
+    with pytest.raises(ValueError, match="v_quantization"):
+        risa.int8_attention(q, q, q, v_quantization="invalid")
+    x = torch.zeros(1, 2, 3, 64)
+    with pytest.raises(ValueError, match="shape"):
+        policy.validate_inputs(x[0], x, x, None)
+    with pytest.raises(TypeError, match="float32, float16, or bfloat16"):
+        policy.validate_inputs(x.double(), x.double(), x.double(), None)
+    with pytest.raises(TypeError, match="same dtype"):
+        policy.validate_inputs(x, x.half(), x, None)
+    with pytest.raises(ValueError, match="same CUDA device"):
+        policy.validate_inputs(x, x, x, None)  # CPU tensors
+
+
+def test_validation_after_device_gate():
+    x = torch.zeros(1, 4, 3, 64)
+
+    class Fake(torch.Tensor):
+        is_cuda = True
+
+    def cuda_like(t):
+        return t.as_subclass(Fake)
+
+    with patch.object(policy, "is_available", return_value=True):
+        q = cuda_like(x)
+        with pytest.raises(ValueError, match="divisible"):
+            policy.validate_inputs(q, cuda_like(torch.zeros(1, 3, 3, 64)), cuda_like(torch.zeros(1, 3, 3, 64)), None)
+        with pytest.raises(ValueError, match=r"head_dim must be in \[1, 256\]"):
+            big = cuda_like(torch.zeros(1, 1, 2, 300))
+            policy.validate_inputs(big, big, big, None)
+        with pytest.raises(TypeError, match="attn_mask must be bool"):
+            policy.validate_inputs(q, q, q, torch.zeros(3, 3, dtype=torch.int32))
+        with pytest.raises(ValueError, match="broadcastable"):
+            policy.validate_inputs(q, q, q, torch.zeros(5, 5, dtype=torch.bool))
+        mask = policy.validate_inputs(q, q, q, torch.ones(1, 1, 1, 3, dtype=torch.bool))
+        assert mask.shape == (1, 4, 3, 3) and mask.stride(-2) == 0
+    with patch.object(policy, "is_available", return_value=False):
+        with pytest.raises(RuntimeError, match="gfx950"):
+            policy.validate_inputs(cuda_like(x), cuda_like(x), cuda_like(x), None)
+
+
+def test_custom_ops_propagate_causal_and_quantization():
+    q = torch.randn(1, 2, 3, 64)
+    for mode in ("midpoint_affine", "absmax"):
+        for causal in (False, True):
+            for mask in (None, torch.ones(3, 3, dtype=torch.bool)):
+                with patch.object(dense, "execute_dense_attention", return_value=q.clone()) as launch:
+                    risa.int8_attention(q, q, q, attn_mask=mask, is_causal=causal, v_quantization=mode)
+                assert launch.call_args.kwargs["is_causal"] == causal
+                assert launch.call_args.kwargs["use_midpoint_affine"] == (mode == "midpoint_affine")
+                assert (launch.call_args.kwargs["attn_mask"] is None) == (mask is None)
+
+
+def test_fake_tensor_shapes():
+    from torch._subclasses.fake_tensor import FakeTensorMode
+
+    with FakeTensorMode():
+        q = torch.empty(1, 2, 17, 64, device="cuda")
+        for mode in ("midpoint_affine", "absmax"):
+            result = risa.int8_attention(q, q, q, is_causal=True, v_quantization=mode)
+            assert result.shape == q.shape
+            masked = risa.int8_attention(q, q, q, attn_mask=torch.empty(17, 17, device="cuda", dtype=torch.bool))
+            assert masked.shape == q.shape
+
+
+def test_mask_signature_and_score_mask():
+    mask = torch.ones(1, 1, 3, 5, dtype=torch.bool)
+    before = policy.mask_signature(mask)
+    mask[..., 0] = False
+    assert before != policy.mask_signature(mask)
+    assert policy.mask_signature(None) is None
+    scores = policy.apply_score_mask(torch.zeros(1, 1, 3, 5), mask, True, 0)
+    assert torch.isneginf(scores[..., 0, :]).all()
+    assert torch.isneginf(scores[..., 1, 2:]).all()
+    assert scores[0, 0, 1, 1] == 0
+    shifted = policy.apply_score_mask(torch.zeros(1, 1, 2, 5), torch.full((1, 1, 3, 5), 2.0), False, 1)
+    assert (shifted == 2).all()
+
+
+def test_pattern_properties_and_prequantized_checks():
+    pattern = types.RetainedMassPattern(
+        row_offsets=torch.tensor([0, 1, 3], dtype=torch.int32), block_indices=torch.tensor([0, 0, 1], dtype=torch.int32),
+        batch_size=1, q_heads=1, q_length=200, kv_length=130, query_block_size=128, key_block_size=64,
+        attention_scale=0.1, retained_mass_target=0.9, measured_retained_mass=0.95)
+    assert pattern.coverage == pytest.approx(3 / 6) and pattern.sparsity == pytest.approx(0.5)
+    assert pattern.index_bytes == 6 * 4
+    with pytest.raises(TypeError, match="prequantize_int8_attention"):
+        risa.int8_attention_from_prequantized(object())
+    packed = types.PrequantizedInt8Attention(*([torch.zeros(1)] * 7), 64, torch.float16, 0.1, 64, None)
+    with pytest.raises(ValueError, match="output_layout"):
+        risa.int8_attention_from_prequantized(packed, output_layout="dnh")
+    with pytest.raises(ValueError, match="return_lse=True"):
+        risa.int8_attention_from_prequantized(packed, return_lse=True)
+    with pytest.raises(ValueError, match="CUDA device"):
+        risa.int8_attention_from_prequantized(packed)
+    with pytest.raises(ValueError, match="theta"):
+        risa.construct_sparse_int8_attention_from_prequantized(packed, theta=0.0)
+    with pytest.raises(TypeError, match="prequantize_int8_attention"):
+        risa.construct_sparse_int8_attention_from_prequantized(object(), theta=0.5)
+
+
+def test_pattern_compatibility_checks():
+    q = torch.zeros(1, 2, 200, 64, dtype=torch.int8)
+    packed = types.PrequantizedInt8Attention(q, torch.zeros(1, 1, 130, 64, dtype=torch.int8), *([torch.zeros(1)] * 5),
+                                             64, torch.float16, 0.125, 64, None)
+    good = dict(row_offsets=torch.zeros(5, dtype=torch.int32), block_indices=torch.zeros(4, dtype=torch.int32),
+                batch_size=1, q_heads=2, q_length=200, kv_length=130, query_block_size=128, key_block_size=64,
+                attention_scale=0.125, retained_mass_target=0.9, measured_retained_mass=0.9)
+    attend.check_pattern(packed, types.RetainedMassPattern(**good))
+    with pytest.raises(ValueError, match="is_causal"):
+        attend.check_pattern(packed, types.RetainedMassPattern(**{**good, "is_causal": True}))
+    with pytest.raises(ValueError, match="metadata"):
+        attend.check_pattern(packed, types.RetainedMassPattern(**{**good, "key_block_size": 128}))
+    with pytest.raises(ValueError, match="same scale"):
+        attend.check_pattern(packed, types.RetainedMassPattern(**{**good, "attention_scale": 0.126}))
+    with pytest.raises(ValueError, match="mask has changed"):
+        attend.check_pattern(packed, types.RetainedMassPattern(**{**good, "mask_signature": (1,)}))
+    with pytest.raises(TypeError, match="contiguous int32"):
+        attend.check_pattern(packed, types.RetainedMassPattern(**{**good, "row_offsets": torch.zeros(5, dtype=torch.int64)}))
+    with pytest.raises(TypeError, match="build_retained_mass_pattern"):
+        attend.check_pattern(packed, object())
+
+
+def test_packed_value_layout_round_trip():
+    logical = torch.arange(2 * 96, dtype=torch.int8).reshape(2, 96)
+    packed = layout.pack_values(logical)
+    assert torch.equal(layout.unpack_values(packed), logical)
+    order = layout.position_to_token()
+    assert order[:8] == [0, 1, 2, 3, 8, 9, 10, 11] and order[16:20] == [4, 5, 6, 7]
+    assert torch.equal(packed[0, :32], logical[0, order])
+
+
+def test_fp32_pattern_builder_and_recall_on_cpu():
+    g = torch.Generator().manual_seed(0)
+    centroids = torch.randn(4, 64, generator=g) * 3
+    tokens = centroids.repeat_interleave(64, 0)[None, None] + torch.randn(1, 2, 256, 64, generator=g) * 0.3
+    q = k = tokens.contiguous()
+    pattern = fp32_patterns.build_retained_mass_pattern(q, k, theta=0.9)
+    assert pattern.key_block_size == 64 and pattern.query_block_size == 128
+    assert pattern.row_offsets.tolist()[0] == 0 and pattern.row_offsets[-1] == pattern.block_indices.numel()
+    assert 0 < pattern.coverage < 1
+    assert pattern.measured_retained_mass >= 0.9
+    recall = fp32_patterns.measure_pattern_recall(q, k, pattern)
+    assert recall == pytest.approx(pattern.measured_retained_mass, abs=1e-5)
+    dense_pattern = fp32_patterns.build_retained_mass_pattern(q, k, theta=1.0)
+    assert fp32_patterns.measure_pattern_recall(q, k, dense_pattern) == pytest.approx(1.0, abs=1e-6)
+    with pytest.raises(ValueError, match="theta"):
+        fp32_patterns.build_retained_mass_pattern(q, k, theta=1.5)
+    with pytest.raises(ValueError, match="pattern mask has changed"):
+        fp32_patterns.measure_pattern_recall(q, k, pattern, attn_mask=torch.ones(256, 256, dtype=torch.bool))
+
+
+def test_bench_rejects_more_than_one_gpu():
+    import subprocess
+    import sys
+
+    done = subprocess.run([sys.executable, str(ROOT / "bench.py"), "--gpus", "2"], capture_output=True, text=True)
+    assert done.returncode != 0 and "one MI355X" in done.stderr
