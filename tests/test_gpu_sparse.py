@@ -1,0 +1,233 @@
+"""GPU parity of capture, block mass, retained-mass selection, sparse reuse, key-mask tile
+skipping, streams/graphs and full-size invariants (all through the C ABI)."""
+
+from dataclasses import replace
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import attention as oracle_attention
+from oracle import pipeline as oracle_pipeline
+from oracle import selection as oracle_selection
+from tests.helpers import oracle_prequantize, relative_l2, seeded, to_numpy
+
+pytestmark = pytest.mark.gpu
+
+
+def block_structured(batch, q_heads, kv_heads, length, dim, groups, seed, dtype=torch.bfloat16):
+    """Per-group centroid*3 plus unit noise for Q/K, unit-noise V (BASELINE sparse config)."""
+    g = torch.Generator().manual_seed(seed)
+    centroids = torch.randn(batch, kv_heads, groups, dim, generator=g) * 3
+    per_token = centroids.repeat_interleave(length // groups, dim=2)
+    k = (per_token + torch.randn(batch, kv_heads, length, dim, generator=g)).to(dtype).cuda()
+    q = (per_token.repeat_interleave(q_heads // kv_heads, dim=1)
+         + torch.randn(batch, q_heads, length, dim, generator=g)).to(dtype).cuda()
+    v = torch.randn(batch, kv_heads, length, dim, generator=g).to(dtype).cuda()
+    return q, k, v
+
+
+def rows_of(row_offsets, block_indices):
+    ro = np.asarray(row_offsets)
+    bi = np.asarray(block_indices)
+    return [set(bi[ro[r] : ro[r + 1]].tolist()) for r in range(len(ro) - 1)]
+
+
+@pytest.mark.parametrize("length,theta", [(1024, 0.99), (2048, 0.9)])
+@pytest.mark.parametrize("mode", ["absmax", "midpoint_affine"])
+def test_constructed_tile_sets_match_oracle(risa, length, theta, mode):
+    q, k, v = block_structured(1, 4, 2, length, 128, 16, seed=length)
+    out, pattern = risa.construct_sparse_int8_attention(q, k, v, theta=theta, v_quantization=mode)
+    prepared = oracle_prequantize(q, k, v, v_quantization=mode)
+    expected_out, _, cap = oracle_pipeline.attend(prepared, capture=True)
+    masses = oracle_attention.block_mass(cap, 1, 4, length)
+    ro, bi, measured, _ = oracle_selection.select_retained_mass(masses, theta)
+    assert relative_l2(to_numpy(out), expected_out) < 1e-3
+    got = rows_of(pattern.row_offsets.cpu().numpy(), pattern.block_indices.cpu().numpy())
+    want = rows_of(ro, bi)
+    assert len(got) == len(want)
+    for r, (g_set, w_set) in enumerate(zip(got, want)):
+        if g_set == w_set:
+            continue
+        # Documented tie: the symmetric difference may only hold tiles whose mass is within
+        # FP32 reduction noise of the cut (the smallest selected mass of the oracle row).
+        cut = min(masses[r, t] for t in w_set)
+        for t in g_set ^ w_set:
+            assert abs(masses[r, t] - cut) <= 1e-4 * max(cut, 1e-6) + 1e-6, (r, t, masses[r, t], cut)
+    assert pattern.measured_retained_mass == pytest.approx(measured, abs=1e-4)
+    assert 0 < pattern.coverage < 1
+    # reuse with the oracle's own pattern gives the oracle's sparse output
+    oracle_pattern = replace(
+        pattern,
+        row_offsets=torch.from_numpy(ro).cuda(),
+        block_indices=torch.from_numpy(bi).cuda(),
+    )
+    sparse = risa.sparse_int8_attention(q, k, v, oracle_pattern, v_quantization=mode)
+    expected_sparse, _, _ = oracle_pipeline.attend(prepared, pattern=(ro, bi))
+    assert relative_l2(to_numpy(sparse), expected_sparse) < 1e-3
+
+
+def test_block_mass_values_match_oracle(risa):
+    q, k, v = block_structured(1, 2, 1, 1280, 128, 8, seed=5)
+    packed = risa.prequantize_int8_attention(q, k, v)
+    blocks = 1280 // packed.cta_k
+    mass_elements = 2 * 10 * blocks
+    workspace = torch.empty(mass_elements + 2 * 1280 * (blocks * 2 + 2), device="cuda")
+    risa.int8_attention_from_prequantized(packed, _block_mass=workspace)
+    prepared = oracle_prequantize(q, k, v)
+    _, _, cap = oracle_pipeline.attend(prepared, capture=True)
+    expected = oracle_attention.block_mass(cap, 1, 2, 1280)
+    got = workspace[:mass_elements].view(-1, blocks).cpu().numpy()
+    np.testing.assert_allclose(got, expected, rtol=2e-3, atol=2e-3)
+    np.testing.assert_allclose(got.sum(1), 128.0, atol=1e-3)
+
+
+@pytest.mark.parametrize("theta", [0.5, 0.99, 1.0])
+def test_selector_kernel_matches_oracle_exactly(risa, theta):
+    from risaattention_amd.patterns import select_retained_mass_csr
+
+    g = torch.Generator().manual_seed(1)
+    masses = (torch.rand(531, 257, generator=g) ** 6).cuda()
+    masses[7] = 0
+    row_offsets, block_indices, measured = select_retained_mass_csr(masses, theta)
+    order = masses.sort(dim=-1, descending=True).indices.cpu().numpy()
+    ro, bi, expected_measured, _ = oracle_selection.select_retained_mass(masses.cpu().numpy(), theta, order=order)
+    np.testing.assert_array_equal(row_offsets.cpu().numpy(), ro)
+    np.testing.assert_array_equal(block_indices.cpu().numpy(), bi)
+    assert measured == pytest.approx(expected_measured, rel=1e-12)
+
+
+@pytest.mark.parametrize("mask_dtype", [torch.bool, torch.float16, torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("dim", [64, 128, 256])
+def test_key_mask_tile_skipping_matches_generic_mask(risa, mask_dtype, dim):
+    """reference tests/cuda/test_key_mask_tiles.py:16-54."""
+    torch.manual_seed(74)
+    q = torch.randn(2, 4, 257, dim, device="cuda", dtype=torch.bfloat16)
+    k = torch.randn(2, 2, 1153, dim, device="cuda", dtype=q.dtype)
+    v = torch.randn_like(k) + 3
+    storage = torch.zeros(2, 4, 1, 2306, device="cuda", dtype=mask_dtype)
+    mask = storage[..., ::2]
+    visible = torch.ones(2, 4, 1, 1153, device="cuda", dtype=torch.bool)
+    visible[..., :128] = False
+    visible[..., 384:768] = False
+    visible[0, 1] = False
+    visible[1, 2, :, -1] = False
+    visible[..., 897:913] = False
+    if mask_dtype == torch.bool:
+        mask.copy_(visible)
+    else:
+        mask.copy_(torch.linspace(-1, 2, 1153, device="cuda"))
+        mask.masked_fill_(~visible, -torch.inf)
+    packed = risa.prequantize_int8_attention(q, k, v, attn_mask=mask, return_lse=True)
+    generic = replace(packed, attn_mask=packed.attn_mask.clone())
+    actual, lse = risa.int8_attention_from_prequantized(packed, return_lse=True)
+    expected, expected_lse = risa.int8_attention_from_prequantized(generic, return_lse=True)
+    torch.testing.assert_close(actual, expected, atol=0.002, rtol=0.01)
+    torch.testing.assert_close(lse, expected_lse, atol=2e-4, rtol=2e-6)
+    assert torch.count_nonzero(actual[0, 1]) == 0
+    assert torch.isneginf(lse[0, 1]).all()
+    torch.testing.assert_close(risa.int8_attention(q, k, v, attn_mask=mask), actual, atol=0, rtol=0)
+    # and against the oracle
+    prepared = oracle_prequantize(q, k, v, attn_mask=mask, return_lse=True)
+    want, want_lse, _ = oracle_pipeline.attend(prepared, return_lse=True)
+    assert relative_l2(to_numpy(actual), want) < 1e-3
+    assert relative_l2(to_numpy(lse), want_lse) < 1e-3
+
+
+def test_key_mask_tiles_known_answer(risa):
+    """reference tests/cuda/test_key_mask_tiles.py:78-104."""
+    from risaattention_amd.key_mask import prepare_key_mask_tiles
+
+    q = torch.randn(1, 4, 257, 128, device="cuda", dtype=torch.bfloat16)
+    k = torch.randn(1, 2, 1153, 128, device="cuda", dtype=q.dtype)
+    v = torch.randn_like(k)
+    mask = torch.ones(1, 1, 1, 1153, device="cuda", dtype=torch.bool)
+    mask[..., :512] = False
+    packed = risa.prequantize_int8_attention(q, k, v, attn_mask=mask)
+    tiles = prepare_key_mask_tiles(packed.attn_mask, packed.cta_k, 257, packed.attention_scale, False)
+    expected = torch.tensor([4, 5, 6, 7, 8, 9], device="cuda", dtype=torch.int32)
+    assert torch.equal(tiles[..., :6], expected.expand(1, 4, 6))
+    assert (tiles[..., -1] == 6).all()
+    assert prepare_key_mask_tiles(packed.attn_mask, packed.cta_k, 255, packed.attention_scale, False) is None
+    assert prepare_key_mask_tiles(packed.attn_mask, packed.cta_k, 257, packed.attention_scale, True) is None
+    assert prepare_key_mask_tiles(packed.attn_mask, packed.cta_k, 257, 0.0, False) is None
+
+
+@pytest.mark.parametrize("mode", ["absmax", "midpoint_affine"])
+def test_nondefault_stream_and_graph_replay(risa, mode):
+    """reference tests/cuda/test_probability_mass.py:94-108 and test_value_quantization.py:75-90."""
+    q = torch.randn(1, 4, 2049, 128, device="cuda", dtype=torch.bfloat16)
+    k, v = [torch.randn(1, 2, 2049, 128, device="cuda", dtype=q.dtype) for _ in range(2)]
+    stream = torch.cuda.Stream()
+    stream.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(stream):
+        packed = risa.prequantize_int8_attention(q, k, v, v_quantization=mode)
+        expected = risa.int8_attention_from_prequantized(packed)
+        expected_full = risa.int8_attention(q, k, v, v_quantization=mode)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            actual = risa.int8_attention_from_prequantized(packed)
+            actual_full = risa.int8_attention(q, k, v, v_quantization=mode)
+        for _ in range(3):
+            actual.zero_()
+            actual_full.zero_()
+            graph.replay()
+            stream.synchronize()
+            assert torch.equal(actual, expected)
+            assert torch.equal(actual_full, expected_full)
+    torch.cuda.current_stream().wait_stream(stream)
+    assert torch.equal(expected, expected_full)
+
+
+def test_prequantized_nhd_layout_and_head_dim_padding(risa):
+    q = seeded((2, 4, 150, 80), torch.float16, 1)
+    k = seeded((2, 2, 333, 80), torch.float16, 2)
+    v = seeded((2, 2, 333, 80), torch.float16, 3)
+    packed = risa.prequantize_int8_attention(q, k, v)
+    hnd = risa.int8_attention_from_prequantized(packed)
+    nhd = risa.int8_attention_from_prequantized(packed, output_layout="nhd")
+    assert hnd.shape == nhd.shape == (2, 4, 150, 80)
+    assert nhd.transpose(1, 2).reshape(2, 150, -1).shape == (2, 150, 320)
+    assert torch.equal(hnd, nhd)
+    assert torch.equal(hnd, risa.int8_attention(q, k, v))
+
+
+def test_input_strides_do_not_change_results(risa):
+    base = seeded((1, 300, 3, 4, 128), torch.bfloat16, 9)
+    q = base[:, :, 0].transpose(1, 2)
+    k = base[:, :, 1, :2].transpose(1, 2)
+    v = base[:, :, 2, :2].transpose(1, 2)
+    strided = risa.int8_attention(q, k, v, v_quantization="midpoint_affine")
+    dense = risa.int8_attention(q.contiguous(), k.contiguous(), v.contiguous(), v_quantization="midpoint_affine")
+    assert torch.equal(strided, dense)
+
+
+def test_dense_fallback_for_nearly_dense_pattern(risa):
+    q = seeded((1, 2, 512, 128), torch.bfloat16, 3)
+    k = seeded((1, 1, 512, 128), torch.bfloat16, 4)
+    v = seeded((1, 1, 512, 128), torch.bfloat16, 5)
+    built, pattern = risa.construct_sparse_int8_attention(q, k, v, theta=1.0)
+    assert pattern.sparsity < 0.05
+    sparse = risa.sparse_int8_attention(q, k, v, pattern)
+    assert torch.equal(sparse, risa.int8_attention(q, k, v))
+    with pytest.raises(ValueError, match="is_causal"):
+        risa.sparse_int8_attention(q, k, v, pattern, is_causal=True)
+
+
+def test_full_size_invariants(risa):
+    """Headline shape (N=32K, Hq16/Hkv4/D128, bf16): properties that need no oracle run."""
+    length = 32768
+    g = torch.Generator(device="cuda").manual_seed(0)
+    q = torch.randn(1, 16, length, 128, generator=g, device="cuda", dtype=torch.bfloat16)
+    k = torch.randn(1, 4, length, 128, generator=g, device="cuda", dtype=torch.bfloat16)
+    values = torch.linspace(-3, 5, 128, device="cuda", dtype=torch.bfloat16)
+    v = values.expand_as(k).contiguous()
+    out, lse = risa.int8_attention(q, k, v, return_lse=True)
+    assert torch.equal(out, values.expand_as(out))
+    zero_scale, lse0 = risa.int8_attention(q, k, v, scale=0.0, return_lse=True)
+    assert torch.equal(zero_scale, values.expand_as(out))
+    torch.testing.assert_close(lse0, torch.full_like(lse0, float(np.log(length))), atol=2e-5, rtol=0)
+    # LSE against FP32 on a slice of queries
+    rows = slice(1000, 1128)
+    scores = q[:, :4, rows].float() @ k[:, :1].float().transpose(-1, -2) / 128**0.5
+    torch.testing.assert_close(lse[:, :4, rows], scores.logsumexp(-1), atol=0.02, rtol=0)
