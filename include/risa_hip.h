@@ -57,8 +57,9 @@ int risa_quantize_qk(const void* q, void* q_int8, float* q_scale, const void* k,
  * csrc/kernels/quantize_v_impl.cuh:314-409).
  *   v [B,Hkv,L,D] strided (16-byte aligned rows), out int8 [B*Hkv*D, padded] in
  *   the packed order documented at risa_unpack_order, scale/center [B*Hkv*D],
- *   tile_sum int32 [B*Hkv, padded/cta_k, D] (sum of the codes of each key tile,
- *   the zero-point term of the signed P*V product; no reference counterpart),
+ *   tile_sum int32 [B*Hkv, padded/cta_k, D] (128 x the sum of the codes of each
+ *   key tile, the zero-point term of the signed P*V product; no reference
+ *   counterpart),
  *   workspace of risa_quantize_v_workspace_bytes(...) bytes.
  */
 size_t risa_quantize_v_workspace_bytes(int batch, int heads, int length, int head_dim,
@@ -70,7 +71,7 @@ int risa_quantize_v(const void* v, void* out, float* scale, float* center, int32
                     void* stream);
 
 /*
- * Tile sums of an already packed V matrix (for callers that build packed V
+ * Zero-point terms (128 x tile sums) of an already packed V matrix (for callers that build packed V
  * themselves, as reference tests/cuda/test_large_offsets.py:35-36 does).
  */
 int risa_value_tile_sums(const void* v_int8, int32_t* tile_sum, int batch_heads, int head_dim,

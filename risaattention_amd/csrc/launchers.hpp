@@ -42,7 +42,7 @@ struct ValueArgs {
   int8_t* codes;     // [B*H*D, padded] in packed MFMA order
   float* scale;      // [B*H*D]
   float* center;     // [B*H*D]
-  int32_t* tile_sum; // [B*H, padded/cta_k, D]
+  int32_t* tile_sum; // [B*H, padded/cta_k, D], 128 x sum of codes
   void* workspace;
   size_t workspace_bytes;
   int batch, heads, length, head_dim, padded, cta_k, dtype;
