@@ -159,9 +159,8 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void attention_kernel(cons
   // --- per-lane copy descriptors (constant over tiles) -----------------------
   // Copy instruction i of this wave fills LDS bytes [(wave*NC+i)*1024, +1024) of
   // a tile; this lane supplies chunk `lane` of that kilobyte.
-  int k_src_offset[NC];          // byte offset of the source chunk inside a K tile
-  int k_row[NC];                 // key row inside the tile (for the tail predicate)
-  const int8_t* v_src_row[NC];   // source pointer of the chunk for tile 0
+  int k_src_offset[NC];       // byte offset of the source chunk inside a K tile
+  uint32_t v_src_offset[NC];  // byte offset of the source chunk inside the head's V slab, tile 0
 #pragma unroll
   for (int i = 0; i < NC; ++i) {
     const int slot = (wave * NC + i) * 64 + lane;
@@ -170,13 +169,12 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void attention_kernel(cons
       const int row = slot / CH, phys = slot % CH;
       const int chunk = phys ^ ((row / (256 / D)) & (CH - 1));
       k_src_offset[i] = row * D + chunk * 16;
-      k_row[i] = row;
     }
     {
       constexpr int CH = CTA_K / 16;
       const int row = slot / CH, phys = slot % CH;
       const int chunk = phys ^ ((row / (256 / CTA_K)) & (CH - 1));
-      v_src_row[i] = v_base + static_cast<int64_t>(row) * p.padded + chunk * 16;
+      v_src_offset[i] = static_cast<uint32_t>(row) * static_cast<uint32_t>(p.padded) + chunk * 16;
     }
   }
   auto issue_tile = [&](int tile, int stage) {
@@ -184,14 +182,17 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void attention_kernel(cons
     unsigned char* vl = kl + Shape::kTileBytes;
     unsigned char* sl = vl + Shape::kTileBytes;
     const int8_t* k_tile = k_base + static_cast<int64_t>(tile) * CTA_K * D;
-    const int rows_left = p.k_len - tile * CTA_K;  // >= CTA_K except for the tail tile
+    const int8_t* v_tile = v_base + static_cast<int64_t>(tile) * CTA_K;
+    // Keys past the end exist only in the tail tile; their LDS rows keep stale
+    // bytes, which is harmless because those scores are masked by index.
+    const int bytes_left = (p.k_len - tile * CTA_K) * D;
 #pragma unroll
     for (int i = 0; i < NC; ++i) {
-      if (k_row[i] < rows_left) copy16_to_lds(k_tile + k_src_offset[i], kl + (wave * NC + i) * 1024);
+      if (k_src_offset[i] < bytes_left) copy16_to_lds(k_tile + k_src_offset[i], kl + (wave * NC + i) * 1024);
     }
 #pragma unroll
     for (int i = 0; i < NC; ++i) {
-      copy16_to_lds(v_src_row[i] + static_cast<int64_t>(tile) * CTA_K, vl + (wave * NC + i) * 1024);
+      copy16_to_lds(v_tile + v_src_offset[i], vl + (wave * NC + i) * 1024);
     }
     if (wave == 0 && lane < D / 4) {
       copy16_to_lds(sum_base + static_cast<int64_t>(tile) * D + lane * 4, sl);
@@ -237,36 +238,54 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void attention_kernel(cons
                 static_cast<int64_t>(query) * p.mask_stride_q
           : 0;
 
-  // One key tile.  LAST selects the formulas of the last listed tile.
-  auto process_tile = [&](auto last_tag, int it, int tile, int stage, float ks0, float ks1) {
-    constexpr bool LAST = decltype(last_tag)::value;
+  // ---- S^T = K · Q^T for the tile staged in `stage` ---------------------------
+  // The K fragments of k-step kk+1 are requested from LDS before the MFMAs of
+  // k-step kk are issued, so the LDS latency hides behind RB matrix instructions.
+  auto load_k_fragments = [&](const unsigned char* kl, int kk, v4i (&frag)[RB]) {
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb)
+      frag[rb] = *reinterpret_cast<const v4i*>(kl + swizzled<D>(rb * 32 + l32, kk * 2 + half));
+  };
+  auto score_tile = [&](int stage, v4i (&first)[RB], v16i (&s)[RB]) {
     const unsigned char* kl = lds + stage * Shape::kStageBytes;
-    const unsigned char* vl = kl + Shape::kTileBytes;
-    const int* sl = reinterpret_cast<const int*>(vl + Shape::kTileBytes);
-
-    // ---- S^T = K · Q^T ----------------------------------------------------
-    v16i s[RB];
+    v4i frag[2][RB];
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) frag[0][rb] = first[rb];
 #pragma unroll
     for (int kk = 0; kk < KK; ++kk) {
+      if (kk + 1 < KK) load_k_fragments(kl, kk + 1, frag[(kk + 1) & 1]);
+      __builtin_amdgcn_sched_group_barrier(0x100, RB, 0);  // RB LDS reads ...
 #pragma unroll
       for (int rb = 0; rb < RB; ++rb) {
-        const v4i a = *reinterpret_cast<const v4i*>(kl + swizzled<D>(rb * 32 + l32, kk * 2 + half));
         if (kk == 0) {
           const v16i zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-          s[rb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, qreg[kk], zero, 0, 0, 0);
+          s[rb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(frag[kk & 1][rb], qreg[kk], zero, 0, 0, 0);
         } else {
-          s[rb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, qreg[kk], s[rb], 0, 0, 0);
+          s[rb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(frag[kk & 1][rb], qreg[kk], s[rb], 0, 0, 0);
         }
       }
+      __builtin_amdgcn_sched_group_barrier(0x008, RB, 0);  // ... then RB MFMAs
     }
+  };
 
+  // ---- scores -> U8 probabilities (as signed bytes) and the online-softmax state.
+  // LAST selects the formulas of the last listed tile.  Returns the factor the
+  // tile's integer P·V is scaled by.
+  //
+  // The running reference m_run only moves when a tile maximum exceeds it by
+  // more than kRescaleSlack: O and d are then relative to 2^m_run instead of
+  // 2^(true running maximum), which cancels in O/d and in log2(d) + m_run and
+  // changes FP32 rounding only, while the output accumulators are rescaled on
+  // a handful of tiles instead of on every new maximum.
+  constexpr float kRescaleSlack = 8.0f;
+  auto softmax_tile = [&](auto last_tag, int it, int tile, float ks0, float ks1, v16i (&s)[RB],
+                          v4i (&pk)[RB]) -> float {
+    constexpr bool LAST = decltype(last_tag)::value;
     // K scale groups of this lane: keys 8b+4*half+r, group (key % 8) / 2 = 2*half + r/2.
     const float sc0 = qs2 * (q_scale * ks0);
     const float sc1 = qs2 * (q_scale * ks1);
     const int key0 = tile * CTA_K + half * 4;  // element (rb, i) is key key0 + rb*32 + (i>>2)*8 + (i&3)
-
     float tile_m;
-    v4i pk[RB];
     uint32_t row_sum = 0;
 
     if constexpr (FAST && !LAST) {
@@ -378,11 +397,18 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void attention_kernel(cons
     }
 
     // ---- online softmax state ----------------------------------------------
-    const float alpha = __builtin_amdgcn_exp2f(-__builtin_fabsf(m_run - tile_m));
-    const float o_scale = m_run < tile_m ? alpha : 1.0f;
-    const float t_scale = tile_m < m_run ? alpha : 1.0f;
-    m_run = __builtin_fmaxf(m_run, tile_m);
-    d_part = d_part * o_scale + static_cast<float>(row_sum) * t_scale;
+    const bool raise = tile_m > m_run + kRescaleSlack;
+    if (__builtin_amdgcn_ballot_w64(raise) != 0) {
+      const float o_scale = raise ? __builtin_amdgcn_exp2f(m_run - tile_m) : 1.0f;
+      m_run = raise ? tile_m : m_run;
+      d_part *= o_scale;
+#pragma unroll
+      for (int cb = 0; cb < CB; ++cb)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) o_acc[cb][i] *= o_scale;
+    }
+    const float t_scale = __builtin_amdgcn_exp2f(tile_m - m_run);
+    d_part = __builtin_fmaf(static_cast<float>(row_sum), t_scale, d_part);
 
     if constexpr (CAPTURE) {
       const uint32_t numerator = row_sum + __shfl_xor(row_sum, 32);
@@ -398,70 +424,127 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void attention_kernel(cons
         }
       }
     }
+    return t_scale;
+  };
 
-    // Rescaling the output accumulators is the identity unless some row of this
-    // wavefront raised its running maximum.
-    if (__builtin_amdgcn_ballot_w64(o_scale != 1.0f) != 0) {
+  // ---- O^T += t_scale * (128*sum(V) + V^T · P_s8^T) -----------------------------
+  // Channel blocks are processed in pairs (two independent MFMA chains keep the
+  // matrix pipe busy).  LDS operands are requested ahead of use: the accumulator
+  // seeds (zero-point terms) and first V fragments of the first pair before the
+  // exponentials when PREFETCH is set, everything else one step ahead of its MFMAs.
+  constexpr bool PREFETCH = FAST && D <= 128;
+  auto load_seed_pair = [&](int stage, int cb, v16i (&acc)[2]) {
+    const int* sl = reinterpret_cast<const int*>(lds + stage * Shape::kStageBytes + 2 * Shape::kTileBytes);
 #pragma unroll
-      for (int cb = 0; cb < CB; ++cb)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) o_acc[cb][i] *= o_scale;
-    }
-
-    // ---- O^T += V^T · P^T: two channel blocks in flight per step ------------
-    auto load_init = [&](int cb) {
-      v16i acc;
+    for (int j = 0; j < 2; ++j) {
 #pragma unroll
       for (int b4 = 0; b4 < 4; ++b4) {
-        const v4i init = *reinterpret_cast<const v4i*>(sl + cb * 32 + b4 * 8 + half * 4);
-        acc[b4 * 4 + 0] = init[0];
-        acc[b4 * 4 + 1] = init[1];
-        acc[b4 * 4 + 2] = init[2];
-        acc[b4 * 4 + 3] = init[3];
-      }
-      return acc;
-    };
-#pragma unroll
-    for (int cb = 0; cb < CB; cb += 2) {
-      v16i acc0 = load_init(cb);
-      v16i acc1 = load_init(cb + 1);
-#pragma unroll
-      for (int rb = 0; rb < RB; ++rb) {
-        const v4i a0 = *reinterpret_cast<const v4i*>(vl + swizzled<CTA_K>(cb * 32 + l32, rb * 2 + half));
-        const v4i a1 = *reinterpret_cast<const v4i*>(vl + swizzled<CTA_K>(cb * 32 + 32 + l32, rb * 2 + half));
-        acc0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a0, pk[rb], acc0, 0, 0, 0);
-        acc1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a1, pk[rb], acc1, 0, 0, 0);
-      }
-#pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        o_acc[cb][i] = __builtin_fmaf(static_cast<float>(acc0[i]), t_scale, o_acc[cb][i]);
-        o_acc[cb + 1][i] = __builtin_fmaf(static_cast<float>(acc1[i]), t_scale, o_acc[cb + 1][i]);
+        const v4i init = *reinterpret_cast<const v4i*>(sl + (cb + j) * 32 + b4 * 8 + half * 4);
+        acc[j][b4 * 4 + 0] = init[0];
+        acc[j][b4 * 4 + 1] = init[1];
+        acc[j][b4 * 4 + 2] = init[2];
+        acc[j][b4 * 4 + 3] = init[3];
       }
     }
   };
+  auto load_v_pair = [&](int stage, int cb, int rb, v4i (&frag)[2]) {
+    const unsigned char* vl = lds + stage * Shape::kStageBytes + Shape::kTileBytes;
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+      frag[j] = *reinterpret_cast<const v4i*>(vl + swizzled<CTA_K>((cb + j) * 32 + l32, rb * 2 + half));
+  };
+  auto value_tile = [&](int stage, const v4i (&pk)[RB], v16i (&seed0)[2], v4i (&first0)[2], float t_scale) {
+    // Three accumulator sets rotate when there are more than two pairs: one being
+    // seeded, one being multiplied, one being folded into the output.
+    constexpr int SETS = CB / 2 > 2 ? 3 : 2;
+    v16i acc[SETS][2];  // [pair % SETS][block of the pair]
+    v4i frag[2][2];     // [step parity][block of the pair]
+    acc[0][0] = seed0[0];
+    acc[0][1] = seed0[1];
+    frag[0][0] = first0[0];
+    frag[0][1] = first0[1];
+    int step = 0;
+#pragma unroll
+    for (int pair = 0; pair < CB / 2; ++pair) {
+      const int cb = pair * 2;
+      if (pair + 1 < CB / 2) load_seed_pair(stage, cb + 2, acc[(pair + 1) % SETS]);
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb, ++step) {
+        // request the operands of the next step before this step's MFMAs
+        if (rb + 1 < RB) {
+          load_v_pair(stage, cb, rb + 1, frag[(step + 1) & 1]);
+        } else if (pair + 1 < CB / 2) {
+          load_v_pair(stage, cb + 2, 0, frag[(step + 1) & 1]);
+        }
+        acc[pair % SETS][0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(frag[step & 1][0], pk[rb], acc[pair % SETS][0], 0, 0, 0);
+        acc[pair % SETS][1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(frag[step & 1][1], pk[rb], acc[pair % SETS][1], 0, 0, 0);
+      }
+      if (pair > 0) {
+        // fold the previous pair while this pair's MFMAs run
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          o_acc[cb - 2][i] = __builtin_fmaf(static_cast<float>(acc[(pair - 1) % SETS][0][i]), t_scale, o_acc[cb - 2][i]);
+          o_acc[cb - 1][i] = __builtin_fmaf(static_cast<float>(acc[(pair - 1) % SETS][1][i]), t_scale, o_acc[cb - 1][i]);
+        }
+      }
+    }
+    constexpr int last_pair = CB / 2 - 1;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      o_acc[CB - 2][i] = __builtin_fmaf(static_cast<float>(acc[last_pair % SETS][0][i]), t_scale, o_acc[CB - 2][i]);
+      o_acc[CB - 1][i] = __builtin_fmaf(static_cast<float>(acc[last_pair % SETS][1][i]), t_scale, o_acc[CB - 1][i]);
+    }
+  };
 
-  // --- main loop --------------------------------------------------------------
+  // --- main loop: one barrier per tile -----------------------------------------
+  // At the barrier of iteration t every wave has finished tile t-1 (so stage
+  // (t+1)&1 may be overwritten) and has seen its own share of tile t land.
   if (n_it > 0) {
-    issue_tile(tile_at(0), 0);
+    v16i s[RB];
+    v4i pk[RB];
+    v4i k_first[RB];
+    v4i v_first[2];
+    v16i seed[2];
     int tile = tile_at(0);
+    issue_tile(tile, 0);
     float ks0 = ks_base[tile * 4 + 2 * half];
     float ks1 = ks_base[tile * 4 + 2 * half + 1];
     for (int it = 0; it < n_it - 1; ++it) {
       const int stage = it & 1;
       const int next_tile = tile_at(it + 1);
-      __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wave's share of the tile has landed
+      __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
       __syncthreads();
+      load_k_fragments(lds + stage * Shape::kStageBytes, 0, k_first);
       issue_tile(next_tile, stage ^ 1);
       const float next_ks0 = ks_base[next_tile * 4 + 2 * half];
       const float next_ks1 = ks_base[next_tile * 4 + 2 * half + 1];
-      process_tile(std::false_type{}, it, tile, stage, ks0, ks1);
+      score_tile(stage, k_first, s);
+      if constexpr (PREFETCH) {
+        load_seed_pair(stage, 0, seed);
+        load_v_pair(stage, 0, 0, v_first);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      const float t_scale = softmax_tile(std::false_type{}, it, tile, ks0, ks1, s, pk);
+      if constexpr (PREFETCH) {
+        __builtin_amdgcn_sched_barrier(0);
+      } else {
+        load_seed_pair(stage, 0, seed);
+        load_v_pair(stage, 0, 0, v_first);
+      }
+      value_tile(stage, pk, seed, v_first, t_scale);
       tile = next_tile;
       ks0 = next_ks0;
       ks1 = next_ks1;
     }
+    const int stage = (n_it - 1) & 1;
     __builtin_amdgcn_s_waitcnt(0x0f70);
     __syncthreads();
-    process_tile(std::true_type{}, n_it - 1, tile, (n_it - 1) & 1, ks0, ks1);
+    load_k_fragments(lds + stage * Shape::kStageBytes, 0, k_first);
+    score_tile(stage, k_first, s);
+    const float t_scale = softmax_tile(std::true_type{}, n_it - 1, tile, ks0, ks1, s, pk);
+    load_seed_pair(stage, 0, seed);
+    load_v_pair(stage, 0, 0, v_first);
+    value_tile(stage, pk, seed, v_first, t_scale);
   }
 
   // ---- epilogue --------------------------------------------------------------
