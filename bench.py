@@ -103,6 +103,8 @@ def main():
     parser.add_argument("--mode", default="absmax", choices=["absmax", "midpoint_affine"])
     parser.add_argument("--no-cpu-baseline", action="store_true")
     parser.add_argument("--no-accuracy", action="store_true")
+    parser.add_argument("--calibrate-copy", action="store_true",
+                        help="only run a 1 GiB device copy (reference point for rocprofv3 FETCH_SIZE/WRITE_SIZE)")
     args = parser.parse_args()
     if args.gpus != 1:
         print("bench.py measures one MI355X; this path uses no second GPU (see DESIGN.md on sharding)",
@@ -118,6 +120,14 @@ def main():
     if not risa.int8_attention_is_available():
         raise SystemExit("bench.py needs a gfx950 GPU and the built HIP extension")
     device = torch.device("cuda", 0)
+    if args.calibrate_copy:
+        source = torch.empty(1 << 30, dtype=torch.uint8, device=device).random_(0, 255)
+        target = torch.empty_like(source)
+        for _ in range(3):
+            target.copy_(source)
+        torch.cuda.synchronize()
+        print(json.dumps({"calibration": "copy", "bytes_read": 1 << 30, "bytes_written": 1 << 30}))
+        return
     length = args.length
     q, k, v = make_inputs(torch, length, 0, device)
     ops = dense_equivalent_ops(SHAPE["batch"], SHAPE["q_heads"], length, length, SHAPE["head_dim"])
