@@ -57,9 +57,10 @@ int risa_quantize_qk(const void* q, void* q_int8, float* q_scale, const void* k,
  * csrc/kernels/quantize_v_impl.cuh:314-409).
  *   v [B,Hkv,L,D] strided (16-byte aligned rows), out int8 [B*Hkv*D, padded] in
  *   the packed order documented at risa_unpack_order, scale/center [B*Hkv*D],
- *   tile_sum int32 [B*Hkv, padded/cta_k, D] (128 x the sum of the codes of each
- *   key tile, the zero-point term of the signed P*V product; no reference
- *   counterpart),
+ *   tile_sum int32 [B*Hkv, padded/cta_k, D]: the accumulator seeds of the P*V
+ *   product, 128 x the sum of the codes of each key tile (the zero-point term
+ *   of the signed product) + 0x4B400000 (the bits of 1.5 * 2^23, which make the
+ *   finished integer accumulator readable as a float); no reference counterpart,
  *   workspace of risa_quantize_v_workspace_bytes(...) bytes.
  */
 size_t risa_quantize_v_workspace_bytes(int batch, int heads, int length, int head_dim,

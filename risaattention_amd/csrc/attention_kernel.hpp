@@ -25,7 +25,9 @@
 //     sum_j P_u8[j] V[c][j] = sum_j P_s8[j] V[c][j] + 128 * sum_j V[c][j]:
 //     the accumulator of every tile starts from 128 * (tile sum of V codes of
 //     channel c), which the preparation kernel provides, and P_s8 = P_u8 ^ 0x80.
-//     The result is the exact integer the unsigned product would give.
+//     The result is the exact integer the unsigned product would give.  The seed
+//     also carries the bit pattern of 1.5 * 2^23, so the finished accumulator read
+//     as a float is 12582912 + n exactly (risa::kAccumulatorSeedBits).
 #pragma once
 
 #include "common.hpp"
@@ -52,7 +54,7 @@ struct KernelParams {
   const float* k_scale;
   const float* v_scale;
   const float* v_center;
-  const int32_t* v_tile_sum;  // 128 * sum of V codes per (kv head, key tile, channel)
+  const int32_t* v_tile_sum;  // accumulator seeds per (kv head, key tile, channel)
   const void* mask;
   int64_t mask_stride_b, mask_stride_h, mask_stride_q, mask_stride_k;
   int mask_dtype;  // -1: no mask
@@ -90,6 +92,17 @@ __device__ __forceinline__ void copy16_to_lds(const void* src, unsigned char* ld
   typedef const __attribute__((address_space(1))) void* GlobalPointer;
   typedef __attribute__((address_space(3))) void* LdsPointer;
   __builtin_amdgcn_global_load_lds((GlobalPointer)src, (LdsPointer)lds_wave_base, 16, 0, 0);
+}
+
+// Same copy with the address given as a wave-uniform base plus a 32-bit byte
+// offset per lane, the form the instruction takes without any vector ALU work
+// (scalar base register pair + one offset register).  The empty asm keeps the
+// zero extension of the offset next to the copy, where instruction selection
+// can fold it; hoisted out of the loop it would cost a 64-bit vector add per copy.
+__device__ __forceinline__ void copy16_to_lds_uniform(const int8_t* uniform_base, uint32_t lane_offset,
+                                                      unsigned char* lds_wave_base) {
+  asm volatile("" : "+v"(lane_offset));
+  copy16_to_lds(uniform_base + static_cast<uint64_t>(lane_offset), lds_wave_base);
 }
 
 template <int D, int CTA_K> struct TileShape {
@@ -159,7 +172,7 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void attention_kernel(cons
   // --- per-lane copy descriptors (constant over tiles) -----------------------
   // Copy instruction i of this wave fills LDS bytes [(wave*NC+i)*1024, +1024) of
   // a tile; this lane supplies chunk `lane` of that kilobyte.
-  int k_src_offset[NC];       // byte offset of the source chunk inside a K tile
+  uint32_t k_src_offset[NC];  // byte offset of the source chunk inside a K tile
   uint32_t v_src_offset[NC];  // byte offset of the source chunk inside the head's V slab, tile 0
 #pragma unroll
   for (int i = 0; i < NC; ++i) {
@@ -178,22 +191,27 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void attention_kernel(cons
     }
   }
   auto issue_tile = [&](int tile, int stage) {
-    unsigned char* kl = lds + stage * Shape::kStageBytes;
-    unsigned char* vl = kl + Shape::kTileBytes;
-    unsigned char* sl = vl + Shape::kTileBytes;
+    unsigned char* k_slot = lds + stage * Shape::kStageBytes + wave * (NC * 1024);
+    unsigned char* v_slot = k_slot + Shape::kTileBytes;
+    unsigned char* sl = lds + stage * Shape::kStageBytes + 2 * Shape::kTileBytes;
     const int8_t* k_tile = k_base + static_cast<int64_t>(tile) * CTA_K * D;
     const int8_t* v_tile = v_base + static_cast<int64_t>(tile) * CTA_K;
-    // Keys past the end exist only in the tail tile; their LDS rows keep stale
-    // bytes, which is harmless because those scores are masked by index.
-    const int bytes_left = (p.k_len - tile * CTA_K) * D;
+    const int keys_left = p.k_len - tile * CTA_K;
+    if (keys_left >= CTA_K) {
 #pragma unroll
-    for (int i = 0; i < NC; ++i) {
-      if (k_src_offset[i] < bytes_left) copy16_to_lds(k_tile + k_src_offset[i], kl + (wave * NC + i) * 1024);
+      for (int i = 0; i < NC; ++i) copy16_to_lds_uniform(k_tile, k_src_offset[i], k_slot + i * 1024);
+    } else {
+      // Keys past the end exist only in the tail tile; their LDS rows keep stale
+      // bytes, which is harmless because those scores are masked by index.
+      const uint32_t bytes_left = static_cast<uint32_t>(keys_left) * D;
+#pragma unroll
+      for (int i = 0; i < NC; ++i) {
+        if (k_src_offset[i] < bytes_left)
+          copy16_to_lds(k_tile + k_src_offset[i], k_slot + i * 1024);
+      }
     }
 #pragma unroll
-    for (int i = 0; i < NC; ++i) {
-      copy16_to_lds(v_tile + v_src_offset[i], vl + (wave * NC + i) * 1024);
-    }
+    for (int i = 0; i < NC; ++i) copy16_to_lds_uniform(v_tile, v_src_offset[i], v_slot + i * 1024);
     if (wave == 0 && lane < D / 4) {
       copy16_to_lds(sum_base + static_cast<int64_t>(tile) * D + lane * 4, sl);
     }
@@ -220,6 +238,11 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void attention_kernel(cons
     for (int i = 0; i < 16; ++i) o_acc[cb][i] = 0.0f;
   float m_run = kRowFloor;
   float d_part = 0.0f;  // this lane's half of the row denominator
+  // The float whose bits the P·V accumulators start from, kept in a vector
+  // register: with a literal or scalar operand the subtraction that removes it
+  // issues at half the rate.
+  float seed_value;
+  asm volatile("v_mov_b32 %0, %1" : "=v"(seed_value) : "s"(kAccumulatorSeedBits));
 
   // capture bookkeeping
   [[maybe_unused]] uint32_t* stats = nullptr;
@@ -453,6 +476,7 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void attention_kernel(cons
     for (int j = 0; j < 2; ++j)
       frag[j] = *reinterpret_cast<const v4i*>(vl + swizzled<CTA_K>((cb + j) * 32 + l32, rb * 2 + half));
   };
+  auto unseed = [&](int bits) { return __int_as_float(bits) - seed_value; };
   auto value_tile = [&](int stage, const v4i (&pk)[RB], v16i (&seed0)[2], v4i (&first0)[2], float t_scale) {
     // Three accumulator sets rotate when there are more than two pairs: one being
     // seeded, one being multiplied, one being folded into the output.
@@ -483,16 +507,16 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void attention_kernel(cons
         // fold the previous pair while this pair's MFMAs run
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
-          o_acc[cb - 2][i] = __builtin_fmaf(static_cast<float>(acc[(pair - 1) % SETS][0][i]), t_scale, o_acc[cb - 2][i]);
-          o_acc[cb - 1][i] = __builtin_fmaf(static_cast<float>(acc[(pair - 1) % SETS][1][i]), t_scale, o_acc[cb - 1][i]);
+          o_acc[cb - 2][i] = __builtin_fmaf(unseed(acc[(pair - 1) % SETS][0][i]), t_scale, o_acc[cb - 2][i]);
+          o_acc[cb - 1][i] = __builtin_fmaf(unseed(acc[(pair - 1) % SETS][1][i]), t_scale, o_acc[cb - 1][i]);
         }
       }
     }
     constexpr int last_pair = CB / 2 - 1;
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
-      o_acc[CB - 2][i] = __builtin_fmaf(static_cast<float>(acc[last_pair % SETS][0][i]), t_scale, o_acc[CB - 2][i]);
-      o_acc[CB - 1][i] = __builtin_fmaf(static_cast<float>(acc[last_pair % SETS][1][i]), t_scale, o_acc[CB - 1][i]);
+      o_acc[CB - 2][i] = __builtin_fmaf(unseed(acc[last_pair % SETS][0][i]), t_scale, o_acc[CB - 2][i]);
+      o_acc[CB - 1][i] = __builtin_fmaf(unseed(acc[last_pair % SETS][1][i]), t_scale, o_acc[CB - 1][i]);
     }
   };
 

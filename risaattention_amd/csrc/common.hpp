@@ -139,6 +139,14 @@ __device__ __forceinline__ uint32_t pack_s8x4(int a, int b, int c, int d) {
          ((static_cast<uint32_t>(c) & 0xffu) << 16) | ((static_cast<uint32_t>(d) & 0xffu) << 24);
 }
 
+// Accumulator seed of the P·V product.  The matrix cores add integers to whatever
+// 32-bit pattern they start from; starting from the bits of 1.5 * 2^23 (plus the
+// zero-point term) leaves the bits of the float 12582912 + n for every result
+// |n| < 2^22, and 255 * 128 * 128 keys stays below that.  One exact float
+// subtraction then replaces the slower integer-to-float conversion.
+constexpr int32_t kAccumulatorSeedBits = 0x4B400000;
+constexpr float kAccumulatorSeed = 12582912.0f;
+
 // Position of token `t` (0..31) inside its 32-token group of the packed V
 // matrix.  Byte p = 16*h + 4*b + r holds token 8*b + 4*h + r, so the sixteen
 // bytes a lane of half h feeds to the 32x32x32 INT8 MFMA are the sixteen keys

@@ -1,5 +1,6 @@
 // V preparation for gfx950: per-channel range, signed INT8 codes in the packed
-// MFMA order, 128 x per-tile code sums (zero-point term of the signed P·V product) and
+// MFMA order, accumulator seeds (128 x per-tile code sums, the zero-point term of the
+// signed P·V product, plus risa::kAccumulatorSeedBits) and
 // the residual-corrected centre of the midpoint_affine mode.
 //
 // Numerical contract (bit-exact): reference csrc/kernels/quantize_v_impl.cuh:83-292
@@ -171,7 +172,8 @@ __global__ __launch_bounds__(256) void value_codes_kernel(const void* __restrict
 #pragma unroll
       for (int offset = CTA_K / 8; offset > 0; offset >>= 1) sum += __shfl_xor(sum, offset);
       if ((lane & (CTA_K / 4 - 1)) == 0 && p0 < padded) {
-        tile_sum[(static_cast<int64_t>(bh) * tiles + p0 / CTA_K) * dim + octet * 8 + i] = sum * 128;
+        tile_sum[(static_cast<int64_t>(bh) * tiles + p0 / CTA_K) * dim + octet * 8 + i] =
+            sum * 128 + kAccumulatorSeedBits;
       }
     }
   }
@@ -239,7 +241,7 @@ __global__ void value_center_kernel(const float* __restrict__ partial,
   center[row] = midpoint[row] + correction;
 }
 
-// grid (ceil(padded/256), rows_bh), 256 threads: 128 x tile sums of already packed codes.
+// grid (ceil(padded/256), rows_bh), 256 threads: accumulator seeds of already packed codes.
 template <int CTA_K>
 __global__ __launch_bounds__(256) void value_tile_sum_kernel(const int8_t* __restrict__ codes,
                                                              int32_t* __restrict__ tile_sum, int dim,
@@ -259,7 +261,7 @@ __global__ __launch_bounds__(256) void value_tile_sum_kernel(const int8_t* __res
 #pragma unroll
     for (int offset = CTA_K / 8; offset > 0; offset >>= 1) sum += __shfl_xor(sum, offset);
     if ((lane & (CTA_K / 4 - 1)) == 0 && p0 < padded) {
-      tile_sum[(static_cast<int64_t>(bh) * tiles + p0 / CTA_K) * dim + c] = sum * 128;
+      tile_sum[(static_cast<int64_t>(bh) * tiles + p0 / CTA_K) * dim + c] = sum * 128 + kAccumulatorSeedBits;
     }
   }
 }

@@ -2,8 +2,9 @@
 
 Field names, order and defaults follow reference src/risa_attention/_types.py:13-79
 so that code written against the reference keeps working; ``v_tile_sum`` is the
-one addition (appended with a default) and carries 128 x the per-tile sums of
-the V codes, the zero-point term the signed-INT8 matrix cores need.
+one addition (appended with a default) and carries the accumulator seeds of the
+P·V product: 128 x the per-tile sums of the V codes (the zero-point term the
+signed-INT8 matrix cores need) + 0x4B400000.
 """
 
 from __future__ import annotations
