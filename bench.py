@@ -61,6 +61,175 @@ def accuracy(torch, actual, reference):
     return {"nrmse": nrmse, "sqnr_db": -20.0 * __import__("math").log10(max(nrmse, 1e-30))}
 
 
+def time_calls(torch, fn, calls, warmup=2):
+    """Median-free mean of ``calls`` back-to-back calls, HIP events on the current stream."""
+    stream = torch.cuda.current_stream()
+    for _ in range(warmup):
+        fn()
+    begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    begin.record(stream)
+    for _ in range(calls):
+        fn()
+    end.record(stream)
+    end.synchronize()
+    return begin.elapsed_time(end) / calls
+
+
+def sqnr_db(torch, actual, reference):
+    noise = (actual.float() - reference.float()).pow(2).mean().item()
+    signal = reference.float().pow(2).mean().item()
+    return 10.0 * __import__("math").log10(max(signal, 1e-30) / max(noise, 1e-30))
+
+
+def workload_sweep(torch, risa, args, device):
+    """Dense sweep over N, three seeds, both V modes; latency includes Q/K/V preparation."""
+    rows = []
+    for length in ([args.length] if args.length else (512, 1024, 2048, 4096, 8192, 16384, 32768)):
+        ops = dense_equivalent_ops(SHAPE["batch"], SHAPE["q_heads"], length, length, SHAPE["head_dim"])
+        for mode in ("absmax", "midpoint_affine"):
+            samples, errors = [], []
+            for seed in (0, 1, 2):
+                q, k, v = make_inputs(torch, length, seed, device)
+                calls = max(3, min(50, int(2e10 / ops * 20)))
+                samples.append(time_calls(torch, lambda: risa.int8_attention(q, k, v, v_quantization=mode), calls))
+                out = risa.int8_attention(q, k, v, v_quantization=mode)
+                errors.append(accuracy(torch, out, fp32_reference(torch, q, k, v))["nrmse"])
+            ms = statistics.median(samples)
+            rows.append({"N": length, "v_quantization": mode, "ms": round(ms, 4),
+                         "tops": round(ops / (ms * 1e-3) / 1e12, 1), "nrmse": round(statistics.median(errors), 5)})
+    return rows
+
+
+def outlier_inputs(torch, shape_q, shape_k, seed, device):
+    generator = torch.Generator(device=device).manual_seed(seed)
+    q = torch.randn(shape_q, generator=generator, device=device)
+    k = torch.randn(shape_k, generator=generator, device=device)
+    v = torch.randn(shape_k, generator=generator, device=device)
+    channels = shape_q[-1]
+    hot = torch.randperm(channels, generator=generator, device=device)[: max(1, channels // 100)]
+    for tensor in (q, k, v):
+        tensor[..., hot] *= 20.0
+    return q.bfloat16(), k.bfloat16(), v.bfloat16()
+
+
+def workload_masked(torch, risa, args, device):
+    """Unequal lengths, outlier channels; causal, key-padding mask, additive bias, LSE."""
+    rows = []
+    batch, heads, q_len, k_len = 2, 24, 4096, 4608
+    for dim in (64, 128):
+        q, k, v = outlier_inputs(torch, (batch, heads, q_len, dim), (batch, heads, k_len, dim), 0, device)
+        ops = dense_equivalent_ops(batch, heads, q_len, k_len, dim)
+        key_padding = torch.ones(batch, 1, 1, k_len, dtype=torch.bool, device=device)
+        key_padding[1, ..., int(k_len * 0.9):] = False
+        generator = torch.Generator(device=device).manual_seed(1)
+        bias = torch.randn(batch, 1, q_len, k_len, generator=generator, device=device).bfloat16()
+        rowmask = torch.ones(batch, 1, q_len, k_len, dtype=torch.bool, device=device)
+        rowmask[0, :, :7] = False  # fully masked rows
+        variants = {
+            "plain": dict(),
+            "causal": dict(is_causal=True),
+            "key_padding": dict(attn_mask=key_padding),
+            "additive_bias": dict(attn_mask=bias),
+            "bool_mask_lse": dict(attn_mask=rowmask, return_lse=True),
+        }
+        for name, kwargs in variants.items():
+            ms = time_calls(torch, lambda: risa.int8_attention(q, k, v, **kwargs), 10)
+            rows.append({"D": dim, "variant": name, "ms": round(ms, 4),
+                         "tops": round(ops / (ms * 1e-3) / 1e12 * (0.5 if name == "causal" else 1.0), 1)})
+    return rows
+
+
+def clustered_inputs(torch, length, groups, seed, device):
+    generator = torch.Generator(device=device).manual_seed(seed)
+    dim = SHAPE["head_dim"]
+    per_group = length // groups
+
+    def clustered(heads):
+        centroids = torch.randn(1, heads, groups, dim, generator=generator, device=device) * 3.0
+        tokens = centroids.repeat_interleave(per_group, 2)
+        return tokens + torch.randn(tokens.shape, generator=generator, device=device)
+
+    q = clustered(SHAPE["q_heads"])
+    k = clustered(SHAPE["kv_heads"])
+    v = torch.randn(1, SHAPE["kv_heads"], length, dim, generator=generator, device=device)
+    return q, k, v, generator
+
+
+def workload_sparse(torch, risa, args, device):
+    """Construct at theta=0.99 on block-structured Q/K, then five drifting reuse calls."""
+    rows = []
+    for length in ([args.length] if args.length else (4096, 8192, 16384, 32768)):
+        q32, k32, v32, generator = clustered_inputs(torch, length, 64, 0, device)
+        q, k, v = q32.bfloat16(), k32.bfloat16(), v32.bfloat16()
+        construct_ms = time_calls(torch, lambda: risa.construct_sparse_int8_attention(q, k, v, theta=0.99), 3, 1)
+        _, pattern = risa.construct_sparse_int8_attention(q, k, v, theta=0.99)
+        dense_samples, sparse_samples, quality = [], [], []
+        for _ in range(5):
+            q32 = q32 + 0.05 * torch.randn(q32.shape, generator=generator, device=device)
+            k32 = k32 + 0.05 * torch.randn(k32.shape, generator=generator, device=device)
+            v32 = v32 + 0.05 * torch.randn(v32.shape, generator=generator, device=device)
+            q, k, v = q32.bfloat16(), k32.bfloat16(), v32.bfloat16()
+            dense_samples.append(time_calls(torch, lambda: risa.int8_attention(q, k, v), 5, 1))
+            sparse_samples.append(time_calls(torch, lambda: risa.sparse_int8_attention(q, k, v, pattern), 5, 1))
+            sparse_out = risa.sparse_int8_attention(q, k, v, pattern)
+            quality.append(sqnr_db(torch, sparse_out, fp32_reference(torch, q, k, v)))
+        dense_ms, sparse_ms = statistics.median(dense_samples), statistics.median(sparse_samples)
+        rows.append({"N": length, "construct_ms": round(construct_ms, 4), "dense_ms": round(dense_ms, 4),
+                     "sparse_ms": round(sparse_ms, 4), "speedup": round(dense_ms / sparse_ms, 3),
+                     "coverage": round(pattern.coverage, 4), "measured_mass": round(pattern.measured_retained_mass, 5),
+                     "sqnr_db_vs_fp32": round(min(quality), 2)})
+    # Half coverage: on unstructured N(0,1) inputs every tile carries about the same
+    # mass, so theta = 0.5 keeps about half of the tiles of every query block.
+    length = args.length or 32768
+    q, k, v = make_inputs(torch, length, 0, device)
+    _, pattern = risa.construct_sparse_int8_attention(q, k, v, theta=0.5)
+    dense_ms = time_calls(torch, lambda: risa.int8_attention(q, k, v), 10, 2)
+    sparse_ms = time_calls(torch, lambda: risa.sparse_int8_attention(q, k, v, pattern), 10, 2)
+    rows.append({"N": length, "inputs": "unstructured N(0,1), theta=0.5", "dense_ms": round(dense_ms, 4),
+                 "sparse_ms": round(sparse_ms, 4), "speedup": round(dense_ms / sparse_ms, 3),
+                 "coverage": round(pattern.coverage, 4)})
+    return rows
+
+
+def workload_video(torch, risa, args, device):
+    """Video-DiT-scale sampling loop: one construction, nine drifting reuses, packed-operand replay."""
+    frames, per_frame, heads, dim = 21, 1560, 40, 128
+    length = frames * per_frame
+    generator = torch.Generator(device=device).manual_seed(0)
+    position = torch.arange(length, device=device, dtype=torch.float32)
+    frame, patch = (position // per_frame) / frames, (position % per_frame) / per_frame
+    frequency = torch.arange(1, dim // 4 + 1, device=device, dtype=torch.float32)
+    phase = torch.rand(heads, 1, dim // 4, generator=generator, device=device) * 6.2831853
+    parts = []
+    for coordinate in (frame, patch):
+        angle = coordinate[None, :, None] * frequency[None, None, :] * 6.2831853 + phase
+        parts += [torch.sin(angle), torch.cos(angle)]
+    smooth = torch.cat(parts, dim=-1)[None] * 2.0  # [1, H, N, D]
+    q32 = smooth + 0.5 * torch.randn(smooth.shape, generator=generator, device=device)
+    k32 = smooth + 0.5 * torch.randn(smooth.shape, generator=generator, device=device)
+    v32 = torch.randn(smooth.shape, generator=generator, device=device)
+    del smooth
+    q, k, v = q32.bfloat16(), k32.bfloat16(), v32.bfloat16()
+    dense_ms = time_calls(torch, lambda: risa.int8_attention(q, k, v), 3, 1)
+    construct_ms = time_calls(torch, lambda: risa.construct_sparse_int8_attention(q, k, v, theta=0.99), 2, 1)
+    _, pattern = risa.construct_sparse_int8_attention(q, k, v, theta=0.99)
+    reuse = []
+    for _ in range(9):
+        q32 += 0.03 * torch.randn(q32.shape, generator=generator, device=device)
+        k32 += 0.03 * torch.randn(k32.shape, generator=generator, device=device)
+        q, k = q32.bfloat16(), k32.bfloat16()
+        reuse.append(time_calls(torch, lambda: risa.sparse_int8_attention(q, k, v, pattern), 2, 1))
+    packed = risa.prequantize_int8_attention(q, k, v)
+    prequantize_ms = time_calls(torch, lambda: risa.prequantize_int8_attention(q, k, v), 5, 1)
+    replay_ms = time_calls(torch, lambda: risa.int8_attention_from_prequantized(packed), 3, 1)
+    ops = dense_equivalent_ops(1, heads, length, length, dim)
+    return {"N": length, "heads": heads, "dense_ms": round(dense_ms, 3), "dense_tops": round(ops / dense_ms / 1e9, 1),
+            "construct_ms": round(construct_ms, 3), "reuse_ms_median": round(statistics.median(reuse), 3),
+            "coverage": round(pattern.coverage, 4), "prequantize_ms": round(prequantize_ms, 3),
+            "from_prequantized_ms": round(replay_ms, 3),
+            "loop_speedup_vs_dense": round(10 * dense_ms / (construct_ms + sum(reuse)), 3)}
+
+
 def cpu_baseline(length=1024, calls=3):
     """Oracle (numpy port of the quantised pipeline) on the host cores, N=1024."""
     import numpy as np
@@ -99,10 +268,14 @@ def main():
     parser.add_argument("--gpus", type=int, default=1)
     parser.add_argument("--steps", type=int, default=20)
     parser.add_argument("--warmup", type=int, default=5)
-    parser.add_argument("--length", type=int, default=32768)
+    parser.add_argument("--length", type=int, default=None,
+                        help="sequence length (default 32768 for dense; restricts sweep/sparse to one N)")
     parser.add_argument("--mode", default="absmax", choices=["absmax", "midpoint_affine"])
     parser.add_argument("--no-cpu-baseline", action="store_true")
     parser.add_argument("--no-accuracy", action="store_true")
+    parser.add_argument("--workload", default="dense", choices=["dense", "sweep", "masked", "sparse", "video"],
+                        help="dense = headline N=32K line (default); the others are the remaining BASELINE.json "
+                             "configurations, reported as one JSON line each")
     parser.add_argument("--calibrate-copy", action="store_true",
                         help="only run a 1 GiB device copy (reference point for rocprofv3 FETCH_SIZE/WRITE_SIZE)")
     args = parser.parse_args()
@@ -128,7 +301,18 @@ def main():
         torch.cuda.synchronize()
         print(json.dumps({"calibration": "copy", "bytes_read": 1 << 30, "bytes_written": 1 << 30}))
         return
-    length = args.length
+    if args.workload != "dense":
+        runner = {"sweep": workload_sweep, "masked": workload_masked, "sparse": workload_sparse,
+                  "video": workload_video}[args.workload]
+        wall = time.perf_counter()
+        rows = runner(torch, risa, args, device)
+        print(json.dumps({"metric": f"{args.workload} workload (see config.rows)", "value": None, "unit": "ms",
+                          "n_gpus": 1, "steps": None, "warmup": None, "ms_per_step": None,
+                          "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "int8",
+                          "data": "synthetic", "wall_seconds": round(time.perf_counter() - wall, 1),
+                          "config": {"workload": args.workload, "rows": rows}}))
+        return
+    length = args.length or 32768
     q, k, v = make_inputs(torch, length, 0, device)
     ops = dense_equivalent_ops(SHAPE["batch"], SHAPE["q_heads"], length, length, SHAPE["head_dim"])
 

@@ -98,10 +98,12 @@ void risa_unpack_order(int32_t* order);
  *   query stride 0 selecting the key-only path; sparse_row_offsets int32
  *   [B*Hq*ceil(Lq/128)+1] and sparse_block_indices int32 (both or neither);
  *   block_mass (nullable) float32 workspace laid out as mass
- *   [B*Hq*ceil(Lq/128), tiles] ++ per-row full-tile stats [rows, tiles-1, 2]
- *   (u32 sum of U8 probabilities, f32 tile maximum) ++ last-tile stats
- *   [rows, 2] (f32, f32) ++ state [rows, 2] (m, d), rows = B*Hq*Lq
- *   (reference attention_int8.cuh:51-143, 871-898); lse (nullable) float32
+ *   [B*Hq*ceil(Lq/128), tiles] ++ full-tile stats [B*Hq, tiles-1, Lq, 2]
+ *   (u32 sum of U8 probabilities, f32 tile maximum; tile-major so that the
+ *   stores of neighbouring queries coalesce) ++ last-tile stats [rows, 2]
+ *   (f32, f32) ++ state [rows, 2] (m, d), rows = B*Hq*Lq (same contents and
+ *   total size as reference attention_int8.cuh:51-143, 871-898, whose full-tile
+ *   stats are row-major); lse (nullable) float32
  *   [B,Hq,Lq]; key_mask_tiles (nullable) int32 [B,Hq,tiles+1] from
  *   risa_prepare_key_mask_tiles.
  */

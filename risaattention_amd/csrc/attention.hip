@@ -16,49 +16,63 @@ template <> int launch_attention_variant<256>(const KernelParams&, int, bool, bo
 
 namespace {
 
-// One workgroup per 128-query block; thread r owns query row r and walks the
-// key tiles.  mass[block, tile] = sum_r numerator * 2^(tile_max - m) / d,
-// reduced by a shuffle-down tree per 32 rows and a second tree over the four
-// partial sums (reference attention_int8.cuh:1028-1088).
-__global__ __launch_bounds__(128) void block_mass_kernel(float* __restrict__ workspace, int q_len,
+// mass[block, tile] = sum_r numerator * 2^(tile_max - m) / d over the 128 query
+// rows r of the block, added in the order of the reference (attention_int8.cuh:
+// 1028-1088): a shuffle-down tree per 32 rows (offsets 16, 8, 4, 2, 1), then
+// (p0 + p2) + (p1 + p3) over the four partial sums.
+//
+// One workgroup per query block, one wavefront per key tile (strided).  Lane l
+// owns rows 2l and 2l+1, so a tile's statistics of the whole block are one
+// coalesced 1 KB load (the attention kernel stores them tile-major).  In the
+// tree, rows 16, 8, 4, 2 apart are lanes 8, 4, 2, 1 apart within a 16-lane
+// group and the last level adds a lane's own two rows.
+__global__ __launch_bounds__(256) void block_mass_kernel(float* __restrict__ workspace, int q_len,
                                                          int n_kb, int n_qb, int q_heads, int batch) {
-  __shared__ float partial[4];
   const int q_block = blockIdx.x, head = blockIdx.y, b = blockIdx.z;
-  const int tid = threadIdx.x;
-  const int query = q_block * kQueryBlock + tid;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int query = q_block * kQueryBlock + 2 * lane;
+  const uint64_t bhq = static_cast<uint64_t>(b) * q_heads + head;
   const uint64_t query_rows = static_cast<uint64_t>(batch) * q_heads * q_len;
   const uint64_t mass_elements = static_cast<uint64_t>(batch) * q_heads * n_qb * n_kb;
   const uint64_t full_words = query_rows * (n_kb - 1) * 2;
   const uint32_t* stats = reinterpret_cast<const uint32_t*>(workspace + mass_elements);
   const float* state = reinterpret_cast<const float*>(stats + full_words + query_rows * 2);
-  const uint64_t row = (static_cast<uint64_t>(b) * q_heads + head) * q_len + query;
-  const bool active = query < q_len;
-  const float m = active ? state[row * 2] : 0.0f;
-  const float d = active ? state[row * 2 + 1] : 0.0f;
-  const uint64_t mass_row = (static_cast<uint64_t>(b) * q_heads + head) * n_qb + q_block;
-  for (int tile = 0; tile < n_kb; ++tile) {
-    float value = 0.0f;
-    if (active && d > 0.0f) {
-      float numerator, tile_max;
-      if (tile + 1 < n_kb) {
-        const uint64_t offset = (row * (n_kb - 1) + tile) * 2;
-        numerator = static_cast<float>(stats[offset]);
-        tile_max = __uint_as_float(stats[offset + 1]);
-      } else {
-        const uint64_t offset = full_words + row * 2;
-        numerator = __uint_as_float(stats[offset]);
-        tile_max = __uint_as_float(stats[offset + 1]);
+  const uint64_t row = bhq * q_len + query;
+  // q_len may be odd: the second row of the last lane can be out of range.
+  const bool active0 = query < q_len, active1 = query + 1 < q_len;
+  float m[2] = {0.0f, 0.0f}, d[2] = {0.0f, 0.0f};
+  if (active0) {
+    m[0] = state[row * 2];
+    d[0] = state[row * 2 + 1];
+  }
+  if (active1) {
+    m[1] = state[row * 2 + 2];
+    d[1] = state[row * 2 + 3];
+  }
+  const uint64_t mass_row = bhq * n_qb + q_block;
+  for (int tile = wave; tile < n_kb; tile += 4) {
+    const bool last = tile + 1 == n_kb;
+    const uint64_t offset =
+        last ? full_words + row * 2 : ((bhq * (n_kb - 1) + tile) * static_cast<uint64_t>(q_len) + query) * 2;
+    float value[2] = {0.0f, 0.0f};
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      if ((j == 0 ? active0 : active1) && d[j] > 0.0f) {
+        const uint32_t raw = stats[offset + 2 * j];
+        const float numerator = last ? __uint_as_float(raw) : static_cast<float>(raw);
+        const float tile_max = __uint_as_float(stats[offset + 2 * j + 1]);
+        value[j] = numerator * __builtin_amdgcn_exp2f(tile_max - m[j]) / d[j];
       }
-      value = numerator * __builtin_amdgcn_exp2f(tile_max - m) / d;
     }
 #pragma unroll
-    for (int offset = 16; offset > 0; offset >>= 1) value += __shfl_down(value, offset, 32);
-    if ((tid & 31) == 0) partial[tid >> 5] = value;
-    __syncthreads();
-    if (tid == 0) {
-      workspace[mass_row * n_kb + tile] = (partial[0] + partial[2]) + (partial[1] + partial[3]);
+    for (int step = 8; step > 0; step >>= 1) {
+      value[0] += __shfl_down(value[0], step, 16);
+      value[1] += __shfl_down(value[1], step, 16);
     }
-    __syncthreads();
+    const float group = value[0] + value[1];              // lanes 0, 16, 32, 48: p0..p3
+    const float pair = group + __shfl_down(group, 32);    // lane 0: p0 + p2, lane 16: p1 + p3
+    const float total = pair + __shfl_down(pair, 16);
+    if (lane == 0) workspace[mass_row * n_kb + tile] = total;
   }
 }
 
@@ -137,7 +151,7 @@ int launch_attention(const AttentionArgs& a, hipStream_t stream) {
   if (status != 0) return status;
   if (capture) {
     const dim3 grid(p.n_qb, a.q_heads, a.batch);
-    block_mass_kernel<<<grid, 128, 0, stream>>>(a.block_mass, a.q_len, p.n_kb, p.n_qb, a.q_heads,
+    block_mass_kernel<<<grid, 256, 0, stream>>>(a.block_mass, a.q_len, p.n_kb, p.n_qb, a.q_heads,
                                                 a.batch);
   }
   return check_launch("risa_attention");

@@ -437,7 +437,8 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void attention_kernel(cons
       const uint32_t numerator = row_sum + __shfl_xor(row_sum, 32);
       if (half == 0 && query_ok) {
         if constexpr (!LAST) {
-          const uint64_t offset = (stat_row * (p.n_kb - 1) + it) * 2;
+          // Tile-major: the 32 queries of a half-wave store 256 contiguous bytes.
+          const uint64_t offset = ((bhq * (p.n_kb - 1) + it) * static_cast<uint64_t>(p.q_len) + query) * 2;
           stats[offset] = numerator;
           stats[offset + 1] = __float_as_uint(tile_m);
         } else {

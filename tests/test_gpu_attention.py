@@ -142,7 +142,7 @@ def test_capture_tile_max_known_answer(risa, mode, dim, length):
     assert torch.equal(plain.view(torch.int16), captured.view(torch.int16))
     if blocks > 1:
         full_stats = workspace[mass_elements : mass_elements + rows * (blocks - 1) * 2]
-        maxima = full_stats.reshape(rows, blocks - 1, 2)[..., 1]
+        maxima = full_stats.reshape(batch * heads, blocks - 1, queries, 2)[..., 1].transpose(1, 2).reshape(rows, blocks - 1)
         scale = torch.tensor(1.44269504088896340736, device="cuda", dtype=torch.float32) / 128
         offset = torch.tensor(7.9943534, device="cuda", dtype=torch.float32)
         expected = (levels[:-1].double() * dim * scale.double() - offset.double()).float()
