@@ -109,6 +109,15 @@ int launch_attention(const AttentionArgs& a, hipStream_t stream) {
   p.mask_stride_q = a.mask_stride_q;
   p.mask_stride_k = a.mask_stride_k;
   p.mask_dtype = a.mask != nullptr ? a.mask_dtype : -1;
+  if (a.mask != nullptr) {
+    // Groups of four keys start at multiples of four, so one load per group needs
+    // unit key stride, the other strides multiples of four elements and the base
+    // aligned to four elements.
+    const int64_t element = a.mask_dtype == kF32 ? 4 : a.mask_dtype == kBool ? 1 : 2;
+    const bool aligned = reinterpret_cast<uintptr_t>(a.mask) % (4 * element) == 0 &&
+                         ((a.mask_stride_b | a.mask_stride_h | a.mask_stride_q) & 3) == 0;
+    p.mask_vector = a.mask_stride_k == 1 && aligned ? 1 : 0;
+  }
   p.q_len = a.q_len;
   p.k_len = a.k_len;
   p.q_heads = a.q_heads;

@@ -9,10 +9,10 @@ namespace risa {
 template <int D> int launch_attention_variant(const KernelParams& p, int cta_k, bool fast,
                                               bool indexed, bool capture, hipStream_t stream);
 
-template <int D, int CTA_K, bool FAST, bool INDEXED, bool CAPTURE>
+template <int D, int CTA_K, bool FAST, bool INDEXED, bool CAPTURE, int MASK_DT>
 int launch_one(const KernelParams& p, hipStream_t stream) {
   using Shape = TileShape<D, CTA_K>;
-  auto kernel = attention_kernel<D, CTA_K, FAST, INDEXED, CAPTURE>;
+  auto kernel = attention_kernel<D, CTA_K, FAST, INDEXED, CAPTURE, MASK_DT>;
   // The dynamic LDS limit is a per-device property of the function; setting it
   // again is cheap and keeps the launcher free of host-side caches.
   static thread_local int configured_device = -1;
@@ -32,16 +32,27 @@ int launch_one(const KernelParams& p, hipStream_t stream) {
   return 0;
 }
 
+template <int D, int CTA_K, int MASK_DT>
+int launch_general(const KernelParams& p, bool indexed, bool capture, hipStream_t stream) {
+  if (capture) return launch_one<D, CTA_K, false, false, true, MASK_DT>(p, stream);
+  if (indexed) return launch_one<D, CTA_K, false, true, false, MASK_DT>(p, stream);
+  return launch_one<D, CTA_K, false, false, false, MASK_DT>(p, stream);
+}
+
 template <int D, int CTA_K>
 int launch_tile(const KernelParams& p, bool fast, bool indexed, bool capture, hipStream_t stream) {
   if (fast) {
-    if (capture) return launch_one<D, CTA_K, true, false, true>(p, stream);
-    if (indexed) return launch_one<D, CTA_K, true, true, false>(p, stream);
-    return launch_one<D, CTA_K, true, false, false>(p, stream);
+    if (capture) return launch_one<D, CTA_K, true, false, true, -1>(p, stream);
+    if (indexed) return launch_one<D, CTA_K, true, true, false, -1>(p, stream);
+    return launch_one<D, CTA_K, true, false, false, -1>(p, stream);
   }
-  if (capture) return launch_one<D, CTA_K, false, false, true>(p, stream);
-  if (indexed) return launch_one<D, CTA_K, false, true, false>(p, stream);
-  return launch_one<D, CTA_K, false, false, false>(p, stream);
+  switch (p.mask_dtype) {
+    case kBool: return launch_general<D, CTA_K, kBool>(p, indexed, capture, stream);
+    case kF32: return launch_general<D, CTA_K, kF32>(p, indexed, capture, stream);
+    case kF16: return launch_general<D, CTA_K, kF16>(p, indexed, capture, stream);
+    case kBF16: return launch_general<D, CTA_K, kBF16>(p, indexed, capture, stream);
+    default: return launch_general<D, CTA_K, -1>(p, indexed, capture, stream);
+  }
 }
 
 #define RISA_DEFINE_ATTENTION_VARIANT(DIM)                                                        \

@@ -58,6 +58,7 @@ struct KernelParams {
   const void* mask;
   int64_t mask_stride_b, mask_stride_h, mask_stride_q, mask_stride_k;
   int mask_dtype;  // -1: no mask
+  int mask_vector;  // keys are contiguous and groups of four keys aligned: one load per group
   int q_len, k_len, q_heads, kv_heads, padded, n_kb, n_qb, batch;
   int64_t out_stride_b, out_stride_n, out_stride_h;
   float sm2;  // sm_scale * log2(e)
@@ -105,6 +106,15 @@ __device__ __forceinline__ void copy16_to_lds_uniform(const int8_t* uniform_base
   copy16_to_lds(uniform_base + static_cast<uint64_t>(lane_offset), lds_wave_base);
 }
 
+// Lane index computed where it is used (two instructions).  The masked kernels
+// use it inside the tile loop instead of values derived from threadIdx before
+// the loop, which the register allocator would otherwise spill.
+__device__ __forceinline__ int fresh_lane() {
+  int lane_id;
+  asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(lane_id));
+  return lane_id;
+}
+
 template <int D, int CTA_K> struct TileShape {
   static constexpr int kTileBytes = CTA_K * D;
   static constexpr int kCopiesPerWave = kTileBytes / 16 / 256;  // 1 KB copy instructions per wave
@@ -112,8 +122,11 @@ template <int D, int CTA_K> struct TileShape {
   static constexpr int kLdsBytes = 2 * kStageBytes;
 };
 
-template <int D, int CTA_K, bool FAST, bool INDEXED, bool CAPTURE>
+// MASK_DT: element type of the mask tensor (risa::kBool, kF32, kF16, kBF16) or -1
+// for none; FAST (raw-score path) implies -1.
+template <int D, int CTA_K, bool FAST, bool INDEXED, bool CAPTURE, int MASK_DT>
 __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void attention_kernel(const KernelParams p) {
+  static_assert(!FAST || MASK_DT < 0, "the raw-score path takes no mask");
   using Shape = TileShape<D, CTA_K>;
   constexpr int RB = CTA_K / 32;  // 32-key blocks per tile
   constexpr int CB = D / 32;      // 32-channel blocks
@@ -126,11 +139,24 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void attention_kernel(cons
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int l32 = lane & 31, half = lane >> 5;
 
-  int block = blockIdx.x;
-  const int bx = block % p.n_qb;
-  block /= p.n_qb;
-  const int head = block % p.q_heads;
-  const int batch = block / p.q_heads;
+  // Workgroup order.  Without a causal mask the query blocks of one head are
+  // neighbours, so co-resident workgroups walk the same K/V tiles and share them
+  // in L2.  Under a causal mask the work per query block differs by up to the
+  // number of key tiles: the launch then goes through all heads of the last query
+  // block first and the first query block last (longest first keeps the tail short).
+  int bx, head, batch;
+  if (!FAST && p.causal) {
+    const int heads = p.q_heads * p.batch;
+    const int rest = blockIdx.x % heads;
+    bx = p.n_qb - 1 - blockIdx.x / heads;
+    head = rest % p.q_heads;
+    batch = rest / p.q_heads;
+  } else {
+    bx = blockIdx.x % p.n_qb;
+    const int rest = blockIdx.x / p.n_qb;
+    head = rest % p.q_heads;
+    batch = rest / p.q_heads;
+  }
   const int kv_head = head / (p.q_heads / p.kv_heads);
   const int64_t bhk = static_cast<int64_t>(batch) * p.kv_heads + kv_head;
   const int64_t bhq = static_cast<int64_t>(batch) * p.q_heads + head;
@@ -169,25 +195,34 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void attention_kernel(cons
     return it;
   };
 
-  // --- per-lane copy descriptors (constant over tiles) -----------------------
+  // --- per-lane copy descriptors -------------------------------------------------
   // Copy instruction i of this wave fills LDS bytes [(wave*NC+i)*1024, +1024) of
-  // a tile; this lane supplies chunk `lane` of that kilobyte.
-  uint32_t k_src_offset[NC];  // byte offset of the source chunk inside a K tile
-  uint32_t v_src_offset[NC];  // byte offset of the source chunk inside the head's V slab, tile 0
+  // a tile; this lane supplies chunk `lane` of that kilobyte.  The source offsets
+  // are constant over tiles.  The raw-score kernels keep them in registers; the
+  // masked kernels have none to spare (a spilled offset would be reloaded through
+  // the same counter the LDS copies complete on, serialising them) and recompute
+  // them per tile from a lane id the compiler cannot see through.
+  constexpr bool KEEP_OFFSETS = FAST;
+  auto k_source_offset = [&](int i, int lane_id) -> uint32_t {
+    constexpr int CH = D / 16;
+    const int slot = (wave * NC + i) * 64 + lane_id;
+    const int row = slot / CH, phys = slot % CH;
+    const int chunk = phys ^ ((row / (256 / D)) & (CH - 1));
+    return row * D + chunk * 16;
+  };
+  auto v_source_offset = [&](int i, int lane_id) -> uint32_t {
+    constexpr int CH = CTA_K / 16;
+    const int slot = (wave * NC + i) * 64 + lane_id;
+    const int row = slot / CH, phys = slot % CH;
+    const int chunk = phys ^ ((row / (256 / CTA_K)) & (CH - 1));
+    return static_cast<uint32_t>(row) * static_cast<uint32_t>(p.padded) + chunk * 16;
+  };
+  [[maybe_unused]] uint32_t k_kept[NC], v_kept[NC];
+  if constexpr (KEEP_OFFSETS) {
 #pragma unroll
-  for (int i = 0; i < NC; ++i) {
-    const int slot = (wave * NC + i) * 64 + lane;
-    {
-      constexpr int CH = D / 16;
-      const int row = slot / CH, phys = slot % CH;
-      const int chunk = phys ^ ((row / (256 / D)) & (CH - 1));
-      k_src_offset[i] = row * D + chunk * 16;
-    }
-    {
-      constexpr int CH = CTA_K / 16;
-      const int row = slot / CH, phys = slot % CH;
-      const int chunk = phys ^ ((row / (256 / CTA_K)) & (CH - 1));
-      v_src_offset[i] = static_cast<uint32_t>(row) * static_cast<uint32_t>(p.padded) + chunk * 16;
+    for (int i = 0; i < NC; ++i) {
+      k_kept[i] = k_source_offset(i, lane);
+      v_kept[i] = v_source_offset(i, lane);
     }
   }
   auto issue_tile = [&](int tile, int stage) {
@@ -196,6 +231,18 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void attention_kernel(cons
     unsigned char* sl = lds + stage * Shape::kStageBytes + 2 * Shape::kTileBytes;
     const int8_t* k_tile = k_base + static_cast<int64_t>(tile) * CTA_K * D;
     const int8_t* v_tile = v_base + static_cast<int64_t>(tile) * CTA_K;
+    uint32_t k_src_offset[NC], v_src_offset[NC];
+    if constexpr (KEEP_OFFSETS) {
+#pragma unroll
+      for (int i = 0; i < NC; ++i) k_src_offset[i] = k_kept[i], v_src_offset[i] = v_kept[i];
+    } else {
+      const int lane_id = fresh_lane();
+#pragma unroll
+      for (int i = 0; i < NC; ++i) {
+        k_src_offset[i] = k_source_offset(i, lane_id);
+        v_src_offset[i] = v_source_offset(i, lane_id);
+      }
+    }
     const int keys_left = p.k_len - tile * CTA_K;
     if (keys_left >= CTA_K) {
 #pragma unroll
@@ -206,14 +253,17 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void attention_kernel(cons
       const uint32_t bytes_left = static_cast<uint32_t>(keys_left) * D;
 #pragma unroll
       for (int i = 0; i < NC; ++i) {
-        if (k_src_offset[i] < bytes_left)
-          copy16_to_lds(k_tile + k_src_offset[i], k_slot + i * 1024);
+        if (k_src_offset[i] < bytes_left) copy16_to_lds_uniform(k_tile, k_src_offset[i], k_slot + i * 1024);
       }
     }
 #pragma unroll
     for (int i = 0; i < NC; ++i) copy16_to_lds_uniform(v_tile, v_src_offset[i], v_slot + i * 1024);
-    if (wave == 0 && lane < D / 4) {
-      copy16_to_lds(sum_base + static_cast<int64_t>(tile) * D + lane * 4, sl);
+    if (wave == 0) {
+      const int lane_id = KEEP_OFFSETS ? lane : fresh_lane();
+      if (lane_id < D / 4) {
+        copy16_to_lds_uniform(reinterpret_cast<const int8_t*>(sum_base + static_cast<int64_t>(tile) * D),
+                              static_cast<uint32_t>(lane_id) * 16, sl);
+      }
     }
   };
 
@@ -256,7 +306,7 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void attention_kernel(cons
   }
 
   const int64_t mask_row =
-      (!FAST && p.mask_dtype >= 0)
+      (MASK_DT >= 0)
           ? static_cast<int64_t>(batch) * p.mask_stride_b + static_cast<int64_t>(head) * p.mask_stride_h +
                 static_cast<int64_t>(query) * p.mask_stride_q
           : 0;
@@ -372,36 +422,112 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void attention_kernel(cons
           pk[rb][b4] = static_cast<int>(packed ^ 0x80808080u);
         }
     } else {
-      // Pre-scaled scores with masks.
+      // Pre-scaled scores with masks.  Whether a tile needs any masking at all is
+      // uniform over the wavefront: tiles below the causal diagonal, inside the key
+      // range and without a mask tensor take the short loop.
       const float neg_inf = -__builtin_inff();
+      constexpr bool has_mask = MASK_DT >= 0;
+      const int first_query = bx * kQueryBlock + wave * 32;
+      const bool on_diagonal = p.causal && tile * CTA_K + CTA_K - 1 > first_query;
+      const bool partial = LAST && (tile + 1) * CTA_K > p.k_len;
       float mx = kRowFloor;
+      if (!has_mask && !on_diagonal && !partial) {
 #pragma unroll
-      for (int rb = 0; rb < RB; ++rb)
+        for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          const int key = key0 + rb * 32 + (i >> 2) * 8 + (i & 3);
-          float value = static_cast<float>(s[rb][i]) * ((i & 2) ? sc1 : sc0);
-          if (p.mask_dtype >= 0) {
-            bool keep = query_ok && key < p.k_len;
-            float bias = 0.0f;
-            if (keep) {
-              const int64_t offset = mask_row + static_cast<int64_t>(key) * p.mask_stride_k;
-              if (p.mask_dtype == kBool) {
-                keep = static_cast<const uint8_t*>(p.mask)[offset] != 0;
-              } else {
-                bias = p.mask_dtype == kF32   ? load1<kF32>(p.mask, offset)
-                       : p.mask_dtype == kF16 ? load1<kF16>(p.mask, offset)
-                                              : load1<kBF16>(p.mask, offset);
-                keep = __builtin_isfinite(bias);
+          for (int i = 0; i < 16; ++i) {
+            const float value = static_cast<float>(s[rb][i]) * ((i & 2) ? sc1 : sc0);
+            s[rb][i] = __float_as_int(value);
+            mx = __builtin_fmaxf(mx, value);
+          }
+      } else {
+        // DT: mask element type (-1: none, only the causal / key-range tests);
+        // VEC: one load per group of four consecutive keys.
+        auto masked_scores = [&](auto dtype_tag, auto vector_tag) {
+          constexpr int DT = decltype(dtype_tag)::value;
+          constexpr bool VEC = decltype(vector_tag)::value;
+          constexpr int ES = DT == kF32 ? 4 : DT == kBool ? 1 : 2;
+          [[maybe_unused]] const unsigned char* lane_mask = nullptr;
+          if constexpr (DT >= 0) {
+            lane_mask = static_cast<const unsigned char*>(p.mask) +
+                        (mask_row + static_cast<int64_t>(key0) * p.mask_stride_k) * ES;
+          }
+#pragma unroll
+          for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+            for (int b4 = 0; b4 < 4; ++b4) {
+              const int local = rb * 32 + b4 * 8;  // first of four consecutive keys of this lane
+              const int key = key0 + local;
+              bool keep[4] = {true, true, true, true};
+              float bias[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+              if constexpr (DT >= 0) {
+                if (!query_ok) {
+#pragma unroll
+                  for (int r = 0; r < 4; ++r) keep[r] = false;
+                } else if (VEC && key + 3 < p.k_len) {
+                  const unsigned char* at = lane_mask + local * ES;
+                  if constexpr (DT == kBool) {
+                    const uint32_t word = *reinterpret_cast<const uint32_t*>(at);
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) keep[r] = ((word >> (8 * r)) & 0xffu) != 0;
+                  } else if constexpr (DT == kF32) {
+                    const float4 w = *reinterpret_cast<const float4*>(at);
+                    bias[0] = w.x, bias[1] = w.y, bias[2] = w.z, bias[3] = w.w;
+                  } else {
+                    const uint2 w = *reinterpret_cast<const uint2*>(at);
+                    const uint32_t bits16[4] = {w.x & 0xffffu, w.x >> 16, w.y & 0xffffu, w.y >> 16};
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                      bias[r] = DT == kF16 ? static_cast<float>(__builtin_bit_cast(
+                                                 _Float16, static_cast<uint16_t>(bits16[r])))
+                                           : __uint_as_float(bits16[r] << 16);
+                    }
+                  }
+                } else {
+#pragma unroll
+                  for (int r = 0; r < 4; ++r) {
+                    keep[r] = key + r < p.k_len;
+                    if (keep[r]) {
+                      const unsigned char* at = lane_mask + (local + r) * p.mask_stride_k * ES;
+                      if constexpr (DT == kBool) {
+                        keep[r] = *at != 0;
+                      } else {
+                        bias[r] = load1<DT>(at, 0);
+                      }
+                    }
+                  }
+                }
+                if constexpr (DT != kBool) {
+#pragma unroll
+                  for (int r = 0; r < 4; ++r) keep[r] = keep[r] && __builtin_isfinite(bias[r]);
+                }
+              }
+#pragma unroll
+              for (int r = 0; r < 4; ++r) {
+                float value = static_cast<float>(s[rb][b4 * 4 + r]) * ((r & 2) ? sc1 : sc0);
+                if constexpr (DT >= 0) value = keep[r] ? value + bias[r] * kLog2e : neg_inf;
+                if (p.causal && key + r > query) value = neg_inf;
+                if (LAST && key + r >= p.k_len) value = neg_inf;
+                s[rb][b4 * 4 + r] = __float_as_int(value);
+                mx = __builtin_fmaxf(mx, value);
+              }
+              // The mask loads of one key block at a time: all of a tile in flight
+              // at once do not fit the register file.
+              if constexpr (DT >= 0) {
+                if (b4 == 3) {
+                  asm volatile("" ::: "memory");
+                  __builtin_amdgcn_sched_barrier(0);
+                }
               }
             }
-            value = keep ? value + bias * kLog2e : neg_inf;
-          }
-          if (p.causal && key > query) value = neg_inf;
-          if (LAST && key >= p.k_len) value = neg_inf;
-          s[rb][i] = __float_as_int(value);
-          mx = __builtin_fmaxf(mx, value);
+        };
+        using MaskType = std::integral_constant<int, MASK_DT>;
+        if (has_mask && p.mask_vector != 0) {
+          masked_scores(MaskType{}, std::true_type{});
+        } else {
+          masked_scores(MaskType{}, std::false_type{});
         }
+      }
       tile_m = mx - kU8Offset;
       tile_m = __builtin_fmaxf(tile_m, __shfl_xor(tile_m, 32));
 #pragma unroll
@@ -541,8 +667,9 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void attention_kernel(cons
       __syncthreads();
       load_k_fragments(lds + stage * Shape::kStageBytes, 0, k_first);
       issue_tile(next_tile, stage ^ 1);
-      const float next_ks0 = ks_base[next_tile * 4 + 2 * half];
-      const float next_ks1 = ks_base[next_tile * 4 + 2 * half + 1];
+      const int scale_pair = KEEP_OFFSETS ? 2 * half : (fresh_lane() >> 5) * 2;
+      const float next_ks0 = ks_base[next_tile * 4 + scale_pair];
+      const float next_ks1 = ks_base[next_tile * 4 + scale_pair + 1];
       score_tile(stage, k_first, s);
       if constexpr (PREFETCH) {
         load_seed_pair(stage, 0, seed);
@@ -582,7 +709,7 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void attention_kernel(cons
       state[stat_row * 2 + 1] = d_total;
     }
   }
-  const bool guard_empty = !FAST && (p.mask_dtype >= 0 || p.causal);
+  const bool guard_empty = !FAST && (MASK_DT >= 0 || p.causal);
   const bool row_valid = d_total > 0.0f;
   const float inv_d = 1.0f / d_total;
   if (query_ok) {
