@@ -197,3 +197,45 @@ def test_lse_restores_shifted_keys_and_empty_rows(risa):
     assert torch.isneginf(lse[:, :, 0]).all()
     assert out[:, :, 0].count_nonzero().item() == 0
     torch.testing.assert_close(lse[:, :, 1:], expected[:, :, 1:], atol=0.15, rtol=0.02)
+
+
+@pytest.mark.parametrize("mask_dtype", [torch.bool, torch.float16, torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("k_len", [264, 263, 1284])
+@pytest.mark.parametrize("key_only", [False, True])
+def test_mask_types_vector_and_scalar_loads(risa, mask_dtype, k_len, key_only):
+    """Every mask element type through both load paths of the kernel: rows of 264 and
+    1284 keys are aligned for one load per four keys, rows of 263 keys are not; a
+    key-only mask over more than 1024 keys selects the 128-key tile."""
+    dim, q_len = 128, 70
+    q = seeded((1, 2, q_len, dim), torch.bfloat16, 41)
+    k = seeded((1, 2, k_len, dim), torch.bfloat16, 42)
+    v = seeded((1, 2, k_len, dim), torch.bfloat16, 43)
+    generator = torch.Generator(device="cpu").manual_seed(44)
+    shape = (1, 1, 1 if key_only else q_len, k_len)
+    if mask_dtype == torch.bool:
+        mask = torch.rand(shape, generator=generator) > 0.3
+        mask[..., -5:] = False
+        if not key_only:
+            mask[:, :, 3] = False  # a fully hidden row
+    else:
+        mask = torch.randn(shape, generator=generator).to(mask_dtype)
+        mask[..., 5::11] = float("-inf")
+    mask = mask.cuda()
+    out, lse = risa.int8_attention(q, k, v, attn_mask=mask, return_lse=True)
+    prepared = oracle_prequantize(q, k, v, attn_mask=mask, return_lse=True)
+    assert prepared.cta_k == (128 if key_only and k_len > 1024 else 64)
+    expected, expected_lse, _ = oracle_pipeline.attend(prepared, return_lse=True)
+    assert relative_l2(to_numpy(out), expected) < TOLERANCE
+    assert relative_l2(to_numpy(lse), expected_lse) < TOLERANCE
+
+
+def test_causal_launch_order_covers_every_block(risa):
+    """Causal launches walk the query blocks longest first; every block of every head
+    and batch entry must still be written exactly as the dense causal oracle says."""
+    q = seeded((2, 3, 700, 64), torch.float16, 51)
+    k = seeded((2, 3, 700, 64), torch.float16, 52)
+    v = seeded((2, 3, 700, 64), torch.float16, 53)
+    out = risa.int8_attention(q, k, v, is_causal=True)
+    prepared = oracle_prequantize(q, k, v, is_causal=True)
+    expected, _, _ = oracle_pipeline.attend(prepared)
+    assert relative_l2(to_numpy(out), expected) < TOLERANCE
