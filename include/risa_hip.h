@@ -105,7 +105,10 @@ void risa_unpack_order(int32_t* order);
  *   total size as reference attention_int8.cuh:51-143, 871-898, whose full-tile
  *   stats are row-major); lse (nullable) float32
  *   [B,Hq,Lq]; key_mask_tiles (nullable) int32 [B,Hq,tiles+1] from
- *   risa_prepare_key_mask_tiles.
+ *   risa_prepare_key_mask_tiles; key_bias (nullable) float32 [Bm,Hm,padded keys]
+ *   from risa_prepare_key_bias with its batch and head strides in elements (0
+ *   for a broadcast extent): given together with a key-only mask (mask_stride_q
+ *   0), the kernel stages this row per key tile instead of reading mask elements.
  */
 int risa_attention(const void* q_int8, const void* k_int8, const void* v_int8, void* out,
                    const float* q_scale, const float* k_scale, const float* v_scale,
@@ -116,6 +119,7 @@ int risa_attention(const void* q_int8, const void* k_int8, const void* v_int8, v
                    int64_t out_stride_n, int64_t out_stride_h, float sm_scale, int out_dtype,
                    const int32_t* sparse_row_offsets, const int32_t* sparse_block_indices,
                    float* block_mass, int is_causal, float* lse, const int32_t* key_mask_tiles,
+                   const float* key_bias, int64_t key_bias_stride_b, int64_t key_bias_stride_h,
                    void* stream);
 
 /*
@@ -139,6 +143,18 @@ int risa_select_retained_mass(const float* sorted_mass, const int64_t* descendin
 int risa_prepare_key_mask_tiles(const void* mask, int32_t* tiles, int batch, int q_heads,
                                 int key_length, int tile_size, int64_t stride_b, int64_t stride_h,
                                 int64_t stride_k, int mask_dtype, void* stream);
+
+/*
+ * Additive form of a key-only mask, in the exp2 domain: bias[b,h,key] =
+ * mask * log2(e) for finite float entries, 0 for true, -inf for false, non-finite
+ * and padded keys (key_length <= key < padded_length).  batch and heads are the
+ * mask's own extents (1 where it broadcasts); bias is [batch,heads,padded_length]
+ * float32.  No counterpart in the reference, whose kernel reads the mask per
+ * score (csrc/kernels/attention_masks.cuh); the values are the ones it adds.
+ */
+int risa_prepare_key_bias(const void* mask, float* bias, int batch, int heads, int key_length,
+                          int padded_length, int64_t stride_b, int64_t stride_h, int64_t stride_k,
+                          int mask_dtype, void* stream);
 
 /*
  * LSE anchor correction out[b,h,i] = scale * <q[b,h,i], k[b,h/G,anchor[b,h/G]]>.

@@ -10,7 +10,7 @@ import math
 import torch
 
 from . import native
-from .key_mask import prepare_key_mask_tiles
+from .key_mask import prepare_key_bias, prepare_key_mask_tiles
 from .policy import (
     DTYPE_CODES,
     MASK_DTYPE_CODES,
@@ -142,6 +142,8 @@ def launch_attention(*, q_codes, k_codes, v_codes, output, q_scale, k_scale, v_s
     ):
         raise RuntimeError("key mask tiles must be contiguous CUDA int32 [B,Hq,tiles+1]")
     sums = ensure_tile_sums(v_codes, v_tile_sum, batch * kv_heads, dim, cta_k)
+    key_bias = prepare_key_bias(attn_mask, cta_k)
+    bias_args = (None, 0, 0) if key_bias is None else (key_bias[0].data_ptr(), key_bias[1], key_bias[2])
     out_b = output.stride(0) if batch > 1 else q_heads * q_len * dim
     out_n = output.stride(2) if q_len > 1 else dim
     out_h = output.stride(1) if q_heads > 1 else q_len * dim
@@ -153,7 +155,7 @@ def launch_attention(*, q_codes, k_codes, v_codes, output, q_scale, k_scale, v_s
             out_b, out_n, out_h, float(sm_scale), DTYPE_CODES[output.dtype],
             native.pointer(row_offsets), native.pointer(block_indices), native.pointer(block_mass),
             int(bool(is_causal)), native.pointer(lse), native.pointer(key_mask_tiles),
-            native.current_stream(q_codes.device),
+            *bias_args, native.current_stream(q_codes.device),
         )
     )
 

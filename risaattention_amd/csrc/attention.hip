@@ -117,6 +117,15 @@ int launch_attention(const AttentionArgs& a, hipStream_t stream) {
     const bool aligned = reinterpret_cast<uintptr_t>(a.mask) % (4 * element) == 0 &&
                          ((a.mask_stride_b | a.mask_stride_h | a.mask_stride_q) & 3) == 0;
     p.mask_vector = a.mask_stride_k == 1 && aligned ? 1 : 0;
+    if (a.key_bias != nullptr) {
+      if (a.mask_stride_q != 0) return fail("risa_attention: a key bias row needs a key-only mask");
+      if (reinterpret_cast<uintptr_t>(a.key_bias) % 16 != 0 || (a.key_bias_stride_b | a.key_bias_stride_h) % 4 != 0)
+        return fail("risa_attention: key bias rows must be 16-byte aligned");
+      p.mask_dtype = kKeyBias;
+      p.key_bias = a.key_bias;
+      p.key_bias_stride_b = a.key_bias_stride_b;
+      p.key_bias_stride_h = a.key_bias_stride_h;
+    }
   }
   p.q_len = a.q_len;
   p.k_len = a.k_len;

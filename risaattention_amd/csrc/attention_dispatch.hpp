@@ -51,6 +51,7 @@ int launch_tile(const KernelParams& p, bool fast, bool indexed, bool capture, hi
     case kF32: return launch_general<D, CTA_K, kF32>(p, indexed, capture, stream);
     case kF16: return launch_general<D, CTA_K, kF16>(p, indexed, capture, stream);
     case kBF16: return launch_general<D, CTA_K, kBF16>(p, indexed, capture, stream);
+    case kKeyBias: return launch_general<D, CTA_K, kKeyBias>(p, indexed, capture, stream);
     default: return launch_general<D, CTA_K, -1>(p, indexed, capture, stream);
   }
 }

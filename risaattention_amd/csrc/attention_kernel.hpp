@@ -59,6 +59,8 @@ struct KernelParams {
   int64_t mask_stride_b, mask_stride_h, mask_stride_q, mask_stride_k;
   int mask_dtype;  // -1: no mask
   int mask_vector;  // keys are contiguous and groups of four keys aligned: one load per group
+  const float* key_bias;  // key-only mask as an additive row [Bm,Hm,padded] (mask_dtype kKeyBias)
+  int64_t key_bias_stride_b, key_bias_stride_h;
   int q_len, k_len, q_heads, kv_heads, padded, n_kb, n_qb, batch;
   int64_t out_stride_b, out_stride_n, out_stride_h;
   float sm2;  // sm_scale * log2(e)
@@ -118,12 +120,15 @@ __device__ __forceinline__ int fresh_lane() {
 template <int D, int CTA_K> struct TileShape {
   static constexpr int kTileBytes = CTA_K * D;
   static constexpr int kCopiesPerWave = kTileBytes / 16 / 256;  // 1 KB copy instructions per wave
-  static constexpr int kStageBytes = 2 * kTileBytes + D * 4;     // K, V, zero-point terms
+  static constexpr int kSeedBytes = D * 4;                       // accumulator seeds of the tile
+  static constexpr int kBiasBytes = CTA_K * 4;                   // key-only mask row of the tile
+  static constexpr int kStageBytes = 2 * kTileBytes + kSeedBytes + kBiasBytes;
   static constexpr int kLdsBytes = 2 * kStageBytes;
 };
 
-// MASK_DT: element type of the mask tensor (risa::kBool, kF32, kF16, kBF16) or -1
-// for none; FAST (raw-score path) implies -1.
+// MASK_DT: element type of the mask tensor (risa::kBool, kF32, kF16, kBF16), kKeyBias
+// for a key-only mask prepared as an FP32 row, or -1 for none; FAST (raw-score path)
+// implies -1.
 template <int D, int CTA_K, bool FAST, bool INDEXED, bool CAPTURE, int MASK_DT>
 __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void attention_kernel(const KernelParams p) {
   static_assert(!FAST || MASK_DT < 0, "the raw-score path takes no mask");
@@ -165,6 +170,10 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void attention_kernel(cons
   const int8_t* v_base = p.v + bhk * D * p.padded;
   const int32_t* sum_base = p.v_tile_sum + bhk * p.n_kb * D;
   const float* ks_base = p.k_scale + bhk * p.n_kb * 4;
+  [[maybe_unused]] const float* bias_base = nullptr;
+  if constexpr (MASK_DT == kKeyBias) {
+    bias_base = p.key_bias + batch * p.key_bias_stride_b + head * p.key_bias_stride_h;
+  }
 
   const int query = bx * kQueryBlock + wave * 32 + l32;
   const bool query_ok = query < p.q_len;
@@ -265,6 +274,15 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void attention_kernel(cons
                               static_cast<uint32_t>(lane_id) * 16, sl);
       }
     }
+    if constexpr (MASK_DT == kKeyBias) {
+      if (wave == 1) {
+        const int lane_id = fresh_lane();
+        if (lane_id < CTA_K / 4) {
+          copy16_to_lds_uniform(reinterpret_cast<const int8_t*>(bias_base + static_cast<int64_t>(tile) * CTA_K),
+                                static_cast<uint32_t>(lane_id) * 16, sl + Shape::kSeedBytes);
+        }
+      }
+    }
   };
 
   // --- Q operand and scales ------------------------------------------------
@@ -306,7 +324,7 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void attention_kernel(cons
   }
 
   const int64_t mask_row =
-      (MASK_DT >= 0)
+      (MASK_DT >= 0 && MASK_DT != kKeyBias)
           ? static_cast<int64_t>(batch) * p.mask_stride_b + static_cast<int64_t>(head) * p.mask_stride_h +
                 static_cast<int64_t>(query) * p.mask_stride_q
           : 0;
@@ -439,6 +457,27 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void attention_kernel(cons
             const float value = static_cast<float>(s[rb][i]) * ((i & 2) ? sc1 : sc0);
             s[rb][i] = __float_as_int(value);
             mx = __builtin_fmaxf(mx, value);
+          }
+      } else if constexpr (MASK_DT == kKeyBias) {
+        // Key-only mask: the tile's row of additive terms (already in the exp2
+        // domain, -inf for hidden and out-of-range keys) sits in LDS next to the
+        // seeds; a lane reads the four consecutive keys of a group in one go.
+        const float* bias_row = reinterpret_cast<const float*>(
+            lds + (it & 1) * Shape::kStageBytes + 2 * Shape::kTileBytes + Shape::kSeedBytes);
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+          for (int b4 = 0; b4 < 4; ++b4) {
+            const int local = rb * 32 + b4 * 8 + half * 4;
+            const float4 bias = *reinterpret_cast<const float4*>(bias_row + local);
+            const float terms[4] = {bias.x, bias.y, bias.z, bias.w};
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+              float value = static_cast<float>(s[rb][b4 * 4 + r]) * ((r & 2) ? sc1 : sc0) + terms[r];
+              if (p.causal && tile * CTA_K + local + r > query) value = neg_inf;
+              s[rb][b4 * 4 + r] = __float_as_int(value);
+              mx = __builtin_fmaxf(mx, value);
+            }
           }
       } else {
         // DT: mask element type (-1: none, only the causal / key-range tests);

@@ -143,6 +143,7 @@ int risa_attention(const void* q_int8, const void* k_int8, const void* v_int8, v
                    int64_t out_stride_n, int64_t out_stride_h, float sm_scale, int out_dtype,
                    const int32_t* sparse_row_offsets, const int32_t* sparse_block_indices,
                    float* block_mass, int is_causal, float* lse, const int32_t* key_mask_tiles,
+                   const float* key_bias, int64_t key_bias_stride_b, int64_t key_bias_stride_h,
                    void* stream) {
   using risa::fail;
   if (out_dtype != 1 && out_dtype != 2)
@@ -187,6 +188,11 @@ int risa_attention(const void* q_int8, const void* k_int8, const void* v_int8, v
   a.is_causal = is_causal != 0;
   a.lse = lse;
   a.key_mask_tiles = key_mask_tiles;
+  if (key_bias != nullptr && (mask == nullptr || mask_stride_q != 0))
+    return fail("risa_attention: a key bias row goes with a key-only mask (query stride 0)");
+  a.key_bias = key_bias;
+  a.key_bias_stride_b = key_bias_stride_b;
+  a.key_bias_stride_h = key_bias_stride_h;
   return risa::launch_attention(a, static_cast<hipStream_t>(stream));
 }
 
@@ -215,6 +221,18 @@ int risa_prepare_key_mask_tiles(const void* mask, int32_t* tiles, int batch, int
   return risa::launch_key_mask_tiles(mask, tiles, batch, q_heads, key_length, tile_size, stride_b,
                                      stride_h, stride_k, mask_dtype,
                                      static_cast<hipStream_t>(stream));
+}
+
+int risa_prepare_key_bias(const void* mask, float* bias, int batch, int heads, int key_length,
+                          int padded_length, int64_t stride_b, int64_t stride_h, int64_t stride_k,
+                          int mask_dtype, void* stream) {
+  if (mask == nullptr || bias == nullptr || batch <= 0 || heads <= 0 || key_length <= 0 ||
+      padded_length < key_length || padded_length % 64 != 0)
+    return risa::fail("risa_prepare_key_bias: bad extents");
+  if (mask_dtype < 0 || mask_dtype > 3)
+    return risa::fail("risa_prepare_key_bias requires a supported mask dtype");
+  return risa::launch_key_bias(mask, bias, batch, heads, key_length, padded_length, stride_b,
+                               stride_h, stride_k, mask_dtype, static_cast<hipStream_t>(stream));
 }
 
 int risa_lse_shift(const void* q, const void* k, const int32_t* anchors, float* out, int batch,

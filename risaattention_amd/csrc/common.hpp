@@ -38,6 +38,8 @@ constexpr int kF32 = 0;
 constexpr int kF16 = 1;
 constexpr int kBF16 = 2;
 constexpr int kBool = 3;
+// Kernel-internal mask kind: a key-only mask staged per tile as an FP32 bias row.
+constexpr int kKeyBias = 4;
 
 constexpr int kWave = 64;
 

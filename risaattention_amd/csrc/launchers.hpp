@@ -77,6 +77,8 @@ struct AttentionArgs {
   bool is_causal;
   float* lse;
   const int32_t* key_mask_tiles;
+  const float* key_bias;  // [Bm,Hm,padded] from launch_key_bias, or null
+  int64_t key_bias_stride_b, key_bias_stride_h;
 };
 int launch_attention(const AttentionArgs& args, hipStream_t stream);
 
@@ -97,5 +99,9 @@ int launch_select_retained_mass(const SelectArgs& args, hipStream_t stream);
 int launch_key_mask_tiles(const void* mask, int32_t* tiles, int batch, int heads, int length,
                           int tile_size, int64_t stride_b, int64_t stride_h, int64_t stride_k,
                           int dtype, hipStream_t stream);
+
+int launch_key_bias(const void* mask, float* bias, int batch, int heads, int length, int padded,
+                    int64_t stride_b, int64_t stride_h, int64_t stride_k, int dtype,
+                    hipStream_t stream);
 
 }  // namespace risa

@@ -191,7 +191,39 @@ __global__ __launch_bounds__(256) void key_mask_tiles_kernel(const void* __restr
   }
 }
 
+// grid (ceil(padded/256), heads, batch), 256 threads: one key each.  The product
+// bias * log2(e) is the FP32 product the attention kernel would form per score.
+__global__ __launch_bounds__(256) void key_bias_kernel(const void* __restrict__ mask,
+                                                       float* __restrict__ bias, int length,
+                                                       int padded, int64_t stride_b, int64_t stride_h,
+                                                       int64_t stride_k, int dtype) {
+  const int key = blockIdx.x * 256 + threadIdx.x;
+  if (key >= padded) return;
+  float value = -__builtin_inff();
+  if (key < length) {
+    const int64_t index = blockIdx.z * stride_b + blockIdx.y * stride_h + key * stride_k;
+    if (dtype == kBool) {
+      if (static_cast<const uint8_t*>(mask)[index] != 0) value = 0.0f;
+    } else {
+      const float raw = dtype == kF32   ? load1<kF32>(mask, index)
+                        : dtype == kF16 ? load1<kF16>(mask, index)
+                                        : load1<kBF16>(mask, index);
+      if (__builtin_isfinite(raw)) value = raw * 1.44269504088896340736f;
+    }
+  }
+  bias[(static_cast<int64_t>(blockIdx.z) * gridDim.y + blockIdx.y) * padded + key] = value;
+}
+
 }  // namespace
+
+int launch_key_bias(const void* mask, float* bias, int batch, int heads, int length, int padded,
+                    int64_t stride_b, int64_t stride_h, int64_t stride_k, int dtype,
+                    hipStream_t stream) {
+  const dim3 grid((padded + 255) / 256, heads, batch);
+  key_bias_kernel<<<grid, 256, 0, stream>>>(mask, bias, length, padded, stride_b, stride_h, stride_k,
+                                            dtype);
+  return check_launch("risa_prepare_key_bias");
+}
 
 int launch_select_retained_mass(const SelectArgs& a, hipStream_t stream) {
   select_rows_kernel<<<(a.rows + 1) / 2, 64, 0, stream>>>(a.sorted_mass, a.descending_indices,

@@ -11,6 +11,31 @@ from . import native
 from .policy import MASK_DTYPE_CODES
 
 
+def prepare_key_bias(mask, key_block_size):
+    """Additive FP32 row of a key-only mask, ``(bias, stride_b, stride_h)`` or ``None``.
+
+    ``mask`` is the expanded ``[B,Hq,Lq,Lk]`` view.  Without a query extent
+    (stride 0) every query of a head sees the same row, so the attention kernel
+    can stage ``bias[b,h,tile]`` per key tile instead of reading mask elements
+    per score: 0 / the float entry times log2(e) / -inf, padded to whole tiles.
+    """
+    if mask is None or mask.stride(2) != 0:
+        return None
+    batch = mask.shape[0] if mask.stride(0) != 0 else 1
+    heads = mask.shape[1] if mask.stride(1) != 0 else 1
+    length = mask.shape[-1]
+    padded = -(-length // key_block_size) * key_block_size
+    bias = torch.empty((batch, heads, padded), device=mask.device, dtype=torch.float32)
+    native.check(
+        native.library().risa_prepare_key_bias(
+            mask.data_ptr(), bias.data_ptr(), batch, heads, length, padded,
+            mask.stride(0), mask.stride(1), mask.stride(3), MASK_DTYPE_CODES[mask.dtype],
+            native.current_stream(mask.device),
+        )
+    )
+    return bias, (bias.stride(0) if batch > 1 else 0), (bias.stride(1) if heads > 1 else 0)
+
+
 def prepare_key_mask_tiles(mask, key_block_size, query_length, scale, is_causal):
     """int32 [B,Hq,tiles+1] (active tile ids, then the count) or None.
 
