@@ -13,6 +13,8 @@
 #include "common.hpp"
 #include "launchers.hpp"
 
+#include <type_traits>
+
 namespace risa {
 namespace {
 
@@ -45,15 +47,52 @@ __device__ __forceinline__ void apply_sign_diagonal(float* v, int sub) {
   }
 }
 
-template <int LANES> __device__ __forceinline__ void lane_butterflies(float* v, int sub) {
-#pragma unroll
-  for (int bit = 1; bit < LANES; bit <<= 1) {
-#pragma unroll
-    for (int c = 0; c < 4; ++c) {
-      const float other = __shfl_xor(v[c], bit);
-      v[c] = (sub & bit) ? other - v[c] : v[c] + other;
-    }
+// Value of lane (l xor BIT) for BIT in {1, 2, 4, 8}, with DPP moves (no LDS
+// traffic): quad permutations inside groups of four lanes, row shifts inside
+// rows of sixteen lanes written under a bank mask (lanes whose partner is above
+// take the left shift, the others the right shift).
+template <int BIT> __device__ __forceinline__ float dpp_partner(float value) {
+  const int bits = __float_as_int(value);
+  if constexpr (BIT == 1) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, bits, 0xB1, 0xf, 0xf, true));  // quad_perm [1,0,3,2]
+  } else if constexpr (BIT == 2) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, bits, 0x4E, 0xf, 0xf, true));  // quad_perm [2,3,0,1]
+  } else if constexpr (BIT == 4) {
+    const int up = __builtin_amdgcn_update_dpp(0, bits, 0x104, 0xf, 0x5, true);      // row_shl:4 -> banks 0, 2
+    return __int_as_float(__builtin_amdgcn_update_dpp(up, bits, 0x114, 0xf, 0xA, false));  // row_shr:4 -> banks 1, 3
+  } else {
+    static_assert(BIT == 8, "DPP reaches partners inside a row of sixteen lanes");
+    const int up = __builtin_amdgcn_update_dpp(0, bits, 0x108, 0xf, 0x3, true);      // row_shl:8 -> banks 0, 1
+    return __int_as_float(__builtin_amdgcn_update_dpp(up, bits, 0x118, 0xf, 0xC, false));  // row_shr:8 -> banks 2, 3
   }
+}
+
+// Hadamard butterflies over the lane bits below LANES, in the reference's order
+// (bit 1 first): the lane with the bit clear keeps a + b, the other b - a.
+template <int LANES> __device__ __forceinline__ void lane_butterflies(float* v, int sub) {
+  auto level = [&](auto bit_tag) {
+    constexpr int BIT = decltype(bit_tag)::value;
+    if constexpr (BIT < LANES) {
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        float other;
+        if constexpr (BIT < 16) {
+          other = dpp_partner<BIT>(v[c]);
+        } else {
+          other = __shfl_xor(v[c], BIT);
+        }
+        // other - v on the lanes with the bit set, other + v on the rest: one sign
+        // flip (exact) and one addition instead of both results and a select
+        const uint32_t flip = (sub & BIT) ? 0x80000000u : 0u;
+        v[c] = other + __uint_as_float(__float_as_uint(v[c]) ^ flip);
+      }
+    }
+  };
+  level(std::integral_constant<int, 1>{});
+  level(std::integral_constant<int, 2>{});
+  level(std::integral_constant<int, 4>{});
+  level(std::integral_constant<int, 8>{});
+  level(std::integral_constant<int, 16>{});
 }
 
 template <int ROT> __device__ __forceinline__ void rotate(float* v, int sub) {
