@@ -95,20 +95,36 @@ template <int LANES> __device__ __forceinline__ void lane_butterflies(float* v, 
   level(std::integral_constant<int, 16>{});
 }
 
-template <int ROT> __device__ __forceinline__ void rotate(float* v, int sub) {
-  if constexpr (ROT == kRot128Signed) {
-    apply_sign_diagonal(v, sub);
-  }
-  rotate4(v);
-  if constexpr (ROT == kRot64) {
-    lane_butterflies<16>(v, sub & 15);
+// Rotation of the channels one lane holds of one 128-channel block (64 for head
+// dim 64).  Sixteen lanes share a token; lane j owns GROUPS runs of four
+// consecutive channels, 4*GROUPS*j + 4g .. +3, i.e. the channels of lanes 2j and
+// 2j+1 (GROUPS 2) or of lane j (GROUPS 1) of the reference's 32-lane layout
+// (csrc/kernels/quantize_qk.cuh).  The additions are the reference's, in its
+// order: 4-point transform per run, then one butterfly level per channel bit from
+// bit 2 up -- the first inside the lane when it holds two runs, the others
+// between lanes with DPP moves.
+template <int ROT, int GROUPS> __device__ __forceinline__ void rotate(float (&v)[GROUPS][4], int j) {
 #pragma unroll
-    for (int c = 0; c < 4; ++c) v[c] *= 0.25f;
-  } else if constexpr (ROT == kRot128Signed || ROT == kRot128Plain) {
-    lane_butterflies<32>(v, sub);
-#pragma unroll
-    for (int c = 0; c < 4; ++c) v[c] *= 0.1767766952966369f;
+  for (int g = 0; g < GROUPS; ++g) {
+    if constexpr (ROT == kRot128Signed) apply_sign_diagonal(v[g], GROUPS * j + g);
+    rotate4(v[g]);
   }
+  if constexpr (ROT == kRot4) return;
+  if constexpr (GROUPS == 2) {
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      const float low = v[0][c], high = v[1][c];
+      v[0][c] = low + high;
+      v[1][c] = low - high;
+    }
+  }
+#pragma unroll
+  for (int g = 0; g < GROUPS; ++g) lane_butterflies<16>(v[g], j);
+  constexpr float factor = ROT == kRot64 ? 0.25f : 0.1767766952966369f;
+#pragma unroll
+  for (int g = 0; g < GROUPS; ++g)
+#pragma unroll
+    for (int c = 0; c < 4; ++c) v[g][c] *= factor;
 }
 
 __device__ __forceinline__ float half_wave_max(float value) {
@@ -119,61 +135,103 @@ __device__ __forceinline__ float half_wave_max(float value) {
   return value;
 }
 
-// One scale group handled by one 32-lane half: NTOK tokens x DK channels.
-// `token_of(i)` gives the i-th token of the group.
+// One scale group handled by one 32-lane half: NTOK tokens x DK channels, two
+// tokens at a time (one per 16-lane row).  `token_of(i)` gives the i-th token of
+// the group.  `wide` says rows are 16-byte aligned, so 16-bit inputs are read
+// eight channels per load.
 template <int DT, int DK, int ROT, int NTOK, typename TokenOf>
 __device__ __forceinline__ void quantize_group(const void* in, int64_t in_base, int64_t stride_n,
                                                int8_t* out, float* scale_slot, int length, int sub,
-                                               const float* bias, TokenOf token_of) {
-  constexpr int CT = DK == 256 ? 2 : 1;
-  float v[CT][NTOK][4];
+                                               const void* bias_row, bool wide, TokenOf token_of) {
+  constexpr int BLOCKS = DK == 256 ? 2 : 1;   // 128-channel rotation blocks
+  constexpr int GROUPS = DK == 64 ? 1 : 2;    // runs of four channels per lane and block
+  constexpr int STEPS = NTOK / 2;
+  static_assert(NTOK % 2 == 0, "two tokens per 32-lane half and step");
+  const int j = sub & 15, row = sub >> 4;
+  auto channel_of = [&](int block, int g) { return block * 128 + (GROUPS * j + g) * 4; };
+
+  auto load_row = [&](int64_t row_base, float (&dst)[BLOCKS][GROUPS][4]) {
 #pragma unroll
-  for (int tile = 0; tile < CT; ++tile) {
-    const int ch = tile * 128 + sub * 4;
+    for (int block = 0; block < BLOCKS; ++block) {
+      if (GROUPS == 2 && DT != kF32 && wide) {
+        float eight[8];
+        load8<DT>(in, row_base + channel_of(block, 0), eight);
 #pragma unroll
-    for (int i = 0; i < NTOK; ++i) {
-      const int n = token_of(i);
-      v[tile][i][0] = v[tile][i][1] = v[tile][i][2] = v[tile][i][3] = 0.0f;
-      if (ch < DK && n < length) {
-        load4<DT>(in, in_base + static_cast<int64_t>(n) * stride_n + ch, v[tile][i]);
-        if (bias != nullptr) {
+        for (int c = 0; c < 8; ++c) dst[block][c / 4][c % 4] = eight[c];
+      } else {
 #pragma unroll
-          for (int c = 0; c < 4; ++c) v[tile][i][c] -= bias[tile * 4 + c];
-        }
+        for (int g = 0; g < GROUPS; ++g) load4<DT>(in, row_base + channel_of(block, g), dst[block][g]);
       }
+    }
+  };
+
+  float bias[BLOCKS][GROUPS][4];
+  if (bias_row != nullptr) load_row(in_base + *static_cast<const int64_t*>(bias_row), bias);
+
+  float v[STEPS][BLOCKS][GROUPS][4];
+#pragma unroll
+  for (int i = 0; i < STEPS; ++i) {
+    const int n = token_of(2 * i + row);
+    if (n < length) {
+      load_row(in_base + static_cast<int64_t>(n) * stride_n, v[i]);
+      if (bias_row != nullptr) {
+#pragma unroll
+        for (int block = 0; block < BLOCKS; ++block)
+#pragma unroll
+          for (int g = 0; g < GROUPS; ++g)
+#pragma unroll
+            for (int c = 0; c < 4; ++c) v[i][block][g][c] -= bias[block][g][c];
+      }
+    } else {
+#pragma unroll
+      for (int block = 0; block < BLOCKS; ++block)
+#pragma unroll
+        for (int g = 0; g < GROUPS; ++g)
+#pragma unroll
+          for (int c = 0; c < 4; ++c) v[i][block][g][c] = 0.0f;
     }
   }
   float mx = 0.0f;
 #pragma unroll
-  for (int tile = 0; tile < CT; ++tile) {
+  for (int i = 0; i < STEPS; ++i)
 #pragma unroll
-    for (int i = 0; i < NTOK; ++i) {
-      rotate<ROT>(v[tile][i], sub);
+    for (int block = 0; block < BLOCKS; ++block) {
+      rotate<ROT, GROUPS>(v[i][block], j);
 #pragma unroll
-      for (int c = 0; c < 4; ++c) mx = __builtin_fmaxf(mx, __builtin_fabsf(v[tile][i][c]));
+      for (int g = 0; g < GROUPS; ++g)
+#pragma unroll
+        for (int c = 0; c < 4; ++c) mx = __builtin_fmaxf(mx, __builtin_fabsf(v[i][block][g][c]));
     }
-  }
   mx = half_wave_max(mx);
   const float scale = mx / 127.0f + 1e-7f;
   const float inverse = 1.0f / scale;
   if (sub == 0) *scale_slot = scale;
 #pragma unroll
-  for (int tile = 0; tile < CT; ++tile) {
-    const int ch = tile * 128 + sub * 4;
+  for (int i = 0; i < STEPS; ++i) {
+    const int n = token_of(2 * i + row);
+    if (n < length) {
 #pragma unroll
-    for (int i = 0; i < NTOK; ++i) {
-      const int n = token_of(i);
-      if (ch < DK && n < length) {
-        const uint32_t packed =
-            pack_s8x4(quantize_s8(v[tile][i][0] * inverse), quantize_s8(v[tile][i][1] * inverse),
-                      quantize_s8(v[tile][i][2] * inverse), quantize_s8(v[tile][i][3] * inverse));
-        *reinterpret_cast<uint32_t*>(out + static_cast<int64_t>(n) * DK + ch) = packed;
+      for (int block = 0; block < BLOCKS; ++block) {
+        uint32_t packed[GROUPS];
+#pragma unroll
+        for (int g = 0; g < GROUPS; ++g) {
+          packed[g] = pack_s8x4(quantize_s8(v[i][block][g][0] * inverse), quantize_s8(v[i][block][g][1] * inverse),
+                                quantize_s8(v[i][block][g][2] * inverse), quantize_s8(v[i][block][g][3] * inverse));
+        }
+        int8_t* at = out + static_cast<int64_t>(n) * DK + channel_of(block, 0);
+        if constexpr (GROUPS == 2) {
+          *reinterpret_cast<uint2*>(at) = make_uint2(packed[0], packed[1]);
+        } else {
+          *reinterpret_cast<uint32_t*>(at) = packed[0];
+        }
       }
     }
   }
 }
 
-// grid (slices, Hq, B), 256 threads: eight 32-lane halves = the eight scale
+constexpr int kSlicesPerBlock = 1;
+
+// grid (ceil(slices / kSlicesPerBlock), Hq, B), 256 threads: eight 32-lane halves = the eight scale
 // groups (token index mod 8) of one W-row slice, W = 32 (16 for head_dim 256).
 template <int DT, int DK, int ROT>
 __global__ __launch_bounds__(256) void quantize_q_kernel(const void* __restrict__ q,
@@ -181,18 +239,27 @@ __global__ __launch_bounds__(256) void quantize_q_kernel(const void* __restrict_
                                                          float* __restrict__ scales, int length,
                                                          int heads, int scales_per_head,
                                                          int64_t stride_b, int64_t stride_h,
-                                                         int64_t stride_n) {
+                                                         int64_t stride_n, int wide) {
   constexpr int W = DK == 256 ? 16 : 32;
   constexpr int NR = W / 8;
-  const int slice = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+  const int h = blockIdx.y, b = blockIdx.z;
   const int sub = threadIdx.x & 31;
   const int group = threadIdx.x >> 5;
-  const int base = slice * W + group;
   const int64_t in_base = static_cast<int64_t>(b) * stride_b + static_cast<int64_t>(h) * stride_h;
   const int64_t bh = static_cast<int64_t>(b) * heads + h;
-  quantize_group<DT, DK, ROT, NR>(q, in_base, stride_n, codes + bh * length * DK,
-                                  scales + bh * scales_per_head + slice * 8 + group, length, sub,
-                                  nullptr, [base](int i) { return base + i * 8; });
+  // kSlicesPerBlock consecutive slices per workgroup.  One is fastest (52.6 us at
+  // 16 x 32768 tokens against 59.8 us with four): the loop serialises the loads of
+  // successive slices, and workgroup launch is not what limits the kernel.
+  const int slices = scales_per_head / 8;
+#pragma unroll 1
+  for (int step = 0; step < kSlicesPerBlock; ++step) {
+    const int slice = blockIdx.x * kSlicesPerBlock + step;
+    if (slice >= slices) break;
+    const int base = slice * W + group;
+    quantize_group<DT, DK, ROT, NR>(q, in_base, stride_n, codes + bh * length * DK,
+                                    scales + bh * scales_per_head + slice * 8 + group, length, sub,
+                                    nullptr, wide != 0, [base](int i) { return base + i * 8; });
+  }
 }
 
 // grid (key tiles, Hkv, B), 128 threads: four 32-lane halves = the four scale
@@ -204,8 +271,7 @@ __global__ __launch_bounds__(128) void quantize_k_kernel(const void* __restrict_
                                                          const int* __restrict__ anchors, int length,
                                                          int heads, int scales_per_head,
                                                          int64_t stride_b, int64_t stride_h,
-                                                         int64_t stride_n) {
-  constexpr int CT = DK == 256 ? 2 : 1;
+                                                         int64_t stride_n, int wide) {
   constexpr int NTOK = CTA_K / 4;
   const int tile = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
   const int sub = threadIdx.x & 31;
@@ -213,19 +279,12 @@ __global__ __launch_bounds__(128) void quantize_k_kernel(const void* __restrict_
   const int64_t in_base = static_cast<int64_t>(b) * stride_b + static_cast<int64_t>(h) * stride_h;
   const int64_t bh = static_cast<int64_t>(b) * heads + h;
   const int anchor = anchors[b * heads + h];
-  float bias[CT * 4];
-#pragma unroll
-  for (int t = 0; t < CT; ++t) {
-    const int ch = t * 128 + sub * 4;
-    bias[t * 4] = bias[t * 4 + 1] = bias[t * 4 + 2] = bias[t * 4 + 3] = 0.0f;
-    if (anchor >= 0 && ch < DK) {
-      load4<DT>(k, in_base + static_cast<int64_t>(anchor) * stride_n + ch, bias + t * 4);
-    }
-  }
+  // element offset of the anchor row (subtracted from every key) when one was chosen
+  const int64_t anchor_offset = static_cast<int64_t>(anchor) * stride_n;
   const int first = tile * CTA_K + group * 2;
   quantize_group<DT, DK, ROT, NTOK>(k, in_base, stride_n, codes + bh * length * DK,
                                     scales + bh * scales_per_head + tile * 4 + group, length, sub,
-                                    anchor >= 0 ? bias : nullptr,
+                                    anchor >= 0 ? &anchor_offset : nullptr, wide != 0,
                                     [first](int i) { return first + (i >> 1) * 8 + (i & 1); });
 }
 
@@ -343,14 +402,22 @@ __global__ __launch_bounds__(128) void detect_anchor_kernel(const void* __restri
   }
 }
 
+// 16-bit inputs can be read eight channels (16 bytes) per load when every row
+// starts on a 16-byte boundary.
+inline int rows_are_16_byte_aligned(const void* base, int64_t stride_b, int64_t stride_h,
+                                    int64_t stride_n, int dtype) {
+  if (dtype == kF32) return 1;
+  return reinterpret_cast<uintptr_t>(base) % 16 == 0 && ((stride_b | stride_h | stride_n) & 7) == 0;
+}
+
 template <int DT, int DK, int ROT>
 void launch_q(const QkArgs& a, hipStream_t stream) {
   constexpr int W = DK == 256 ? 16 : 32;
   const int slices = (a.q_len + 127) / 128 * (128 / W);
-  dim3 grid(slices, a.q_heads, a.batch);
-  quantize_q_kernel<DT, DK, ROT><<<grid, 256, 0, stream>>>(a.q, a.q_codes, a.q_scale, a.q_len,
-                                                           a.q_heads, slices * 8, a.q_stride_b,
-                                                           a.q_stride_h, a.q_stride_n);
+  dim3 grid((slices + kSlicesPerBlock - 1) / kSlicesPerBlock, a.q_heads, a.batch);
+  quantize_q_kernel<DT, DK, ROT><<<grid, 256, 0, stream>>>(
+      a.q, a.q_codes, a.q_scale, a.q_len, a.q_heads, slices * 8, a.q_stride_b, a.q_stride_h,
+      a.q_stride_n, rows_are_16_byte_aligned(a.q, a.q_stride_b, a.q_stride_h, a.q_stride_n, a.dtype));
 }
 
 template <int DT, int DK, int CTA_K, int ROT>
@@ -359,7 +426,8 @@ void launch_k(const QkArgs& a, hipStream_t stream) {
   dim3 grid(tiles, a.kv_heads, a.batch);
   quantize_k_kernel<DT, DK, CTA_K, ROT><<<grid, 128, 0, stream>>>(
       a.k, a.k_codes, a.k_scale, a.anchors, a.k_len, a.kv_heads, tiles * 4, a.k_stride_b,
-      a.k_stride_h, a.k_stride_n);
+      a.k_stride_h, a.k_stride_n,
+      rows_are_16_byte_aligned(a.k, a.k_stride_b, a.k_stride_h, a.k_stride_n, a.dtype));
 }
 
 template <int DT, int DK, int ROT>
