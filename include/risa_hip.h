@@ -45,12 +45,17 @@ int risa_abi_version(void);
  *   q_int8 [B,Hq,Lq,D], k_int8 [B,Hkv,Lk,D] contiguous.
  *   q_scale [B,Hq,ceil(Lq/128)*(D==256?64:32)], k_scale [B,Hkv,ceil(Lk/cta_k)*4].
  *   anchor_indices int32 [B,Hkv]: receives the anchor row or -1.
+  *   kv_permutation (nullable) int32 [B,Hkv,Lk]: key n is read from source token
+ *   kv_permutation[b,h,n] (the reference's fused gather, csrc/kernels/
+ *   quantize_gather.cu, bindings.cpp:195-272 permutation_ptr); anchors, codes
+ *   and scales are those of the gathered K.
  */
 int risa_quantize_qk(const void* q, void* q_int8, float* q_scale, const void* k, void* k_int8,
                      float* k_scale, int batch, int q_heads, int q_len, int kv_heads, int k_len,
                      int head_dim, int cta_k, int64_t q_stride_b, int64_t q_stride_h,
                      int64_t q_stride_n, int64_t k_stride_b, int64_t k_stride_h,
-                     int64_t k_stride_n, int input_dtype, int32_t* anchor_indices, void* stream);
+                     int64_t k_stride_n, int input_dtype, int32_t* anchor_indices,
+                     const int32_t* kv_permutation, void* stream);
 
 /*
  * V preparation.  Replaces launch_quantize_v (reference csrc/launchers.h:30-34,
@@ -62,6 +67,7 @@ int risa_quantize_qk(const void* q, void* q_int8, float* q_scale, const void* k,
  *   of the signed product) + 0x4B400000 (the bits of 1.5 * 2^23, which make the
  *   finished integer accumulator readable as a float); no reference counterpart,
  *   workspace of risa_quantize_v_workspace_bytes(...) bytes.
+  *   kv_permutation (nullable) int32 [B,Hkv,L] as for risa_quantize_qk.
  */
 size_t risa_quantize_v_workspace_bytes(int batch, int heads, int length, int head_dim,
                                        int midpoint_affine);
@@ -69,7 +75,7 @@ int risa_quantize_v(const void* v, void* out, float* scale, float* center, int32
                     void* workspace, size_t workspace_bytes, int batch, int heads, int length,
                     int head_dim, int padded_length, int cta_k, int64_t stride_b,
                     int64_t stride_h, int64_t stride_n, int input_dtype, int midpoint_affine,
-                    void* stream);
+                    const int32_t* kv_permutation, void* stream);
 
 /*
  * Zero-point terms (128 x tile sums) of an already packed V matrix (for callers that build packed V

@@ -29,7 +29,8 @@ int risa_quantize_qk(const void* q, void* q_int8, float* q_scale, const void* k,
                      float* k_scale, int batch, int q_heads, int q_len, int kv_heads, int k_len,
                      int head_dim, int cta_k, int64_t q_stride_b, int64_t q_stride_h,
                      int64_t q_stride_n, int64_t k_stride_b, int64_t k_stride_h,
-                     int64_t k_stride_n, int input_dtype, int32_t* anchor_indices, void* stream) {
+                     int64_t k_stride_n, int input_dtype, int32_t* anchor_indices,
+                     const int32_t* kv_permutation, void* stream) {
   using risa::fail;
   if (head_dim != 64 && head_dim != 128 && head_dim != 256)
     return fail("risa_quantize_qk: padded head_dim must be 64, 128, or 256");
@@ -56,6 +57,7 @@ int risa_quantize_qk(const void* q, void* q_int8, float* q_scale, const void* k,
   a.k_codes = static_cast<int8_t*>(k_int8);
   a.k_scale = k_scale;
   a.anchors = anchor_indices;
+  a.permutation = kv_permutation;
   a.batch = batch;
   a.q_heads = q_heads;
   a.q_len = q_len;
@@ -82,7 +84,7 @@ int risa_quantize_v(const void* v, void* out, float* scale, float* center, int32
                     void* workspace, size_t workspace_bytes, int batch, int heads, int length,
                     int head_dim, int padded_length, int cta_k, int64_t stride_b,
                     int64_t stride_h, int64_t stride_n, int input_dtype, int midpoint_affine,
-                    void* stream) {
+                    const int32_t* kv_permutation, void* stream) {
   using risa::fail;
   if (head_dim != 64 && head_dim != 128 && head_dim != 256)
     return fail("risa_quantize_v: padded head_dim must be 64, 128, or 256");
@@ -107,6 +109,7 @@ int risa_quantize_v(const void* v, void* out, float* scale, float* center, int32
   a.tile_sum = tile_sum;
   a.workspace = workspace;
   a.workspace_bytes = workspace_bytes;
+  a.permutation = kv_permutation;
   a.batch = batch;
   a.heads = heads;
   a.length = length;

@@ -19,6 +19,7 @@ struct QkArgs {
   int8_t* k_codes;
   float* k_scale;
   int* anchors;
+  const int32_t* permutation;  // [B,Hkv,Lk] source token of every key, or null
   int batch, q_heads, q_len, kv_heads, k_len, head_dim, cta_k, dtype;
   int64_t q_stride_b, q_stride_h, q_stride_n;
   int64_t k_stride_b, k_stride_h, k_stride_n;
@@ -45,6 +46,7 @@ struct ValueArgs {
   int32_t* tile_sum; // [B*H, padded/cta_k, D], 128 x sum of codes
   void* workspace;
   size_t workspace_bytes;
+  const int32_t* permutation;  // [B,H,L] source token of every value row, or null
   int batch, heads, length, head_dim, padded, cta_k, dtype;
   int64_t stride_b, stride_h, stride_n;
   bool midpoint_affine;

@@ -142,7 +142,8 @@ __device__ __forceinline__ float half_wave_max(float value) {
 template <int DT, int DK, int ROT, int NTOK, typename TokenOf>
 __device__ __forceinline__ void quantize_group(const void* in, int64_t in_base, int64_t stride_n,
                                                int8_t* out, float* scale_slot, int length, int sub,
-                                               const void* bias_row, bool wide, TokenOf token_of) {
+                                               const void* bias_row, bool wide, TokenOf token_of,
+                                               const int32_t* source = nullptr) {
   constexpr int BLOCKS = DK == 256 ? 2 : 1;   // 128-channel rotation blocks
   constexpr int GROUPS = DK == 64 ? 1 : 2;    // runs of four channels per lane and block
   constexpr int STEPS = NTOK / 2;
@@ -173,7 +174,9 @@ __device__ __forceinline__ void quantize_group(const void* in, int64_t in_base, 
   for (int i = 0; i < STEPS; ++i) {
     const int n = token_of(2 * i + row);
     if (n < length) {
-      load_row(in_base + static_cast<int64_t>(n) * stride_n, v[i]);
+      // with a permutation, token n of the gathered sequence is source row source[n]
+      const int from = source != nullptr ? source[n] : n;
+      load_row(in_base + static_cast<int64_t>(from) * stride_n, v[i]);
       if (bias_row != nullptr) {
 #pragma unroll
         for (int block = 0; block < BLOCKS; ++block)
@@ -271,7 +274,8 @@ __global__ __launch_bounds__(128) void quantize_k_kernel(const void* __restrict_
                                                          const int* __restrict__ anchors, int length,
                                                          int heads, int scales_per_head,
                                                          int64_t stride_b, int64_t stride_h,
-                                                         int64_t stride_n, int wide) {
+                                                         int64_t stride_n, int wide,
+                                                         const int32_t* __restrict__ permutation) {
   constexpr int NTOK = CTA_K / 4;
   const int tile = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
   const int sub = threadIdx.x & 31;
@@ -279,13 +283,15 @@ __global__ __launch_bounds__(128) void quantize_k_kernel(const void* __restrict_
   const int64_t in_base = static_cast<int64_t>(b) * stride_b + static_cast<int64_t>(h) * stride_h;
   const int64_t bh = static_cast<int64_t>(b) * heads + h;
   const int anchor = anchors[b * heads + h];
+  const int32_t* source = permutation != nullptr ? permutation + bh * length : nullptr;
   // element offset of the anchor row (subtracted from every key) when one was chosen
-  const int64_t anchor_offset = static_cast<int64_t>(anchor) * stride_n;
+  const int anchor_row = anchor >= 0 && source != nullptr ? source[anchor] : anchor;
+  const int64_t anchor_offset = static_cast<int64_t>(anchor_row) * stride_n;
   const int first = tile * CTA_K + group * 2;
   quantize_group<DT, DK, ROT, NTOK>(k, in_base, stride_n, codes + bh * length * DK,
                                     scales + bh * scales_per_head + tile * 4 + group, length, sub,
                                     anchor >= 0 ? &anchor_offset : nullptr, wide != 0,
-                                    [first](int i) { return first + (i >> 1) * 8 + (i & 1); });
+                                    [first](int i) { return first + (i >> 1) * 8 + (i & 1); }, source);
 }
 
 // ---------------------------------------------------------------------------
@@ -311,7 +317,8 @@ template <int DT>
 __global__ __launch_bounds__(128) void detect_anchor_kernel(const void* __restrict__ k,
                                                             int* __restrict__ anchors, int length,
                                                             int dim, int heads, int64_t stride_b,
-                                                            int64_t stride_h, int64_t stride_n) {
+                                                            int64_t stride_h, int64_t stride_n,
+                                                            const int32_t* __restrict__ permutation) {
   __shared__ float samples[kSamples * 256];
   __shared__ float seg_energy[4], seg_max[4], seg_dist[kSamples][4], seg_best_energy[4],
       seg_best_max[4];
@@ -322,7 +329,8 @@ __global__ __launch_bounds__(128) void detect_anchor_kernel(const void* __restri
   for (int index = tid; index < kSamples * dim; index += 128) {
     const int s = index / dim;
     const int c = index - s * dim;
-    const int64_t row = static_cast<int64_t>(s) * (length - 1) / (kSamples - 1);
+    int64_t row = static_cast<int64_t>(s) * (length - 1) / (kSamples - 1);
+    if (permutation != nullptr) row = permutation[(static_cast<int64_t>(b) * heads + h) * length + row];
     samples[index] = load1<DT>(k, base + row * stride_n + c);
   }
   __syncthreads();
@@ -427,7 +435,7 @@ void launch_k(const QkArgs& a, hipStream_t stream) {
   quantize_k_kernel<DT, DK, CTA_K, ROT><<<grid, 128, 0, stream>>>(
       a.k, a.k_codes, a.k_scale, a.anchors, a.k_len, a.kv_heads, tiles * 4, a.k_stride_b,
       a.k_stride_h, a.k_stride_n,
-      rows_are_16_byte_aligned(a.k, a.k_stride_b, a.k_stride_h, a.k_stride_n, a.dtype));
+      rows_are_16_byte_aligned(a.k, a.k_stride_b, a.k_stride_h, a.k_stride_n, a.dtype), a.permutation);
 }
 
 template <int DT, int DK, int ROT>
@@ -447,7 +455,7 @@ template <int DT> void launch_qk_dtype(const QkArgs& a, hipStream_t stream) {
   dim3 grid(a.kv_heads, a.batch);
   detect_anchor_kernel<DT><<<grid, 128, 0, stream>>>(a.k, a.anchors, a.k_len, a.head_dim,
                                                      a.kv_heads, a.k_stride_b, a.k_stride_h,
-                                                     a.k_stride_n);
+                                                     a.k_stride_n, a.permutation);
   const bool short_keys = a.k_len <= 256;
   if (a.head_dim == 64) {
     if (short_keys)

@@ -131,7 +131,8 @@ __global__ __launch_bounds__(256) void value_codes_kernel(const void* __restrict
                                                           const float* __restrict__ midpoint,
                                                           int length, int padded, int dim, int heads,
                                                           int64_t stride_b, int64_t stride_h,
-                                                          int64_t stride_n) {
+                                                          int64_t stride_n,
+                                                          const int32_t* __restrict__ permutation) {
   const int bh = blockIdx.y;
   const int b = bh / heads, h = bh - b * heads;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -153,8 +154,9 @@ __global__ __launch_bounds__(256) void value_codes_kernel(const void* __restrict
     for (int r = 0; r < 4; ++r) {
       const int n = n0 + r;
       if (n < length) {
+        const int from = permutation != nullptr ? permutation[static_cast<int64_t>(bh) * length + n] : n;
         float x[8];
-        load8<DT>(v, base + static_cast<int64_t>(n) * stride_n + octet * 8, x);
+        load8<DT>(v, base + static_cast<int64_t>(from) * stride_n + octet * 8, x);
 #pragma unroll
         for (int i = 0; i < 8; ++i) q[i][r] = quantize_s8((x[i] - mid[i]) * inv[i]);
       } else {
@@ -187,7 +189,8 @@ __global__ __launch_bounds__(256) void value_residual_kernel(const void* __restr
                                                              const float* __restrict__ midpoint,
                                                              int length, int dim, int heads,
                                                              int threads, int64_t stride_b,
-                                                             int64_t stride_h, int64_t stride_n) {
+                                                             int64_t stride_h, int64_t stride_n,
+                                                             const int32_t* __restrict__ permutation) {
   const int bh = blockIdx.y;
   const int b = bh / heads, h = bh - b * heads;
   const int octets = dim / 8;
@@ -203,8 +206,9 @@ __global__ __launch_bounds__(256) void value_residual_kernel(const void* __restr
     residual[i] = 0.0f;
   }
   for (int src = length - 1 - t; src >= 0; src -= threads) {
+    const int from = permutation != nullptr ? permutation[static_cast<int64_t>(bh) * length + src] : src;
     float x[8];
-    load8<DT>(v, base + static_cast<int64_t>(src) * stride_n + octet * 8, x);
+    load8<DT>(v, base + static_cast<int64_t>(from) * stride_n + octet * 8, x);
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       const float normalized = (x[i] - mid[i]) * inv[i];
@@ -319,11 +323,11 @@ template <int DT> int run(const ValueArgs& a, hipStream_t stream) {
   if (a.cta_k == 128) {
     value_codes_kernel<DT, 128><<<code_grid, 256, 0, stream>>>(
         a.v, a.codes, a.tile_sum, w.inverse, w.midpoint, a.length, a.padded, a.head_dim, a.heads,
-        a.stride_b, a.stride_h, a.stride_n);
+        a.stride_b, a.stride_h, a.stride_n, a.permutation);
   } else {
     value_codes_kernel<DT, 64><<<code_grid, 256, 0, stream>>>(
         a.v, a.codes, a.tile_sum, w.inverse, w.midpoint, a.length, a.padded, a.head_dim, a.heads,
-        a.stride_b, a.stride_h, a.stride_n);
+        a.stride_b, a.stride_h, a.stride_n, a.permutation);
   }
   if (a.midpoint_affine) {
     const int threads = summation_threads(a.length);
@@ -331,7 +335,7 @@ template <int DT> int run(const ValueArgs& a, hipStream_t stream) {
     dim3 residual_grid(threads / per_block, bh);
     value_residual_kernel<DT><<<residual_grid, 256, 0, stream>>>(
         a.v, w.partial, w.inverse, w.midpoint, a.length, a.head_dim, a.heads, threads, a.stride_b,
-        a.stride_h, a.stride_n);
+        a.stride_h, a.stride_n, a.permutation);
     value_center_kernel<<<(rows + 63) / 64, 64, 0, stream>>>(w.partial, w.inverse, w.midpoint,
                                                              a.center, rows, threads, a.length);
   }

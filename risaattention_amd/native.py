@@ -31,12 +31,12 @@ SIGNATURES = {
     "risa_abi_version": (_c_int, []),
     "risa_quantize_qk": (
         _c_int,
-        [_c_ptr] * 6 + [_c_int] * 7 + [_c_i64] * 6 + [_c_int, _c_ptr, _c_ptr],
+        [_c_ptr] * 6 + [_c_int] * 7 + [_c_i64] * 6 + [_c_int, _c_ptr, _c_ptr, _c_ptr],
     ),
     "risa_quantize_v_workspace_bytes": (_c_size, [_c_int] * 5),
     "risa_quantize_v": (
         _c_int,
-        [_c_ptr] * 6 + [_c_size] + [_c_int] * 6 + [_c_i64] * 3 + [_c_int, _c_int, _c_ptr],
+        [_c_ptr] * 6 + [_c_size] + [_c_int] * 6 + [_c_i64] * 3 + [_c_int, _c_int, _c_ptr, _c_ptr],
     ),
     "risa_value_tile_sums": (_c_int, [_c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr]),
     "risa_unpack_order": (None, [_c_ptr]),

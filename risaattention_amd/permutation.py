@@ -1,8 +1,10 @@
-"""Validated K/V token permutation, applied by an eager gather before quantisation.
+"""Validated K/V token permutation, fused into quantisation or applied eagerly.
 
 Counterpart of reference src/risa_attention/permutation.py:1-52.  The
-reference can fuse the gather into its BF16/D128 quantisers; this build always
-gathers eagerly, which gives the same packed tensors.
+reference fuses the gather into its BF16/D128 quantisers only; here the K, anchor
+and V kernels read through the permutation for every dtype and head dim.  As in
+the reference, ``return_lse`` (whose anchor correction reads K rows itself) and
+``fuse_gather=False`` take the eager gather; both routes give the same tensors.
 """
 
 from __future__ import annotations
@@ -52,5 +54,7 @@ def prepare_inputs(q, k, v, *, permutation, mask, causal, return_lse, fuse):
         raise ValueError("permutation must match K batch, heads, length, and device")
     if mask is not None or causal:
         raise ValueError("K/V permutation requires dense, unmasked, noncausal attention")
+    if fuse and not return_lse:
+        return q, k, v, perm
     index = perm.long()[..., None].expand_as(k)
-    return q, k.gather(2, index), v.gather(2, index)
+    return q, k.gather(2, index), v.gather(2, index), None

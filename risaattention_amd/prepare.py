@@ -61,11 +61,14 @@ def resolve_scale(scale: float | None, head_dim: int) -> float:
     return value
 
 
-def quantize_inputs(q, k, v, attn_mask, scale, use_midpoint_affine: bool) -> PreparedBuffers:
+def quantize_inputs(q, k, v, attn_mask, scale, use_midpoint_affine: bool,
+                    kv_permutation: torch.Tensor | None = None) -> PreparedBuffers:
     """Allocate the packed buffers and enqueue the Q/K and V preparation kernels.
 
     ``q``, ``k``, ``v`` are validated; ``attn_mask`` is already broadcast (its
-    query stride decides the key tile size).
+    query stride decides the key tile size).  ``kv_permutation`` (int32
+    ``[B,Hkv,Lk]``) makes the K and V kernels read key ``n`` from source token
+    ``kv_permutation[b,h,n]``: the gather fused into quantisation.
     """
     lib = native.library()
     original_dim = q.shape[-1]
@@ -104,7 +107,7 @@ def quantize_inputs(q, k, v, attn_mask, scale, use_midpoint_affine: bool) -> Pre
             k.data_ptr(), k_codes.data_ptr(), k_scale.data_ptr(),
             batch, q_heads, q_len, kv_heads, k_len, dim, cta_k,
             q.stride(0), q.stride(1), q.stride(2), k.stride(0), k.stride(1), k.stride(2),
-            code, anchors.data_ptr(), stream,
+            code, anchors.data_ptr(), native.pointer(kv_permutation), stream,
         )
     )
     native.check(
@@ -112,7 +115,8 @@ def quantize_inputs(q, k, v, attn_mask, scale, use_midpoint_affine: bool) -> Pre
             v.data_ptr(), v_codes.data_ptr(), v_scale.data_ptr(), v_center.data_ptr(),
             v_tile_sum.data_ptr(), workspace.data_ptr(), workspace.numel(),
             batch, kv_heads, k_len, dim, padded, cta_k,
-            v.stride(0), v.stride(1), v.stride(2), code, int(use_midpoint_affine), stream,
+            v.stride(0), v.stride(1), v.stride(2), code, int(use_midpoint_affine),
+            native.pointer(kv_permutation), stream,
         )
     )
     return PreparedBuffers(q_codes, k_codes, v_codes, q_scale, k_scale, v_scale, v_center,
@@ -154,18 +158,21 @@ def prequantize_int8_attention(
     :func:`int8_attention_from_prequantized`.  Everything is enqueued on the
     current stream without host synchronisation.  ``return_lse=True`` also
     stores the K-anchor logit offset so that LSE values of different key
-    windows can be merged.  ``kv_permutation`` gathers K and V eagerly before
-    quantisation (``fuse_gather`` is accepted for compatibility).
+    windows can be merged.  ``kv_permutation`` reorders the keys and values; with
+    ``fuse_gather`` (and no LSE) the quantisation kernels read through it,
+    otherwise K and V are gathered eagerly first.  Both give the same tensors.
     """
     attn_mask = validate_inputs(q, k, v, attn_mask)
+    fused_permutation = None
     if kv_permutation is not None:
         from .permutation import prepare_inputs
 
-        q, k, v = prepare_inputs(q, k, v, permutation=kv_permutation, mask=attn_mask,
-                                 causal=is_causal, return_lse=return_lse, fuse=fuse_gather)
+        q, k, v, fused_permutation = prepare_inputs(
+            q, k, v, permutation=kv_permutation, mask=attn_mask, causal=is_causal,
+            return_lse=return_lse, fuse=fuse_gather)
     use_midpoint_affine = uses_centered_values(v_quantization)
     original_dim, input_dtype = q.shape[-1], q.dtype
-    buffers = quantize_inputs(q, k, v, attn_mask, scale, use_midpoint_affine)
+    buffers = quantize_inputs(q, k, v, attn_mask, scale, use_midpoint_affine, fused_permutation)
     shift = lse_shift(buffers, input_dtype) if return_lse else None
     return PrequantizedInt8Attention(
         q=buffers.q_codes,

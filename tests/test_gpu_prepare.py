@@ -107,3 +107,38 @@ def test_lse_shift_closed_form(risa, dtype, dim):
     reference = (q.float() * selected.repeat_interleave(2, 1)).sum(-1) * dim**-0.5
     torch.testing.assert_close(out, reference, rtol=2e-5, atol=5e-6)
     assert torch.count_nonzero(out[0, :2]) == 0
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("layout", ["hnd", "nhd", "interleaved"])
+@pytest.mark.parametrize("mode", ["absmax", "midpoint_affine"])
+def test_fused_permutation_matches_materialized_gather(risa, dtype, layout, mode):
+    """reference tests/cuda/test_value_quantization.py:55-72, extended to K, the anchor,
+    both V modes and the accumulator seeds: reading through the permutation inside
+    the quantisation kernels gives the tensors of an eager gather, bit for bit."""
+    torch.manual_seed(5)
+    q = torch.randn(1, 4, 17, 128, device="cuda", dtype=dtype)
+    k = torch.randn(1, 2, 2049, 128, device="cuda", dtype=dtype) * 0.1 + 3.0  # the anchor fires
+    v = torch.randn(1, 2, 2049, 128, device="cuda", dtype=dtype) + 1.5
+    if layout == "nhd":
+        v = v.transpose(1, 2).contiguous().transpose(1, 2)
+        k = k.transpose(1, 2).contiguous().transpose(1, 2)
+    elif layout == "interleaved":
+        storage = torch.empty(1, 2049, 3, 2, 128, device="cuda", dtype=dtype)
+        v = storage[:, :, 1].transpose(1, 2).copy_(v)
+    indices = torch.stack([torch.randperm(2049, device="cuda") for _ in range(2)])[None]
+    permutation = risa.prepare_kv_permutation(indices)
+    fused = risa.prequantize_int8_attention(q, k, v, kv_permutation=permutation, fuse_gather=True,
+                                            v_quantization=mode)
+    eager = risa.prequantize_int8_attention(q, k, v, kv_permutation=permutation, fuse_gather=False,
+                                            v_quantization=mode)
+    assert fused.kv_permuted and eager.kv_permuted
+    for attribute in ("q", "q_scale", "k", "k_scale", "v", "v_scale", "v_center", "v_tile_sum"):
+        assert torch.equal(getattr(fused, attribute), getattr(eager, attribute)), attribute
+    # and the eager route is the plain path on gathered tensors
+    index = indices[..., None].expand_as(k)
+    plain = risa.prequantize_int8_attention(q, k.gather(2, index), v.gather(2, index), v_quantization=mode)
+    assert torch.equal(plain.k, fused.k) and torch.equal(plain.v, fused.v)
+    out = risa.int8_attention(q, k, v, kv_permutation=permutation, v_quantization=mode)
+    expected = risa.int8_attention_from_prequantized(plain)
+    assert torch.equal(out, expected)
