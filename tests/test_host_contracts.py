@@ -36,7 +36,7 @@ def test_host_only_entry_points():
     assert 0 < small < large
     # rejected calls report through risa_last_error and launch nothing
     assert lib.risa_quantize_qk(None, None, None, None, None, None, 1, 1, 1, 1, 1, 96, 64,
-                                0, 0, 0, 0, 0, 0, 2, None, None) != 0
+                                0, 0, 0, 0, 0, 0, 2, None, None, None) != 0
     assert b"head_dim" in lib.risa_last_error()
     with pytest.raises(RuntimeError, match="head_dim"):
         native.check(1)
