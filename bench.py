@@ -127,7 +127,7 @@ def workload_masked(torch, risa, args, device):
         key_padding = torch.ones(batch, 1, 1, k_len, dtype=torch.bool, device=device)
         key_padding[1, ..., int(k_len * 0.9):] = False
         generator = torch.Generator(device=device).manual_seed(1)
-        bias = torch.randn(batch, 1, q_len, k_len, generator=generator, device=device).bfloat16()
+        bias = torch.randn(batch, 1, q_len, k_len, generator=generator, device=device)  # float32
         rowmask = torch.ones(batch, 1, q_len, k_len, dtype=torch.bool, device=device)
         rowmask[0, :, :7] = False  # fully masked rows
         variants = {
@@ -149,13 +149,14 @@ def clustered_inputs(torch, length, groups, seed, device):
     dim = SHAPE["head_dim"]
     per_group = length // groups
 
-    def clustered(heads):
-        centroids = torch.randn(1, heads, groups, dim, generator=generator, device=device) * 3.0
-        tokens = centroids.repeat_interleave(per_group, 2)
-        return tokens + torch.randn(tokens.shape, generator=generator, device=device)
-
-    q = clustered(SHAPE["q_heads"])
-    k = clustered(SHAPE["kv_heads"])
+    # one centroid per (KV head, token group), shared by K and by the query heads of
+    # that KV head's group, plus unit noise (reference benchmarks/sparse.py:30-60)
+    kv_heads, q_heads = SHAPE["kv_heads"], SHAPE["q_heads"]
+    centroids = torch.randn(1, kv_heads, groups, dim, generator=generator, device=device) * 3.0
+    tokens = centroids.repeat_interleave(per_group, 2)
+    q = tokens.repeat_interleave(q_heads // kv_heads, 1)
+    q = q + torch.randn(q.shape, generator=generator, device=device)
+    k = tokens + torch.randn(tokens.shape, generator=generator, device=device)
     v = torch.randn(1, SHAPE["kv_heads"], length, dim, generator=generator, device=device)
     return q, k, v, generator
 
