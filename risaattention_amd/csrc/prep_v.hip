@@ -10,7 +10,7 @@
 // The reference runs one block per (batch, head, 8 channels) that walks the whole
 // sequence twice; at 32K tokens and four KV heads that is 64 blocks.  Here the
 // sequence axis is split across the grid:
-//   1. value_range_kernel     partial min/max per (1024-token chunk, channel)
+//   1. value_range_kernel     partial min/max per (wavefront chunk of 64+ tokens, channel)
 //   2. value_params_kernel    scale, midpoint and reciprocal per channel
 //   3. value_codes_kernel     codes + packed transposed store + tile sums
 //   4. value_residual_kernel  (affine) per-summation-thread residual sums in the
@@ -27,7 +27,15 @@
 namespace risa {
 namespace {
 
-constexpr int kChunk = 1024;  // tokens per block of the range pass
+// The range pass gives every wavefront tokens_per_wave(length) consecutive tokens:
+// 64 up to 32768 tokens, then whatever keeps the number of partial ranges per
+// (batch, head) at 512, which one wavefront of the parameter pass reduces in eight
+// loads per lane.
+__host__ __device__ inline int tokens_per_wave(int length) { return 64 * ((length + 64 * 512 - 1) / (64 * 512)); }
+__host__ __device__ inline int range_chunks(int length) {
+  const int per_wave = tokens_per_wave(length);
+  return (length + per_wave - 1) / per_wave;
+}
 
 __host__ __device__ inline int summation_threads(int length) { return length <= 256 ? 128 : 512; }
 
@@ -39,6 +47,11 @@ __device__ __forceinline__ int first_token_of_positions(int p0) {
   return (p0 & ~31) + 8 * b + 4 * h;
 }
 
+// grid (ceil(chunks/4), B*H), 256 threads: one wavefront per chunk of
+// tokens_per_wave(length) tokens.  A token row is dim/8 lanes wide (8 channels =
+// 16 bytes of a 16-bit input per lane), so every load instruction of the wavefront
+// covers whole consecutive rows; the lanes holding the same channels are combined
+// with xor shuffles at the end.  min/max do not depend on the order.
 template <int DT, bool AFFINE>
 __global__ __launch_bounds__(256) void value_range_kernel(const void* __restrict__ v,
                                                           float* __restrict__ part_max,
@@ -46,83 +59,114 @@ __global__ __launch_bounds__(256) void value_range_kernel(const void* __restrict
                                                           int dim, int heads, int chunks,
                                                           int64_t stride_b, int64_t stride_h,
                                                           int64_t stride_n) {
-  const int chunk = blockIdx.x, bh = blockIdx.y;
+  const int bh = blockIdx.y;
   const int b = bh / heads, h = bh - b * heads;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int64_t base = static_cast<int64_t>(b) * stride_b + static_cast<int64_t>(h) * stride_h;
+  const int chunk = blockIdx.x * 4 + wave;
+  if (chunk >= chunks) return;
   const int octets = dim / 8;
-  for (int octet = wave; octet < octets; octet += 4) {
-    float mx[8], mn[8];
+  const int octet = lane % octets, row = lane / octets, rows_per_load = 64 / octets;
+  const int per_wave = tokens_per_wave(length);
+  const int64_t base = static_cast<int64_t>(b) * stride_b + static_cast<int64_t>(h) * stride_h;
+  float mx[8], mn[8];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      mx[i] = AFFINE ? -FLT_MAX : 0.0f;
-      mn[i] = FLT_MAX;
-    }
-    for (int pass = 0; pass < kChunk / 256; ++pass) {
-      const int n0 = chunk * kChunk + pass * 256 + lane * 4;
+  for (int i = 0; i < 8; ++i) {
+    mx[i] = AFFINE ? -FLT_MAX : 0.0f;
+    mn[i] = FLT_MAX;
+  }
+  const int first = chunk * per_wave;
+#pragma unroll 8
+  for (int t = row; t < per_wave; t += rows_per_load) {
+    const int n = first + t;
+    if (n < length) {
+      float x[8];
+      load8<DT>(v, base + static_cast<int64_t>(n) * stride_n + octet * 8, x);
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const int n = n0 + r;
-        if (n < length) {
-          float x[8];
-          load8<DT>(v, base + static_cast<int64_t>(n) * stride_n + octet * 8, x);
-#pragma unroll
-          for (int i = 0; i < 8; ++i) {
-            if constexpr (AFFINE) {
-              mx[i] = __builtin_fmaxf(mx[i], x[i]);
-              mn[i] = __builtin_fminf(mn[i], x[i]);
-            } else {
-              mx[i] = __builtin_fmaxf(mx[i], __builtin_fabsf(x[i]));
-            }
-          }
+      for (int i = 0; i < 8; ++i) {
+        if constexpr (AFFINE) {
+          mx[i] = __builtin_fmaxf(mx[i], x[i]);
+          mn[i] = __builtin_fminf(mn[i], x[i]);
+        } else {
+          mx[i] = __builtin_fmaxf(mx[i], __builtin_fabsf(x[i]));
         }
       }
     }
+  }
+  for (int offset = octets; offset < 64; offset <<= 1) {
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-#pragma unroll
-      for (int offset = 32; offset > 0; offset >>= 1) {
-        mx[i] = __builtin_fmaxf(mx[i], __shfl_xor(mx[i], offset));
-        if constexpr (AFFINE) mn[i] = __builtin_fminf(mn[i], __shfl_xor(mn[i], offset));
-      }
+      mx[i] = __builtin_fmaxf(mx[i], __shfl_xor(mx[i], offset));
+      if constexpr (AFFINE) mn[i] = __builtin_fminf(mn[i], __shfl_xor(mn[i], offset));
     }
-    if (lane == 0) {
-      const int64_t slot = (static_cast<int64_t>(bh) * chunks + chunk) * dim + octet * 8;
+  }
+  if (lane < octets) {
+    const int64_t slot = (static_cast<int64_t>(bh) * chunks + chunk) * dim + octet * 8;
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        part_max[slot + i] = mx[i];
-        if constexpr (AFFINE) part_min[slot + i] = mn[i];
-      }
+    for (int i = 0; i < 8; ++i) {
+      part_max[slot + i] = mx[i];
+      if constexpr (AFFINE) part_min[slot + i] = mn[i];
     }
   }
 }
 
+// grid (ceil(B*H*dim/8 / 4)), 256 threads: one wavefront per (batch, head, 8
+// channels); lanes stride over the partial ranges, xor shuffles combine them.
 template <bool AFFINE>
-__global__ void value_params_kernel(const float* __restrict__ part_max,
-                                    const float* __restrict__ part_min, float* __restrict__ scale,
-                                    float* __restrict__ center, float* __restrict__ inverse,
-                                    float* __restrict__ midpoint, int dim, int chunks, int rows) {
-  const int row = blockIdx.x * blockDim.x + threadIdx.x;  // (b*H + h)*D + c
-  if (row >= rows) return;
-  const int bh = row / dim, c = row - bh * dim;
-  float mx = AFFINE ? -FLT_MAX : 0.0f, mn = FLT_MAX;
-  for (int chunk = 0; chunk < chunks; ++chunk) {
-    const int64_t slot = (static_cast<int64_t>(bh) * chunks + chunk) * dim + c;
-    mx = __builtin_fmaxf(mx, part_max[slot]);
-    if constexpr (AFFINE) mn = __builtin_fminf(mn, part_min[slot]);
+__global__ __launch_bounds__(256) void value_params_kernel(const float* __restrict__ part_max,
+                                                           const float* __restrict__ part_min,
+                                                           float* __restrict__ scale,
+                                                           float* __restrict__ center,
+                                                           float* __restrict__ inverse,
+                                                           float* __restrict__ midpoint, int dim,
+                                                           int chunks, int groups) {
+  const int lane = threadIdx.x & 63;
+  const int group = blockIdx.x * 4 + (threadIdx.x >> 6);  // (b*H + h) * dim/8 + octet
+  if (group >= groups) return;
+  const int octets = dim / 8;
+  const int bh = group / octets, octet = group - bh * octets;
+  float mx[8], mn[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    mx[i] = AFFINE ? -FLT_MAX : 0.0f;
+    mn[i] = FLT_MAX;
   }
-  const float mid = AFFINE ? 0.5f * (mn + mx) : 0.0f;
-  const float radius = AFFINE ? 0.5f * (mx - mn) : mx;
-  const float sc = __builtin_fmaxf(radius * (1.0f / 127.0f), 1e-12f);
-  scale[row] = sc;
-  inverse[row] = 1.0f / sc;
-  midpoint[row] = mid;
-  if constexpr (!AFFINE) center[row] = 0.0f;
+  for (int chunk = lane; chunk < chunks; chunk += 64) {
+    const int64_t slot = (static_cast<int64_t>(bh) * chunks + chunk) * dim + octet * 8;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      mx[i] = __builtin_fmaxf(mx[i], part_max[slot + i]);
+      if constexpr (AFFINE) mn[i] = __builtin_fminf(mn[i], part_min[slot + i]);
+    }
+  }
+#pragma unroll
+  for (int offset = 32; offset > 0; offset >>= 1) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      mx[i] = __builtin_fmaxf(mx[i], __shfl_xor(mx[i], offset));
+      if constexpr (AFFINE) mn[i] = __builtin_fminf(mn[i], __shfl_xor(mn[i], offset));
+    }
+  }
+  if (lane < 8) {
+    const int row = group * 8 + lane;
+    float hi = mx[0], lo = mn[0];
+#pragma unroll
+    for (int i = 1; i < 8; ++i) {
+      hi = lane == i ? mx[i] : hi;
+      lo = lane == i ? mn[i] : lo;
+    }
+    const float mid = AFFINE ? 0.5f * (lo + hi) : 0.0f;
+    const float radius = AFFINE ? 0.5f * (hi - lo) : hi;
+    const float sc = __builtin_fmaxf(radius * (1.0f / 127.0f), 1e-12f);
+    scale[row] = sc;
+    inverse[row] = 1.0f / sc;
+    midpoint[row] = mid;
+    if constexpr (!AFFINE) center[row] = 0.0f;
+  }
 }
 
-// grid (ceil(padded/256), B*H), 256 threads.  Lane l of every wave owns the four
-// packed positions 256*blockIdx.x + 4*l .. +3 (four consecutive tokens) and the
-// wave iterates over groups of eight channels.
+// grid (ceil(padded/256), B*H, dim/32), 256 threads.  Lane l of every wave owns the
+// four packed positions 256*blockIdx.x + 4*l .. +3 (four consecutive tokens); wave
+// w of the workgroup takes the eight channels 32*blockIdx.z + 8*w .. +7.
 template <int DT, int CTA_K>
 __global__ __launch_bounds__(256) void value_codes_kernel(const void* __restrict__ v,
                                                           int8_t* __restrict__ codes,
@@ -139,9 +183,9 @@ __global__ __launch_bounds__(256) void value_codes_kernel(const void* __restrict
   const int p0 = blockIdx.x * 256 + lane * 4;
   const int n0 = first_token_of_positions(p0);
   const int64_t base = static_cast<int64_t>(b) * stride_b + static_cast<int64_t>(h) * stride_h;
-  const int octets = dim / 8;
   const int tiles = padded / CTA_K;
-  for (int octet = wave; octet < octets; octet += 4) {
+  {
+    const int octet = blockIdx.z * 4 + wave;
     const int64_t row0 = static_cast<int64_t>(bh) * dim + octet * 8;
     float inv[8], mid[8];
 #pragma unroll
@@ -281,7 +325,7 @@ struct Workspace {
 
 Workspace carve(void* base, int batch, int heads, int length, int dim, bool affine) {
   const size_t bh = static_cast<size_t>(batch) * heads;
-  const size_t chunks = (length + kChunk - 1) / kChunk;
+  const size_t chunks = range_chunks(length);
   const size_t rows = bh * dim;
   float* p = static_cast<float*>(base);
   Workspace w{};
@@ -303,23 +347,24 @@ Workspace carve(void* base, int batch, int heads, int length, int dim, bool affi
 template <int DT> int run(const ValueArgs& a, hipStream_t stream) {
   const Workspace w = carve(a.workspace, a.batch, a.heads, a.length, a.head_dim, a.midpoint_affine);
   const int bh = a.batch * a.heads;
-  const int chunks = (a.length + kChunk - 1) / kChunk;
+  const int chunks = range_chunks(a.length);
   const int rows = bh * a.head_dim;
-  dim3 range_grid(chunks, bh);
+  const int groups = rows / 8;
+  dim3 range_grid((chunks + 3) / 4, bh);
   if (a.midpoint_affine) {
     value_range_kernel<DT, true><<<range_grid, 256, 0, stream>>>(
         a.v, w.part_max, w.part_min, a.length, a.head_dim, a.heads, chunks, a.stride_b, a.stride_h,
         a.stride_n);
-    value_params_kernel<true><<<(rows + 255) / 256, 256, 0, stream>>>(
-        w.part_max, w.part_min, a.scale, a.center, w.inverse, w.midpoint, a.head_dim, chunks, rows);
+    value_params_kernel<true><<<(groups + 3) / 4, 256, 0, stream>>>(
+        w.part_max, w.part_min, a.scale, a.center, w.inverse, w.midpoint, a.head_dim, chunks, groups);
   } else {
     value_range_kernel<DT, false><<<range_grid, 256, 0, stream>>>(
         a.v, w.part_max, w.part_min, a.length, a.head_dim, a.heads, chunks, a.stride_b, a.stride_h,
         a.stride_n);
-    value_params_kernel<false><<<(rows + 255) / 256, 256, 0, stream>>>(
-        w.part_max, w.part_min, a.scale, a.center, w.inverse, w.midpoint, a.head_dim, chunks, rows);
+    value_params_kernel<false><<<(groups + 3) / 4, 256, 0, stream>>>(
+        w.part_max, w.part_min, a.scale, a.center, w.inverse, w.midpoint, a.head_dim, chunks, groups);
   }
-  dim3 code_grid((a.padded + 255) / 256, bh);
+  dim3 code_grid((a.padded + 255) / 256, bh, a.head_dim / 32);
   if (a.cta_k == 128) {
     value_codes_kernel<DT, 128><<<code_grid, 256, 0, stream>>>(
         a.v, a.codes, a.tile_sum, w.inverse, w.midpoint, a.length, a.padded, a.head_dim, a.heads,
