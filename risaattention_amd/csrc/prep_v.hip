@@ -167,7 +167,25 @@ __global__ __launch_bounds__(256) void value_params_kernel(const float* __restri
 // grid (ceil(padded/256), B*H, dim/32), 256 threads.  Lane l of every wave owns the
 // four packed positions 256*blockIdx.x + 4*l .. +3 (four consecutive tokens); wave
 // w of the workgroup takes the eight channels 32*blockIdx.z + 8*w .. +7.
-template <int DT, int CTA_K>
+//
+// PARAMS says where the per-channel scale and midpoint come from: kParamsStored reads
+// what value_params_kernel left; kParamsAbsmax / kParamsAffine reduce the partial
+// ranges (at most 64 of them, one per lane) inside every wavefront, which saves a
+// launch for short sequences; the workgroups of the first 256 positions also store
+// the parameters for the kernels that follow.
+constexpr int kParamsStored = 0, kParamsAbsmax = 1, kParamsAffine = 2;
+
+struct FusedParams {
+  const float* part_max;
+  const float* part_min;
+  float* scale;
+  float* center;
+  float* inverse;
+  float* midpoint;
+  int chunks;
+};
+
+template <int DT, int CTA_K, int PARAMS>
 __global__ __launch_bounds__(256) void value_codes_kernel(const void* __restrict__ v,
                                                           int8_t* __restrict__ codes,
                                                           int32_t* __restrict__ tile_sum,
@@ -176,7 +194,8 @@ __global__ __launch_bounds__(256) void value_codes_kernel(const void* __restrict
                                                           int length, int padded, int dim, int heads,
                                                           int64_t stride_b, int64_t stride_h,
                                                           int64_t stride_n,
-                                                          const int32_t* __restrict__ permutation) {
+                                                          const int32_t* __restrict__ permutation,
+                                                          FusedParams fused) {
   const int bh = blockIdx.y;
   const int b = bh / heads, h = bh - b * heads;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -188,10 +207,49 @@ __global__ __launch_bounds__(256) void value_codes_kernel(const void* __restrict
     const int octet = blockIdx.z * 4 + wave;
     const int64_t row0 = static_cast<int64_t>(bh) * dim + octet * 8;
     float inv[8], mid[8];
+    if constexpr (PARAMS == kParamsStored) {
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      inv[i] = inverse[row0 + i];
-      mid[i] = midpoint[row0 + i];
+      for (int i = 0; i < 8; ++i) {
+        inv[i] = inverse[row0 + i];
+        mid[i] = midpoint[row0 + i];
+      }
+    } else {
+      constexpr bool AFFINE = PARAMS == kParamsAffine;
+      float mx[8], mn[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        mx[i] = AFFINE ? -FLT_MAX : 0.0f;
+        mn[i] = FLT_MAX;
+      }
+      if (lane < fused.chunks) {
+        const int64_t slot = (static_cast<int64_t>(bh) * fused.chunks + lane) * dim + octet * 8;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          mx[i] = fused.part_max[slot + i];
+          if constexpr (AFFINE) mn[i] = fused.part_min[slot + i];
+        }
+      }
+#pragma unroll
+      for (int offset = 32; offset > 0; offset >>= 1) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          mx[i] = __builtin_fmaxf(mx[i], __shfl_xor(mx[i], offset));
+          if constexpr (AFFINE) mn[i] = __builtin_fminf(mn[i], __shfl_xor(mn[i], offset));
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        mid[i] = AFFINE ? 0.5f * (mn[i] + mx[i]) : 0.0f;
+        const float radius = AFFINE ? 0.5f * (mx[i] - mn[i]) : mx[i];
+        const float sc = __builtin_fmaxf(radius * (1.0f / 127.0f), 1e-12f);
+        inv[i] = 1.0f / sc;
+        if (blockIdx.x == 0 && lane == i) {
+          fused.scale[row0 + i] = sc;
+          fused.inverse[row0 + i] = inv[i];
+          fused.midpoint[row0 + i] = mid[i];
+          if constexpr (!AFFINE) fused.center[row0 + i] = 0.0f;
+        }
+      }
     }
     int q[8][4];
 #pragma unroll
@@ -351,29 +409,46 @@ template <int DT> int run(const ValueArgs& a, hipStream_t stream) {
   const int rows = bh * a.head_dim;
   const int groups = rows / 8;
   dim3 range_grid((chunks + 3) / 4, bh);
+  // At most 64 partial ranges (sequences up to 4096 tokens): the code pass reduces
+  // them itself and no separate parameter launch is needed.
+  const bool fuse_params = chunks <= 64;
+  const FusedParams fused{w.part_max, w.part_min, a.scale, a.center, w.inverse, w.midpoint, chunks};
   if (a.midpoint_affine) {
     value_range_kernel<DT, true><<<range_grid, 256, 0, stream>>>(
         a.v, w.part_max, w.part_min, a.length, a.head_dim, a.heads, chunks, a.stride_b, a.stride_h,
         a.stride_n);
-    value_params_kernel<true><<<(groups + 3) / 4, 256, 0, stream>>>(
-        w.part_max, w.part_min, a.scale, a.center, w.inverse, w.midpoint, a.head_dim, chunks, groups);
+    if (!fuse_params)
+      value_params_kernel<true><<<(groups + 3) / 4, 256, 0, stream>>>(
+          w.part_max, w.part_min, a.scale, a.center, w.inverse, w.midpoint, a.head_dim, chunks, groups);
   } else {
     value_range_kernel<DT, false><<<range_grid, 256, 0, stream>>>(
         a.v, w.part_max, w.part_min, a.length, a.head_dim, a.heads, chunks, a.stride_b, a.stride_h,
         a.stride_n);
-    value_params_kernel<false><<<(groups + 3) / 4, 256, 0, stream>>>(
-        w.part_max, w.part_min, a.scale, a.center, w.inverse, w.midpoint, a.head_dim, chunks, groups);
+    if (!fuse_params)
+      value_params_kernel<false><<<(groups + 3) / 4, 256, 0, stream>>>(
+          w.part_max, w.part_min, a.scale, a.center, w.inverse, w.midpoint, a.head_dim, chunks, groups);
   }
   dim3 code_grid((a.padded + 255) / 256, bh, a.head_dim / 32);
+#define RISA_CODES(TILE, PARAMS)                                                                   \
+  value_codes_kernel<DT, TILE, PARAMS><<<code_grid, 256, 0, stream>>>(                             \
+      a.v, a.codes, a.tile_sum, w.inverse, w.midpoint, a.length, a.padded, a.head_dim, a.heads,    \
+      a.stride_b, a.stride_h, a.stride_n, a.permutation, fused)
   if (a.cta_k == 128) {
-    value_codes_kernel<DT, 128><<<code_grid, 256, 0, stream>>>(
-        a.v, a.codes, a.tile_sum, w.inverse, w.midpoint, a.length, a.padded, a.head_dim, a.heads,
-        a.stride_b, a.stride_h, a.stride_n, a.permutation);
+    if (!fuse_params)
+      RISA_CODES(128, kParamsStored);
+    else if (a.midpoint_affine)
+      RISA_CODES(128, kParamsAffine);
+    else
+      RISA_CODES(128, kParamsAbsmax);
   } else {
-    value_codes_kernel<DT, 64><<<code_grid, 256, 0, stream>>>(
-        a.v, a.codes, a.tile_sum, w.inverse, w.midpoint, a.length, a.padded, a.head_dim, a.heads,
-        a.stride_b, a.stride_h, a.stride_n, a.permutation);
+    if (!fuse_params)
+      RISA_CODES(64, kParamsStored);
+    else if (a.midpoint_affine)
+      RISA_CODES(64, kParamsAffine);
+    else
+      RISA_CODES(64, kParamsAbsmax);
   }
+#undef RISA_CODES
   if (a.midpoint_affine) {
     const int threads = summation_threads(a.length);
     const int per_block = 256 / (a.head_dim / 8);
