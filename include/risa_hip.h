@@ -129,6 +129,29 @@ int risa_attention(const void* q_int8, const void* k_int8, const void* v_int8, v
                    void* stream);
 
 /*
+ * Quantise and attend in one call.  Replaces risa_sdpa (reference
+ * csrc/bindings.cpp:497-616): the calls above back to back on one stream, with
+ * every intermediate buffer (codes, scales, accumulator seeds, anchors, the V
+ * workspace, the key bias row and key tile list of a key-only mask) carved from
+ * one caller-provided workspace of risa_sdpa_workspace_bytes(...) bytes (256-byte
+ * aligned).  q/k/v are [B,H,L,D] with element strides, head_dim 64, 128 or 256;
+ * out and the mask as for risa_attention; mask_batch / mask_heads are the mask's
+ * own extents (1 where it broadcasts).  key_only_mask in the size query says
+ * whether a mask with query stride 0 will be passed.
+ */
+size_t risa_sdpa_workspace_bytes(int batch, int q_heads, int q_len, int kv_heads, int k_len,
+                                 int head_dim, int cta_k, int midpoint_affine, int key_only_mask);
+int risa_sdpa(const void* q, const void* k, const void* v, void* out, void* workspace,
+              size_t workspace_bytes, int batch, int q_heads, int q_len, int kv_heads, int k_len,
+              int head_dim, int cta_k, int64_t q_stride_b, int64_t q_stride_h, int64_t q_stride_n,
+              int64_t k_stride_b, int64_t k_stride_h, int64_t k_stride_n, int64_t v_stride_b,
+              int64_t v_stride_h, int64_t v_stride_n, int64_t out_stride_b, int64_t out_stride_n,
+              int64_t out_stride_h, float sm_scale, int input_dtype, int output_dtype,
+              int midpoint_affine, const void* mask, int64_t mask_stride_b, int64_t mask_stride_h,
+              int64_t mask_stride_q, int64_t mask_stride_k, int mask_dtype, int mask_batch,
+              int mask_heads, int is_causal, void* stream);
+
+/*
  * Retained-mass selection over masses already sorted in descending order.
  * Replaces launch_select_retained_mass and retained_mass_selector_workspace_size
  * (reference csrc/launchers.h:56-63, csrc/kernels/sparse_selection.cu:129-159).

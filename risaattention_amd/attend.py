@@ -20,9 +20,10 @@ from .policy import (
     UNAVAILABLE,
     is_available,
     mask_signature,
+    select_key_block_size,
     validate_inputs,
 )
-from .prepare import quantize_inputs
+from .prepare import pad_head_dim, resolve_scale
 from .types import PrequantizedInt8Attention, RetainedMassPattern
 
 
@@ -170,22 +171,41 @@ def execute_dense_attention(
     use_midpoint_affine: bool = False,
     is_causal: bool = False,
 ) -> torch.Tensor:
-    """Quantize and attend in one call; buffers live only for the call."""
+    """Quantize and attend in one native call; the intermediate buffers are sections of
+    one workspace that lives only for the call (reference _execution.py:28-134 over
+    ``_C.risa_sdpa``)."""
     attn_mask = validate_inputs(q, k, v, attn_mask)
     original_dim, input_dtype = q.shape[-1], q.dtype
-    buffers = quantize_inputs(q, k, v, attn_mask, scale, use_midpoint_affine)
+    q, k, v, dim = pad_head_dim(q, k, v)
+    attention_scale = resolve_scale(scale, original_dim)
     batch, q_heads, q_len, _ = q.shape
-    output = torch.empty(batch, q_heads, q_len, buffers.kernel_dim,
-                         dtype=output_dtype_for(input_dtype), device=q.device)
-    tiles = prepare_key_mask_tiles(attn_mask, buffers.cta_k, q_len, buffers.attention_scale, is_causal)
-    launch_attention(
-        q_codes=buffers.q_codes, k_codes=buffers.k_codes, v_codes=buffers.v_codes, output=output,
-        q_scale=buffers.q_scale, k_scale=buffers.k_scale, v_scale=buffers.v_scale,
-        v_center=buffers.v_center, v_tile_sum=buffers.v_tile_sum, cta_k=buffers.cta_k,
-        sm_scale=buffers.attention_scale, attn_mask=attn_mask, is_causal=is_causal,
-        key_mask_tiles=tiles,
+    kv_heads, k_len = k.shape[1], k.shape[2]
+    query_mask = attn_mask is not None and attn_mask.stride(-2) != 0
+    key_only = attn_mask is not None and not query_mask
+    cta_k = select_key_block_size(dim, k_len, has_mask=query_mask)
+    lib = native.library()
+    output = torch.empty(batch, q_heads, q_len, dim, dtype=output_dtype_for(input_dtype), device=q.device)
+    workspace = torch.empty(
+        lib.risa_sdpa_workspace_bytes(batch, q_heads, q_len, kv_heads, k_len, dim, cta_k,
+                                      int(use_midpoint_affine), int(key_only)),
+        dtype=torch.uint8, device=q.device)
+    if attn_mask is None:
+        mask_args = (None, 0, 0, 0, 0, -1, 1, 1)
+    else:
+        mask_args = (attn_mask.data_ptr(), *attn_mask.stride(), MASK_DTYPE_CODES[attn_mask.dtype],
+                     batch if attn_mask.stride(0) != 0 else 1, q_heads if attn_mask.stride(1) != 0 else 1)
+    native.check(
+        lib.risa_sdpa(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), output.data_ptr(), workspace.data_ptr(),
+            workspace.numel(), batch, q_heads, q_len, kv_heads, k_len, dim, cta_k,
+            q.stride(0), q.stride(1), q.stride(2), k.stride(0), k.stride(1), k.stride(2),
+            v.stride(0), v.stride(1), v.stride(2), output.stride(0), output.stride(2), output.stride(1),
+            attention_scale, DTYPE_CODES[input_dtype], DTYPE_CODES[output.dtype],
+            int(use_midpoint_affine), *mask_args, int(bool(is_causal)),
+            native.current_stream(q.device),
+        )
     )
-    if original_dim != buffers.kernel_dim:
+    if original_dim != dim:
         output = output[..., :original_dim]
     return output.float() if input_dtype == torch.float32 else output
 

@@ -250,3 +250,126 @@ int risa_lse_shift(const void* q, const void* k, const int32_t* anchors, float* 
 }
 
 }  // extern "C"
+
+namespace {
+
+// Sections of the risa_sdpa workspace, each aligned to 256 bytes.
+struct SdpaLayout {
+  size_t q_codes, k_codes, v_codes, q_scale, k_scale, v_scale, v_center, tile_sum, anchors,
+      v_workspace, v_workspace_bytes, key_bias, key_tiles, bytes;
+};
+
+SdpaLayout sdpa_layout(int batch, int q_heads, int q_len, int kv_heads, int k_len, int head_dim,
+                       int cta_k, bool affine, bool key_only_mask) {
+  SdpaLayout l{};
+  size_t offset = 0;
+  auto take = [&](size_t bytes) {
+    const size_t at = offset;
+    offset += (bytes + 255) / 256 * 256;
+    return at;
+  };
+  const size_t tiles = (static_cast<size_t>(k_len) + cta_k - 1) / cta_k;
+  const size_t padded = tiles * cta_k;
+  const size_t kv = static_cast<size_t>(batch) * kv_heads;
+  const size_t q_groups = (static_cast<size_t>(q_len) + 127) / 128 * (head_dim == 256 ? 64 : 32);
+  l.q_codes = take(static_cast<size_t>(batch) * q_heads * q_len * head_dim);
+  l.k_codes = take(kv * k_len * head_dim);
+  l.v_codes = take(kv * head_dim * padded);
+  l.q_scale = take(static_cast<size_t>(batch) * q_heads * q_groups * 4);
+  l.k_scale = take(kv * tiles * 4 * 4);
+  l.v_scale = take(kv * head_dim * 4);
+  l.v_center = take(kv * head_dim * 4);
+  l.tile_sum = take(kv * tiles * head_dim * 4);
+  l.anchors = take(kv * 4);
+  l.v_workspace_bytes = risa::value_workspace_bytes(batch, kv_heads, k_len, head_dim, affine);
+  l.v_workspace = take(l.v_workspace_bytes);
+  l.key_bias = key_only_mask ? take(static_cast<size_t>(batch) * q_heads * padded * 4) : 0;
+  l.key_tiles = key_only_mask ? take(static_cast<size_t>(batch) * q_heads * (tiles + 1) * 4) : 0;
+  l.bytes = offset;
+  return l;
+}
+
+}  // namespace
+
+extern "C" {
+
+size_t risa_sdpa_workspace_bytes(int batch, int q_heads, int q_len, int kv_heads, int k_len,
+                                 int head_dim, int cta_k, int midpoint_affine, int key_only_mask) {
+  if (batch <= 0 || q_heads <= 0 || q_len <= 0 || kv_heads <= 0 || k_len <= 0 || head_dim <= 0 ||
+      (cta_k != 64 && cta_k != 128))
+    return 0;
+  return sdpa_layout(batch, q_heads, q_len, kv_heads, k_len, head_dim, cta_k, midpoint_affine != 0,
+                     key_only_mask != 0)
+      .bytes;
+}
+
+int risa_sdpa(const void* q, const void* k, const void* v, void* out, void* workspace,
+              size_t workspace_bytes, int batch, int q_heads, int q_len, int kv_heads, int k_len,
+              int head_dim, int cta_k, int64_t q_stride_b, int64_t q_stride_h, int64_t q_stride_n,
+              int64_t k_stride_b, int64_t k_stride_h, int64_t k_stride_n, int64_t v_stride_b,
+              int64_t v_stride_h, int64_t v_stride_n, int64_t out_stride_b, int64_t out_stride_n,
+              int64_t out_stride_h, float sm_scale, int input_dtype, int output_dtype,
+              int midpoint_affine, const void* mask, int64_t mask_stride_b, int64_t mask_stride_h,
+              int64_t mask_stride_q, int64_t mask_stride_k, int mask_dtype, int mask_batch,
+              int mask_heads, int is_causal, void* stream) {
+  using risa::fail;
+  if (batch <= 0 || q_heads <= 0 || q_len <= 0 || kv_heads <= 0 || k_len <= 0 ||
+      (cta_k != 64 && cta_k != 128))
+    return fail("risa_sdpa: extents must be positive and cta_k 64 or 128");
+  const bool key_only = mask != nullptr && mask_stride_q == 0;
+  const SdpaLayout l = sdpa_layout(batch, q_heads, q_len, kv_heads, k_len, head_dim, cta_k,
+                                   midpoint_affine != 0, key_only);
+  if (workspace == nullptr || !aligned(workspace, 256) || workspace_bytes < l.bytes)
+    return fail("risa_sdpa: workspace must be 256-byte aligned and hold risa_sdpa_workspace_bytes");
+  auto* base = static_cast<unsigned char*>(workspace);
+  auto* q_scale = reinterpret_cast<float*>(base + l.q_scale);
+  auto* k_scale = reinterpret_cast<float*>(base + l.k_scale);
+  auto* v_scale = reinterpret_cast<float*>(base + l.v_scale);
+  auto* v_center = reinterpret_cast<float*>(base + l.v_center);
+  auto* tile_sum = reinterpret_cast<int32_t*>(base + l.tile_sum);
+  const int tiles = (k_len + cta_k - 1) / cta_k;
+  const int padded = tiles * cta_k;
+  int status = risa_quantize_qk(q, base + l.q_codes, q_scale, k, base + l.k_codes, k_scale, batch,
+                                q_heads, q_len, kv_heads, k_len, head_dim, cta_k, q_stride_b,
+                                q_stride_h, q_stride_n, k_stride_b, k_stride_h, k_stride_n,
+                                input_dtype, reinterpret_cast<int32_t*>(base + l.anchors), nullptr,
+                                stream);
+  if (status != 0) return status;
+  status = risa_quantize_v(v, base + l.v_codes, v_scale, v_center, tile_sum, base + l.v_workspace,
+                           l.v_workspace_bytes, batch, kv_heads, k_len, head_dim, padded, cta_k,
+                           v_stride_b, v_stride_h, v_stride_n, input_dtype, midpoint_affine, nullptr,
+                           stream);
+  if (status != 0) return status;
+  const float* key_bias = nullptr;
+  const int32_t* key_tiles = nullptr;
+  int64_t bias_stride_b = 0, bias_stride_h = 0;
+  if (key_only) {
+    if (mask_batch != 1 && mask_batch != batch) return fail("risa_sdpa: mask batch extent");
+    if (mask_heads != 1 && mask_heads != q_heads) return fail("risa_sdpa: mask head extent");
+    auto* bias = reinterpret_cast<float*>(base + l.key_bias);
+    status = risa_prepare_key_bias(mask, bias, mask_batch, mask_heads, k_len, padded,
+                                   mask_batch > 1 ? mask_stride_b : 0,
+                                   mask_heads > 1 ? mask_stride_h : 0, mask_stride_k, mask_dtype,
+                                   stream);
+    if (status != 0) return status;
+    key_bias = bias;
+    bias_stride_h = mask_heads > 1 ? padded : 0;
+    bias_stride_b = mask_batch > 1 ? static_cast<int64_t>(mask_heads) * padded : 0;
+    // tile lists pay off under the conditions of reference _key_mask.py:9-28
+    if (k_len > 1024 && q_len >= 256 && sm_scale > 0.0f && is_causal == 0) {
+      auto* list = reinterpret_cast<int32_t*>(base + l.key_tiles);
+      status = risa_prepare_key_mask_tiles(mask, list, batch, q_heads, k_len, cta_k, mask_stride_b,
+                                           mask_stride_h, mask_stride_k, mask_dtype, stream);
+      if (status != 0) return status;
+      key_tiles = list;
+    }
+  }
+  return risa_attention(base + l.q_codes, base + l.k_codes, base + l.v_codes, out, q_scale, k_scale,
+                        v_scale, v_center, tile_sum, mask, mask_stride_b, mask_stride_h,
+                        mask_stride_q, mask_stride_k, mask_dtype, cta_k, batch, q_len, k_len,
+                        q_heads, kv_heads, head_dim, out_stride_b, out_stride_n, out_stride_h,
+                        sm_scale, output_dtype, nullptr, nullptr, nullptr, is_causal, nullptr,
+                        key_tiles, key_bias, bias_stride_b, bias_stride_h, stream);
+}
+
+}  // extern "C"
