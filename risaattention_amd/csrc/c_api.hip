@@ -17,20 +17,12 @@ bool stride_multiple(int64_t stride, int extent, int64_t multiple) {
   return extent < 2 || (stride > 0 && stride % multiple == 0);
 }
 
-}  // namespace
-
-extern "C" {
-
-const char* risa_last_error(void) { return risa::last_error_storage().c_str(); }
-
-int risa_abi_version(void) { return 1; }
-
-int risa_quantize_qk(const void* q, void* q_int8, float* q_scale, const void* k, void* k_int8,
-                     float* k_scale, int batch, int q_heads, int q_len, int kv_heads, int k_len,
-                     int head_dim, int cta_k, int64_t q_stride_b, int64_t q_stride_h,
-                     int64_t q_stride_n, int64_t k_stride_b, int64_t k_stride_h,
-                     int64_t k_stride_n, int input_dtype, int32_t* anchor_indices,
-                     const int32_t* kv_permutation, void* stream) {
+// Validation and argument block shared by risa_quantize_qk and risa_sdpa.
+int checked_qk_args(risa::QkArgs& a, const void* q, void* q_int8, float* q_scale, const void* k,
+                    void* k_int8, float* k_scale, int batch, int q_heads, int q_len, int kv_heads,
+                    int k_len, int head_dim, int cta_k, int64_t q_stride_b, int64_t q_stride_h,
+                    int64_t q_stride_n, int64_t k_stride_b, int64_t k_stride_h, int64_t k_stride_n,
+                    int input_dtype, int32_t* anchor_indices, const int32_t* kv_permutation) {
   using risa::fail;
   if (head_dim != 64 && head_dim != 128 && head_dim != 256)
     return fail("risa_quantize_qk: padded head_dim must be 64, 128, or 256");
@@ -49,7 +41,6 @@ int risa_quantize_qk(const void* q, void* q_int8, float* q_scale, const void* k,
   if (!q_ok || !k_ok)
     return fail("risa_quantize_qk: Q/K base pointers and batch/head/sequence strides must "
                 "preserve 4-element alignment");
-  risa::QkArgs a{};
   a.q = q;
   a.q_codes = static_cast<int8_t*>(q_int8);
   a.q_scale = q_scale;
@@ -72,19 +63,15 @@ int risa_quantize_qk(const void* q, void* q_int8, float* q_scale, const void* k,
   a.k_stride_b = k_stride_b;
   a.k_stride_h = k_stride_h;
   a.k_stride_n = k_stride_n;
-  return risa::launch_quantize_qk(a, static_cast<hipStream_t>(stream));
+  return 0;
 }
 
-size_t risa_quantize_v_workspace_bytes(int batch, int heads, int length, int head_dim,
-                                       int midpoint_affine) {
-  return risa::value_workspace_bytes(batch, heads, length, head_dim, midpoint_affine != 0);
-}
-
-int risa_quantize_v(const void* v, void* out, float* scale, float* center, int32_t* tile_sum,
-                    void* workspace, size_t workspace_bytes, int batch, int heads, int length,
-                    int head_dim, int padded_length, int cta_k, int64_t stride_b,
-                    int64_t stride_h, int64_t stride_n, int input_dtype, int midpoint_affine,
-                    const int32_t* kv_permutation, void* stream) {
+// Validation and argument block shared by risa_quantize_v and risa_sdpa.
+int checked_v_args(risa::ValueArgs& a, const void* v, void* out, float* scale, float* center,
+                   int32_t* tile_sum, void* workspace, size_t workspace_bytes, int batch, int heads,
+                   int length, int head_dim, int padded_length, int cta_k, int64_t stride_b,
+                   int64_t stride_h, int64_t stride_n, int input_dtype, int midpoint_affine,
+                   const int32_t* kv_permutation) {
   using risa::fail;
   if (head_dim != 64 && head_dim != 128 && head_dim != 256)
     return fail("risa_quantize_v: padded head_dim must be 64, 128, or 256");
@@ -101,7 +88,6 @@ int risa_quantize_v(const void* v, void* out, float* scale, float* center, int32
                 "16-byte aligned");
   if (tile_sum == nullptr || workspace == nullptr)
     return fail("risa_quantize_v: tile sums and workspace are required");
-  risa::ValueArgs a{};
   a.v = v;
   a.codes = static_cast<int8_t*>(out);
   a.scale = scale;
@@ -121,6 +107,47 @@ int risa_quantize_v(const void* v, void* out, float* scale, float* center, int32
   a.stride_h = stride_h;
   a.stride_n = stride_n;
   a.midpoint_affine = midpoint_affine != 0;
+  return 0;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* risa_last_error(void) { return risa::last_error_storage().c_str(); }
+
+int risa_abi_version(void) { return 1; }
+
+int risa_quantize_qk(const void* q, void* q_int8, float* q_scale, const void* k, void* k_int8,
+                     float* k_scale, int batch, int q_heads, int q_len, int kv_heads, int k_len,
+                     int head_dim, int cta_k, int64_t q_stride_b, int64_t q_stride_h,
+                     int64_t q_stride_n, int64_t k_stride_b, int64_t k_stride_h,
+                     int64_t k_stride_n, int input_dtype, int32_t* anchor_indices,
+                     const int32_t* kv_permutation, void* stream) {
+  risa::QkArgs a{};
+  const int status = checked_qk_args(a, q, q_int8, q_scale, k, k_int8, k_scale, batch, q_heads, q_len,
+                                     kv_heads, k_len, head_dim, cta_k, q_stride_b, q_stride_h,
+                                     q_stride_n, k_stride_b, k_stride_h, k_stride_n, input_dtype,
+                                     anchor_indices, kv_permutation);
+  if (status != 0) return status;
+  return risa::launch_quantize_qk(a, static_cast<hipStream_t>(stream));
+}
+
+size_t risa_quantize_v_workspace_bytes(int batch, int heads, int length, int head_dim,
+                                       int midpoint_affine) {
+  return risa::value_workspace_bytes(batch, heads, length, head_dim, midpoint_affine != 0);
+}
+
+int risa_quantize_v(const void* v, void* out, float* scale, float* center, int32_t* tile_sum,
+                    void* workspace, size_t workspace_bytes, int batch, int heads, int length,
+                    int head_dim, int padded_length, int cta_k, int64_t stride_b,
+                    int64_t stride_h, int64_t stride_n, int input_dtype, int midpoint_affine,
+                    const int32_t* kv_permutation, void* stream) {
+  risa::ValueArgs a{};
+  const int status = checked_v_args(a, v, out, scale, center, tile_sum, workspace, workspace_bytes,
+                                    batch, heads, length, head_dim, padded_length, cta_k, stride_b,
+                                    stride_h, stride_n, input_dtype, midpoint_affine, kv_permutation);
+  if (status != 0) return status;
   return risa::launch_quantize_v(a, static_cast<hipStream_t>(stream));
 }
 
@@ -329,16 +356,25 @@ int risa_sdpa(const void* q, const void* k, const void* v, void* out, void* work
   auto* tile_sum = reinterpret_cast<int32_t*>(base + l.tile_sum);
   const int tiles = (k_len + cta_k - 1) / cta_k;
   const int padded = tiles * cta_k;
-  int status = risa_quantize_qk(q, base + l.q_codes, q_scale, k, base + l.k_codes, k_scale, batch,
-                                q_heads, q_len, kv_heads, k_len, head_dim, cta_k, q_stride_b,
-                                q_stride_h, q_stride_n, k_stride_b, k_stride_h, k_stride_n,
-                                input_dtype, reinterpret_cast<int32_t*>(base + l.anchors), nullptr,
-                                stream);
+  risa::QkArgs qk{};
+  int status = checked_qk_args(qk, q, base + l.q_codes, q_scale, k, base + l.k_codes, k_scale, batch,
+                               q_heads, q_len, kv_heads, k_len, head_dim, cta_k, q_stride_b,
+                               q_stride_h, q_stride_n, k_stride_b, k_stride_h, k_stride_n,
+                               input_dtype, reinterpret_cast<int32_t*>(base + l.anchors), nullptr);
   if (status != 0) return status;
-  status = risa_quantize_v(v, base + l.v_codes, v_scale, v_center, tile_sum, base + l.v_workspace,
-                           l.v_workspace_bytes, batch, kv_heads, k_len, head_dim, padded, cta_k,
-                           v_stride_b, v_stride_h, v_stride_n, input_dtype, midpoint_affine, nullptr,
-                           stream);
+  risa::ValueArgs value{};
+  status = checked_v_args(value, v, base + l.v_codes, v_scale, v_center, tile_sum,
+                          base + l.v_workspace, l.v_workspace_bytes, batch, kv_heads, k_len, head_dim,
+                          padded, cta_k, v_stride_b, v_stride_h, v_stride_n, input_dtype,
+                          midpoint_affine, nullptr);
+  if (status != 0) return status;
+  hipStream_t hip_stream = static_cast<hipStream_t>(stream);
+  if (risa::can_prepare_fused(qk, value)) {
+    status = risa::launch_prepare_fused(qk, value, hip_stream);
+  } else {
+    status = risa::launch_quantize_qk(qk, hip_stream);
+    if (status == 0) status = risa::launch_quantize_v(value, hip_stream);
+  }
   if (status != 0) return status;
   const float* key_bias = nullptr;
   const int32_t* key_tiles = nullptr;

@@ -102,6 +102,10 @@ int launch_key_mask_tiles(const void* mask, int32_t* tiles, int batch, int heads
                           int tile_size, int64_t stride_b, int64_t stride_h, int64_t stride_k,
                           int dtype, hipStream_t stream);
 
+// Q/K/V preparation in two launches (short sequences, no permutation).
+bool can_prepare_fused(const QkArgs& qk, const ValueArgs& v);
+int launch_prepare_fused(const QkArgs& qk, const ValueArgs& v, hipStream_t stream);
+
 int launch_key_bias(const void* mask, float* bias, int batch, int heads, int length, int padded,
                     int64_t stride_b, int64_t stride_h, int64_t stride_k, int dtype,
                     hipStream_t stream);

@@ -1,0 +1,181 @@
+// Q/K/V preparation in two launches for short sequences.
+//
+// The separate preparation kernels (prep_qk.hip, prep_v.hip) are five to seven
+// launches whose order is fixed by data: anchor -> K codes, V range -> V parameters
+// -> V codes.  Up to a few thousand tokens every one of them runs for about five
+// microseconds however little it does, and the chain is longer than the attention
+// kernel.  The work has only two levels of dependence, so two launches are enough:
+//   stage 1  Q codes | K anchor | V partial ranges      (independent workgroups)
+//   stage 2  K codes (needs the anchor) | V codes (reduce the partial ranges themselves)
+// A workgroup finds its role from its index; every role runs the same device
+// function as the stand-alone kernel, so results are bit-identical.  Used when the
+// V range has at most 64 partial chunks (4096 tokens) and no permutation is given.
+
+#include "prep_qk_kernels.hpp"
+#include "prep_v_kernels.hpp"
+
+namespace risa {
+namespace {
+
+struct FusedArgs {
+  QkArgs qk;
+  ValueArgs v;
+  float* part_max;
+  float* part_min;
+  float* inverse;
+  float* midpoint;
+  float* partial;
+  int q_slices, q_blocks, anchor_blocks, range_groups, chunks;
+  int key_tiles, key_pairs, key_blocks, code_blocks_x, kv;
+  int q_wide, k_wide;
+};
+
+template <int DT, int DK, int ROT, bool AFFINE>
+__global__ __launch_bounds__(256) void prepare_stage1_kernel(const FusedArgs a) {
+  int block = blockIdx.x;
+  if (block < a.q_blocks) {
+    const int slice = block % a.q_slices;
+    const int rest = block / a.q_slices;
+    quantize_q_block<DT, DK, ROT>(a.qk.q, a.qk.q_codes, a.qk.q_scale, a.qk.q_len, a.qk.q_heads,
+                                  a.q_slices * 8, a.qk.q_stride_b, a.qk.q_stride_h, a.qk.q_stride_n,
+                                  a.q_wide, slice, rest % a.qk.q_heads, rest / a.qk.q_heads);
+    return;
+  }
+  block -= a.q_blocks;
+  if (block < a.anchor_blocks) {
+    detect_anchor_block<DT>(a.qk.k, a.qk.anchors, a.qk.k_len, a.qk.head_dim, a.qk.kv_heads,
+                            a.qk.k_stride_b, a.qk.k_stride_h, a.qk.k_stride_n, nullptr,
+                            block % a.qk.kv_heads, block / a.qk.kv_heads);
+    return;
+  }
+  block -= a.anchor_blocks;
+  value_range_block<DT, AFFINE>(a.v.v, a.part_max, a.part_min, a.v.length, a.v.head_dim, a.v.heads,
+                                a.chunks, a.v.stride_b, a.v.stride_h, a.v.stride_n,
+                                block % a.range_groups, block / a.range_groups);
+}
+
+template <int DT, int DK, int CTA_K, int ROT, int PARAMS>
+__global__ __launch_bounds__(256) void prepare_stage2_kernel(const FusedArgs a) {
+  int block = blockIdx.x;
+  if (block < a.key_blocks) {
+    // two key tiles per workgroup: eight 32-lane halves = 2 x four scale groups
+    const int pair = block % a.key_pairs;
+    const int rest = block / a.key_pairs;
+    const int half = threadIdx.x >> 5;
+    const int tile = pair * 2 + half / 4;
+    if (tile < a.key_tiles) {
+      quantize_k_block<DT, DK, CTA_K, ROT>(a.qk.k, a.qk.k_codes, a.qk.k_scale, a.qk.anchors, a.qk.k_len,
+                                           a.qk.kv_heads, a.key_tiles * 4, a.qk.k_stride_b,
+                                           a.qk.k_stride_h, a.qk.k_stride_n, a.k_wide, nullptr, tile,
+                                           half % 4, rest % a.qk.kv_heads, rest / a.qk.kv_heads);
+    }
+    return;
+  }
+  block -= a.key_blocks;
+  const FusedParams fused{a.part_max, a.part_min, a.v.scale, a.v.center, a.inverse, a.midpoint, a.chunks};
+  const int x = block % a.code_blocks_x;
+  const int rest = block / a.code_blocks_x;
+  value_codes_block<DT, CTA_K, PARAMS>(a.v.v, a.v.codes, a.v.tile_sum, a.inverse, a.midpoint, a.v.length,
+                                       a.v.padded, a.v.head_dim, a.v.heads, a.v.stride_b, a.v.stride_h,
+                                       a.v.stride_n, nullptr, fused, x, rest % a.kv, rest / a.kv);
+}
+
+template <int DT, int DK, int CTA_K, int ROT>
+void launch_stages(const FusedArgs& a, hipStream_t stream) {
+  const int stage1_blocks = a.q_blocks + a.anchor_blocks + a.range_groups * a.kv;
+  const int stage2_blocks = a.key_blocks + a.code_blocks_x * a.kv * (a.v.head_dim / 32);
+  if (a.v.midpoint_affine) {
+    prepare_stage1_kernel<DT, DK, ROT, true><<<stage1_blocks, 256, 0, stream>>>(a);
+    prepare_stage2_kernel<DT, DK, CTA_K, ROT, kParamsAffine><<<stage2_blocks, 256, 0, stream>>>(a);
+    const int threads = summation_threads(a.v.length);
+    const int per_block = 256 / (a.v.head_dim / 8);
+    const int rows = a.kv * a.v.head_dim;
+    dim3 residual_grid(threads / per_block, a.kv);
+    value_residual_kernel<DT><<<residual_grid, 256, 0, stream>>>(
+        a.v.v, a.partial, a.inverse, a.midpoint, a.v.length,
+        a.v.head_dim, a.v.heads, threads, a.v.stride_b, a.v.stride_h, a.v.stride_n, nullptr);
+    value_center_kernel<<<(rows + 63) / 64, 64, 0, stream>>>(
+        a.partial, a.inverse, a.midpoint, a.v.center, rows, threads,
+        a.v.length);
+  } else {
+    prepare_stage1_kernel<DT, DK, ROT, false><<<stage1_blocks, 256, 0, stream>>>(a);
+    prepare_stage2_kernel<DT, DK, CTA_K, ROT, kParamsAbsmax><<<stage2_blocks, 256, 0, stream>>>(a);
+  }
+}
+
+template <int DT, int DK> void launch_by_rotation(const FusedArgs& a, hipStream_t stream) {
+  const bool short_keys = a.qk.k_len <= 256;
+  constexpr int LONG_ROT = DK == 64 ? kRot64 : DK == 128 ? kRot128Signed : kRot128Plain;
+  if constexpr (DK == 64) {
+    if (short_keys)
+      launch_stages<DT, DK, 64, kRot4>(a, stream);
+    else
+      launch_stages<DT, DK, 64, LONG_ROT>(a, stream);
+  } else {
+    if (a.qk.cta_k == 128) {
+      if (short_keys)
+        launch_stages<DT, DK, 128, kRot4>(a, stream);
+      else
+        launch_stages<DT, DK, 128, LONG_ROT>(a, stream);
+    } else {
+      if (short_keys)
+        launch_stages<DT, DK, 64, kRot4>(a, stream);
+      else
+        launch_stages<DT, DK, 64, LONG_ROT>(a, stream);
+    }
+  }
+}
+
+template <int DT> void launch_by_dim(const FusedArgs& a, hipStream_t stream) {
+  if (a.qk.head_dim == 64)
+    launch_by_rotation<DT, 64>(a, stream);
+  else if (a.qk.head_dim == 128)
+    launch_by_rotation<DT, 128>(a, stream);
+  else
+    launch_by_rotation<DT, 256>(a, stream);
+}
+
+}  // namespace
+
+bool can_prepare_fused(const QkArgs& qk, const ValueArgs& v) {
+  return qk.permutation == nullptr && v.permutation == nullptr && qk.k_len == v.length &&
+         qk.batch == v.batch && qk.kv_heads == v.heads && qk.head_dim == v.head_dim &&
+         qk.cta_k == v.cta_k && qk.dtype == v.dtype && range_chunks(v.length) <= 64;
+}
+
+int launch_prepare_fused(const QkArgs& qk, const ValueArgs& v, hipStream_t stream) {
+  if (!can_prepare_fused(qk, v)) return fail("risa_sdpa: operands do not qualify for the two-launch preparation");
+  if (v.workspace_bytes < value_workspace_bytes(v.batch, v.heads, v.length, v.head_dim, v.midpoint_affine))
+    return fail("risa_quantize_v: workspace is too small");
+  const Workspace w = carve(v.workspace, v.batch, v.heads, v.length, v.head_dim, v.midpoint_affine);
+  FusedArgs a{};
+  a.qk = qk;
+  a.v = v;
+  a.part_max = w.part_max;
+  a.part_min = w.part_min;
+  a.inverse = w.inverse;
+  a.midpoint = w.midpoint;
+  a.partial = w.partial;
+  const int slice_rows = qk.head_dim == 256 ? 16 : 32;
+  a.q_slices = (qk.q_len + 127) / 128 * (128 / slice_rows);
+  a.q_blocks = a.q_slices * qk.q_heads * qk.batch;
+  a.kv = qk.batch * qk.kv_heads;
+  a.anchor_blocks = a.kv;
+  a.chunks = range_chunks(v.length);
+  a.range_groups = (a.chunks + 3) / 4;
+  a.key_tiles = (qk.k_len + qk.cta_k - 1) / qk.cta_k;
+  a.key_pairs = (a.key_tiles + 1) / 2;
+  a.key_blocks = a.key_pairs * a.kv;
+  a.code_blocks_x = (v.padded + 255) / 256;
+  a.q_wide = rows_are_16_byte_aligned(qk.q, qk.q_stride_b, qk.q_stride_h, qk.q_stride_n, qk.dtype);
+  a.k_wide = rows_are_16_byte_aligned(qk.k, qk.k_stride_b, qk.k_stride_h, qk.k_stride_n, qk.dtype);
+  if (qk.dtype == kF32)
+    launch_by_dim<kF32>(a, stream);
+  else if (qk.dtype == kF16)
+    launch_by_dim<kF16>(a, stream);
+  else
+    launch_by_dim<kBF16>(a, stream);
+  return check_launch("risa_sdpa preparation");
+}
+
+}  // namespace risa

@@ -1,428 +1,16 @@
-// Q/K preparation for gfx950: K anchor detection, sign-diagonal + Walsh-Hadamard
-// rotation and per-group signed INT8 quantisation.
-//
-// Numerical contract (bit-exact): reference csrc/kernels/quantize_qk_impl.cuh
-//   detect_k_anchor :442-577, rotations :69-147, process_q :153-269,
-//   process_k :278-426, dispatch by (head_dim, key_length) :769-811.
-// The reference assigns one scale group to a 32-lane warp in which every lane
-// owns four adjacent channels.  Here one 32-lane half of a 64-wide wavefront
-// plays that role, so a wavefront quantises two scale groups at once and the
-// butterfly order (4-point local stage, then lane bits 1, 2, 4, 8, 16) is the
-// reference's.  All arithmetic is IEEE binary32 without contraction.
+// Launchers of the Q/K preparation kernels (prep_qk_kernels.hpp) and the LSE anchor
+// correction.
 
-#include "common.hpp"
-#include "launchers.hpp"
-
-#include <type_traits>
+#include "prep_qk_kernels.hpp"
 
 namespace risa {
 namespace {
-
-constexpr int kRot4 = 4;
-constexpr int kRot64 = 64;
-constexpr int kRot128Signed = 128;
-constexpr int kRot128Plain = 129;
-
-__device__ __forceinline__ void rotate4(float* v) {
-  const float a0 = v[0] + v[1];
-  const float a1 = v[0] - v[1];
-  const float a2 = v[2] + v[3];
-  const float a3 = v[2] - v[3];
-  v[0] = (a0 + a2) * 0.5f;
-  v[1] = (a1 + a3) * 0.5f;
-  v[2] = (a0 - a2) * 0.5f;
-  v[3] = (a1 - a3) * 0.5f;
-}
-
-// Channel c keeps its sign when bit c%32 of word c/32 is set and is negated
-// otherwise; `sub` is the lane inside the 32-lane half, owning channels 4*sub..
-__device__ __forceinline__ void apply_sign_diagonal(float* v, int sub) {
-  const uint32_t words[4] = {0x1035997bu, 0x8087f5eeu, 0xee2e4e1au, 0x71132418u};
-  const uint32_t word = words[sub >> 3];
-  const int shift = (sub & 7) * 4;
-#pragma unroll
-  for (int c = 0; c < 4; ++c) {
-    const uint32_t flip = ((word >> (shift + c)) & 1u) ^ 1u;
-    v[c] = __uint_as_float(__float_as_uint(v[c]) ^ (flip << 31));
-  }
-}
-
-// Value of lane (l xor BIT) for BIT in {1, 2, 4, 8}, with DPP moves (no LDS
-// traffic): quad permutations inside groups of four lanes, row shifts inside
-// rows of sixteen lanes written under a bank mask (lanes whose partner is above
-// take the left shift, the others the right shift).
-template <int BIT> __device__ __forceinline__ float dpp_partner(float value) {
-  const int bits = __float_as_int(value);
-  if constexpr (BIT == 1) {
-    return __int_as_float(__builtin_amdgcn_update_dpp(0, bits, 0xB1, 0xf, 0xf, true));  // quad_perm [1,0,3,2]
-  } else if constexpr (BIT == 2) {
-    return __int_as_float(__builtin_amdgcn_update_dpp(0, bits, 0x4E, 0xf, 0xf, true));  // quad_perm [2,3,0,1]
-  } else if constexpr (BIT == 4) {
-    const int up = __builtin_amdgcn_update_dpp(0, bits, 0x104, 0xf, 0x5, true);      // row_shl:4 -> banks 0, 2
-    return __int_as_float(__builtin_amdgcn_update_dpp(up, bits, 0x114, 0xf, 0xA, false));  // row_shr:4 -> banks 1, 3
-  } else {
-    static_assert(BIT == 8, "DPP reaches partners inside a row of sixteen lanes");
-    const int up = __builtin_amdgcn_update_dpp(0, bits, 0x108, 0xf, 0x3, true);      // row_shl:8 -> banks 0, 1
-    return __int_as_float(__builtin_amdgcn_update_dpp(up, bits, 0x118, 0xf, 0xC, false));  // row_shr:8 -> banks 2, 3
-  }
-}
-
-// Hadamard butterflies over the lane bits below LANES, in the reference's order
-// (bit 1 first): the lane with the bit clear keeps a + b, the other b - a.
-template <int LANES> __device__ __forceinline__ void lane_butterflies(float* v, int sub) {
-  auto level = [&](auto bit_tag) {
-    constexpr int BIT = decltype(bit_tag)::value;
-    if constexpr (BIT < LANES) {
-#pragma unroll
-      for (int c = 0; c < 4; ++c) {
-        float other;
-        if constexpr (BIT < 16) {
-          other = dpp_partner<BIT>(v[c]);
-        } else {
-          other = __shfl_xor(v[c], BIT);
-        }
-        // other - v on the lanes with the bit set, other + v on the rest: one sign
-        // flip (exact) and one addition instead of both results and a select
-        const uint32_t flip = (sub & BIT) ? 0x80000000u : 0u;
-        v[c] = other + __uint_as_float(__float_as_uint(v[c]) ^ flip);
-      }
-    }
-  };
-  level(std::integral_constant<int, 1>{});
-  level(std::integral_constant<int, 2>{});
-  level(std::integral_constant<int, 4>{});
-  level(std::integral_constant<int, 8>{});
-  level(std::integral_constant<int, 16>{});
-}
-
-// Rotation of the channels one lane holds of one 128-channel block (64 for head
-// dim 64).  Sixteen lanes share a token; lane j owns GROUPS runs of four
-// consecutive channels, 4*GROUPS*j + 4g .. +3, i.e. the channels of lanes 2j and
-// 2j+1 (GROUPS 2) or of lane j (GROUPS 1) of the reference's 32-lane layout
-// (csrc/kernels/quantize_qk.cuh).  The additions are the reference's, in its
-// order: 4-point transform per run, then one butterfly level per channel bit from
-// bit 2 up -- the first inside the lane when it holds two runs, the others
-// between lanes with DPP moves.
-template <int ROT, int GROUPS> __device__ __forceinline__ void rotate(float (&v)[GROUPS][4], int j) {
-#pragma unroll
-  for (int g = 0; g < GROUPS; ++g) {
-    if constexpr (ROT == kRot128Signed) apply_sign_diagonal(v[g], GROUPS * j + g);
-    rotate4(v[g]);
-  }
-  if constexpr (ROT == kRot4) return;
-  if constexpr (GROUPS == 2) {
-#pragma unroll
-    for (int c = 0; c < 4; ++c) {
-      const float low = v[0][c], high = v[1][c];
-      v[0][c] = low + high;
-      v[1][c] = low - high;
-    }
-  }
-#pragma unroll
-  for (int g = 0; g < GROUPS; ++g) lane_butterflies<16>(v[g], j);
-  constexpr float factor = ROT == kRot64 ? 0.25f : 0.1767766952966369f;
-#pragma unroll
-  for (int g = 0; g < GROUPS; ++g)
-#pragma unroll
-    for (int c = 0; c < 4; ++c) v[g][c] *= factor;
-}
-
-__device__ __forceinline__ float half_wave_max(float value) {
-#pragma unroll
-  for (int offset = 16; offset > 0; offset >>= 1) {
-    value = __builtin_fmaxf(value, __shfl_xor(value, offset));
-  }
-  return value;
-}
-
-// One scale group handled by one 32-lane half: NTOK tokens x DK channels, two
-// tokens at a time (one per 16-lane row).  `token_of(i)` gives the i-th token of
-// the group.  `wide` says rows are 16-byte aligned, so 16-bit inputs are read
-// eight channels per load.
-template <int DT, int DK, int ROT, int NTOK, typename TokenOf>
-__device__ __forceinline__ void quantize_group(const void* in, int64_t in_base, int64_t stride_n,
-                                               int8_t* out, float* scale_slot, int length, int sub,
-                                               const void* bias_row, bool wide, TokenOf token_of,
-                                               const int32_t* source = nullptr) {
-  constexpr int BLOCKS = DK == 256 ? 2 : 1;   // 128-channel rotation blocks
-  constexpr int GROUPS = DK == 64 ? 1 : 2;    // runs of four channels per lane and block
-  constexpr int STEPS = NTOK / 2;
-  static_assert(NTOK % 2 == 0, "two tokens per 32-lane half and step");
-  const int j = sub & 15, row = sub >> 4;
-  auto channel_of = [&](int block, int g) { return block * 128 + (GROUPS * j + g) * 4; };
-
-  auto load_row = [&](int64_t row_base, float (&dst)[BLOCKS][GROUPS][4]) {
-#pragma unroll
-    for (int block = 0; block < BLOCKS; ++block) {
-      if (GROUPS == 2 && DT != kF32 && wide) {
-        float eight[8];
-        load8<DT>(in, row_base + channel_of(block, 0), eight);
-#pragma unroll
-        for (int c = 0; c < 8; ++c) dst[block][c / 4][c % 4] = eight[c];
-      } else {
-#pragma unroll
-        for (int g = 0; g < GROUPS; ++g) load4<DT>(in, row_base + channel_of(block, g), dst[block][g]);
-      }
-    }
-  };
-
-  float bias[BLOCKS][GROUPS][4];
-  if (bias_row != nullptr) load_row(in_base + *static_cast<const int64_t*>(bias_row), bias);
-
-  float v[STEPS][BLOCKS][GROUPS][4];
-#pragma unroll
-  for (int i = 0; i < STEPS; ++i) {
-    const int n = token_of(2 * i + row);
-    if (n < length) {
-      // with a permutation, token n of the gathered sequence is source row source[n]
-      const int from = source != nullptr ? source[n] : n;
-      load_row(in_base + static_cast<int64_t>(from) * stride_n, v[i]);
-      if (bias_row != nullptr) {
-#pragma unroll
-        for (int block = 0; block < BLOCKS; ++block)
-#pragma unroll
-          for (int g = 0; g < GROUPS; ++g)
-#pragma unroll
-            for (int c = 0; c < 4; ++c) v[i][block][g][c] -= bias[block][g][c];
-      }
-    } else {
-#pragma unroll
-      for (int block = 0; block < BLOCKS; ++block)
-#pragma unroll
-        for (int g = 0; g < GROUPS; ++g)
-#pragma unroll
-          for (int c = 0; c < 4; ++c) v[i][block][g][c] = 0.0f;
-    }
-  }
-  float mx = 0.0f;
-#pragma unroll
-  for (int i = 0; i < STEPS; ++i)
-#pragma unroll
-    for (int block = 0; block < BLOCKS; ++block) {
-      rotate<ROT, GROUPS>(v[i][block], j);
-#pragma unroll
-      for (int g = 0; g < GROUPS; ++g)
-#pragma unroll
-        for (int c = 0; c < 4; ++c) mx = __builtin_fmaxf(mx, __builtin_fabsf(v[i][block][g][c]));
-    }
-  mx = half_wave_max(mx);
-  const float scale = mx / 127.0f + 1e-7f;
-  const float inverse = 1.0f / scale;
-  if (sub == 0) *scale_slot = scale;
-#pragma unroll
-  for (int i = 0; i < STEPS; ++i) {
-    const int n = token_of(2 * i + row);
-    if (n < length) {
-#pragma unroll
-      for (int block = 0; block < BLOCKS; ++block) {
-        uint32_t packed[GROUPS];
-#pragma unroll
-        for (int g = 0; g < GROUPS; ++g) {
-          packed[g] = pack_s8x4(quantize_s8(v[i][block][g][0] * inverse), quantize_s8(v[i][block][g][1] * inverse),
-                                quantize_s8(v[i][block][g][2] * inverse), quantize_s8(v[i][block][g][3] * inverse));
-        }
-        int8_t* at = out + static_cast<int64_t>(n) * DK + channel_of(block, 0);
-        if constexpr (GROUPS == 2) {
-          *reinterpret_cast<uint2*>(at) = make_uint2(packed[0], packed[1]);
-        } else {
-          *reinterpret_cast<uint32_t*>(at) = packed[0];
-        }
-      }
-    }
-  }
-}
-
-constexpr int kSlicesPerBlock = 1;
-
-// grid (ceil(slices / kSlicesPerBlock), Hq, B), 256 threads: eight 32-lane halves = the eight scale
-// groups (token index mod 8) of one W-row slice, W = 32 (16 for head_dim 256).
-template <int DT, int DK, int ROT>
-__global__ __launch_bounds__(256) void quantize_q_kernel(const void* __restrict__ q,
-                                                         int8_t* __restrict__ codes,
-                                                         float* __restrict__ scales, int length,
-                                                         int heads, int scales_per_head,
-                                                         int64_t stride_b, int64_t stride_h,
-                                                         int64_t stride_n, int wide) {
-  constexpr int W = DK == 256 ? 16 : 32;
-  constexpr int NR = W / 8;
-  const int h = blockIdx.y, b = blockIdx.z;
-  const int sub = threadIdx.x & 31;
-  const int group = threadIdx.x >> 5;
-  const int64_t in_base = static_cast<int64_t>(b) * stride_b + static_cast<int64_t>(h) * stride_h;
-  const int64_t bh = static_cast<int64_t>(b) * heads + h;
-  // kSlicesPerBlock consecutive slices per workgroup.  One is fastest (52.6 us at
-  // 16 x 32768 tokens against 59.8 us with four): the loop serialises the loads of
-  // successive slices, and workgroup launch is not what limits the kernel.
-  const int slices = scales_per_head / 8;
-#pragma unroll 1
-  for (int step = 0; step < kSlicesPerBlock; ++step) {
-    const int slice = blockIdx.x * kSlicesPerBlock + step;
-    if (slice >= slices) break;
-    const int base = slice * W + group;
-    quantize_group<DT, DK, ROT, NR>(q, in_base, stride_n, codes + bh * length * DK,
-                                    scales + bh * scales_per_head + slice * 8 + group, length, sub,
-                                    nullptr, wide != 0, [base](int i) { return base + i * 8; });
-  }
-}
-
-// grid (key tiles, Hkv, B), 128 threads: four 32-lane halves = the four scale
-// groups ((token mod 8) / 2) of one key tile of CTA_K tokens.
-template <int DT, int DK, int CTA_K, int ROT>
-__global__ __launch_bounds__(128) void quantize_k_kernel(const void* __restrict__ k,
-                                                         int8_t* __restrict__ codes,
-                                                         float* __restrict__ scales,
-                                                         const int* __restrict__ anchors, int length,
-                                                         int heads, int scales_per_head,
-                                                         int64_t stride_b, int64_t stride_h,
-                                                         int64_t stride_n, int wide,
-                                                         const int32_t* __restrict__ permutation) {
-  constexpr int NTOK = CTA_K / 4;
-  const int tile = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
-  const int sub = threadIdx.x & 31;
-  const int group = threadIdx.x >> 5;
-  const int64_t in_base = static_cast<int64_t>(b) * stride_b + static_cast<int64_t>(h) * stride_h;
-  const int64_t bh = static_cast<int64_t>(b) * heads + h;
-  const int anchor = anchors[b * heads + h];
-  const int32_t* source = permutation != nullptr ? permutation + bh * length : nullptr;
-  // element offset of the anchor row (subtracted from every key) when one was chosen
-  const int anchor_row = anchor >= 0 && source != nullptr ? source[anchor] : anchor;
-  const int64_t anchor_offset = static_cast<int64_t>(anchor_row) * stride_n;
-  const int first = tile * CTA_K + group * 2;
-  quantize_group<DT, DK, ROT, NTOK>(k, in_base, stride_n, codes + bh * length * DK,
-                                    scales + bh * scales_per_head + tile * 4 + group, length, sub,
-                                    anchor >= 0 ? &anchor_offset : nullptr, wide != 0,
-                                    [first](int i) { return first + (i >> 1) * 8 + (i & 1); }, source);
-}
-
-// ---------------------------------------------------------------------------
-// Anchor detector: grid (Hkv, B), 128 threads.  Thread t owns channels t and
-// t+128; partial sums are combined by a 32-lane shuffle-down tree and then the
-// four 32-lane segments are added in order, which is the reference's order.
-// ---------------------------------------------------------------------------
-constexpr int kSamples = 9;
-
-__device__ __forceinline__ float segment_down_sum(float value) {
-#pragma unroll
-  for (int offset = 16; offset > 0; offset >>= 1) value += __shfl_down(value, offset, 32);
-  return value;
-}
-__device__ __forceinline__ float segment_down_max(float value) {
-#pragma unroll
-  for (int offset = 16; offset > 0; offset >>= 1)
-    value = __builtin_fmaxf(value, __shfl_down(value, offset, 32));
-  return value;
-}
-
-template <int DT>
-__global__ __launch_bounds__(128) void detect_anchor_kernel(const void* __restrict__ k,
-                                                            int* __restrict__ anchors, int length,
-                                                            int dim, int heads, int64_t stride_b,
-                                                            int64_t stride_h, int64_t stride_n,
-                                                            const int32_t* __restrict__ permutation) {
-  __shared__ float samples[kSamples * 256];
-  __shared__ float seg_energy[4], seg_max[4], seg_dist[kSamples][4], seg_best_energy[4],
-      seg_best_max[4];
-  __shared__ int chosen;
-  const int h = blockIdx.x, b = blockIdx.y;
-  const int tid = threadIdx.x, sub = tid & 31, seg = tid >> 5;
-  const int64_t base = static_cast<int64_t>(b) * stride_b + static_cast<int64_t>(h) * stride_h;
-  for (int index = tid; index < kSamples * dim; index += 128) {
-    const int s = index / dim;
-    const int c = index - s * dim;
-    int64_t row = static_cast<int64_t>(s) * (length - 1) / (kSamples - 1);
-    if (permutation != nullptr) row = permutation[(static_cast<int64_t>(b) * heads + h) * length + row];
-    samples[index] = load1<DT>(k, base + row * stride_n + c);
-  }
-  __syncthreads();
-
-  float energy = 0.0f, peak = 0.0f, dist[kSamples];
-#pragma unroll
-  for (int c = 0; c < kSamples; ++c) dist[c] = 0.0f;
-  for (int channel = tid; channel < dim; channel += 128) {
-    float sum = 0.0f;
-#pragma unroll
-    for (int s = 0; s < kSamples; ++s) {
-      const float value = samples[s * dim + channel];
-      energy = __builtin_fmaf(value, value, energy);
-      peak = __builtin_fmaxf(peak, __builtin_fabsf(value));
-      sum += value;
-    }
-#pragma unroll
-    for (int c = 0; c < kSamples; ++c) {
-      const float d = 9.0f * samples[c * dim + channel] - sum;
-      dist[c] = __builtin_fmaf(d, d, dist[c]);
-    }
-  }
-  energy = segment_down_sum(energy);
-  peak = segment_down_max(peak);
-#pragma unroll
-  for (int c = 0; c < kSamples; ++c) dist[c] = segment_down_sum(dist[c]);
-  if (sub == 0) {
-    seg_energy[seg] = energy;
-    seg_max[seg] = peak;
-#pragma unroll
-    for (int c = 0; c < kSamples; ++c) seg_dist[c][seg] = dist[c];
-  }
-  __syncthreads();
-  if (tid == 0) {
-    int best = 0;
-    float best_distance = 3.402823466e+38f;
-    for (int c = 0; c < kSamples; ++c) {
-      float total = 0.0f;
-      for (int w = 0; w < 4; ++w) total += seg_dist[c][w];
-      if (total < best_distance) {
-        best = c;
-        best_distance = total;
-      }
-    }
-    chosen = best;
-  }
-  __syncthreads();
-  const int best = chosen;
-  float best_energy = 0.0f, best_peak = 0.0f;
-  for (int channel = tid; channel < dim; channel += 128) {
-    const float anchor = samples[best * dim + channel];
-#pragma unroll
-    for (int s = 0; s < kSamples; ++s) {
-      const float residual = samples[s * dim + channel] - anchor;
-      best_energy = __builtin_fmaf(residual, residual, best_energy);
-      best_peak = __builtin_fmaxf(best_peak, __builtin_fabsf(residual));
-    }
-  }
-  best_energy = segment_down_sum(best_energy);
-  best_peak = segment_down_max(best_peak);
-  if (sub == 0) {
-    seg_best_energy[seg] = best_energy;
-    seg_best_max[seg] = best_peak;
-  }
-  __syncthreads();
-  if (tid == 0) {
-    float e0 = 0.0f, m0 = 0.0f, e1 = 0.0f, m1 = 0.0f;
-    for (int w = 0; w < 4; ++w) {
-      e0 += seg_energy[w];
-      m0 = __builtin_fmaxf(m0, seg_max[w]);
-      e1 += seg_best_energy[w];
-      m1 = __builtin_fmaxf(m1, seg_best_max[w]);
-    }
-    const bool improves = e1 < e0 && m1 <= m0 * 1.125f;
-    anchors[b * heads + h] =
-        improves ? static_cast<int>(static_cast<int64_t>(best) * (length - 1) / (kSamples - 1)) : -1;
-  }
-}
-
-// 16-bit inputs can be read eight channels (16 bytes) per load when every row
-// starts on a 16-byte boundary.
-inline int rows_are_16_byte_aligned(const void* base, int64_t stride_b, int64_t stride_h,
-                                    int64_t stride_n, int dtype) {
-  if (dtype == kF32) return 1;
-  return reinterpret_cast<uintptr_t>(base) % 16 == 0 && ((stride_b | stride_h | stride_n) & 7) == 0;
-}
 
 template <int DT, int DK, int ROT>
 void launch_q(const QkArgs& a, hipStream_t stream) {
   constexpr int W = DK == 256 ? 16 : 32;
   const int slices = (a.q_len + 127) / 128 * (128 / W);
-  dim3 grid((slices + kSlicesPerBlock - 1) / kSlicesPerBlock, a.q_heads, a.batch);
+  dim3 grid(slices, a.q_heads, a.batch);
   quantize_q_kernel<DT, DK, ROT><<<grid, 256, 0, stream>>>(
       a.q, a.q_codes, a.q_scale, a.q_len, a.q_heads, slices * 8, a.q_stride_b, a.q_stride_h,
       a.q_stride_n, rows_are_16_byte_aligned(a.q, a.q_stride_b, a.q_stride_h, a.q_stride_n, a.dtype));

@@ -1,0 +1,431 @@
+// V preparation for gfx950: per-channel range, signed INT8 codes in the packed
+// MFMA order, accumulator seeds (128 x per-tile code sums, the zero-point term of the
+// signed P·V product, plus risa::kAccumulatorSeedBits) and
+// the residual-corrected centre of the midpoint_affine mode.
+//
+// Numerical contract (bit-exact): reference csrc/kernels/quantize_v_impl.cuh:83-292
+// (range :104-186, codes :203-246, residual centre :248-275) and the schedule
+// choice of launch_quantize_v :356-401 (512 summation threads, 128 when L <= 256).
+//
+// The reference runs one block per (batch, head, 8 channels) that walks the whole
+// sequence twice; at 32K tokens and four KV heads that is 64 blocks.  Here the
+// sequence axis is split across the grid:
+//   1. value_range_kernel     partial min/max per (wavefront chunk of 64+ tokens, channel)
+//   2. value_params_kernel    scale, midpoint and reciprocal per channel
+//   3. value_codes_kernel     codes + packed transposed store + tile sums
+//   4. value_residual_kernel  (affine) per-summation-thread residual sums in the
+//                             reference's order: thread t adds tokens L-1-t-k*T
+//   5. value_center_kernel    (affine) xor-tree per 32 threads, warps in order
+// min/max are order independent, so 1-3 are exact for any split; 4-5 keep the
+// floating-point summation order explicitly.
+
+#pragma once
+
+#include "common.hpp"
+#include "launchers.hpp"
+
+#include <cfloat>
+
+namespace risa {
+namespace {
+
+// The range pass gives every wavefront tokens_per_wave(length) consecutive tokens:
+// 64 up to 32768 tokens, then whatever keeps the number of partial ranges per
+// (batch, head) at 512, which one wavefront of the parameter pass reduces in eight
+// loads per lane.
+__host__ __device__ inline int tokens_per_wave(int length) { return 64 * ((length + 64 * 512 - 1) / (64 * 512)); }
+__host__ __device__ inline int range_chunks(int length) {
+  const int per_wave = tokens_per_wave(length);
+  return (length + per_wave - 1) / per_wave;
+}
+
+__host__ __device__ inline int summation_threads(int length) { return length <= 256 ? 128 : 512; }
+
+// Tokens held by the four consecutive packed positions starting at p0 (multiple of 4).
+__device__ __forceinline__ int first_token_of_positions(int p0) {
+  const int pos = p0 & 31;
+  const int h = pos >> 4;
+  const int b = (pos & 15) >> 2;
+  return (p0 & ~31) + 8 * b + 4 * h;
+}
+
+// grid (ceil(chunks/4), B*H), 256 threads: one wavefront per chunk of
+// tokens_per_wave(length) tokens.  A token row is dim/8 lanes wide (8 channels =
+// 16 bytes of a 16-bit input per lane), so every load instruction of the wavefront
+// covers whole consecutive rows; the lanes holding the same channels are combined
+// with xor shuffles at the end.  min/max do not depend on the order.
+template <int DT, bool AFFINE>
+__device__ __forceinline__ void value_range_block(const void* __restrict__ v, float* __restrict__ part_max,
+                                                  float* __restrict__ part_min, int length, int dim,
+                                                  int heads, int chunks, int64_t stride_b,
+                                                  int64_t stride_h, int64_t stride_n, int chunk_group,
+                                                  int bh) {
+  const int b = bh / heads, h = bh - b * heads;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int chunk = chunk_group * 4 + wave;
+  if (chunk >= chunks) return;
+  const int octets = dim / 8;
+  const int octet = lane % octets, row = lane / octets, rows_per_load = 64 / octets;
+  const int per_wave = tokens_per_wave(length);
+  const int64_t base = static_cast<int64_t>(b) * stride_b + static_cast<int64_t>(h) * stride_h;
+  float mx[8], mn[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    mx[i] = AFFINE ? -FLT_MAX : 0.0f;
+    mn[i] = FLT_MAX;
+  }
+  const int first = chunk * per_wave;
+#pragma unroll 8
+  for (int t = row; t < per_wave; t += rows_per_load) {
+    const int n = first + t;
+    if (n < length) {
+      float x[8];
+      load8<DT>(v, base + static_cast<int64_t>(n) * stride_n + octet * 8, x);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        if constexpr (AFFINE) {
+          mx[i] = __builtin_fmaxf(mx[i], x[i]);
+          mn[i] = __builtin_fminf(mn[i], x[i]);
+        } else {
+          mx[i] = __builtin_fmaxf(mx[i], __builtin_fabsf(x[i]));
+        }
+      }
+    }
+  }
+  for (int offset = octets; offset < 64; offset <<= 1) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      mx[i] = __builtin_fmaxf(mx[i], __shfl_xor(mx[i], offset));
+      if constexpr (AFFINE) mn[i] = __builtin_fminf(mn[i], __shfl_xor(mn[i], offset));
+    }
+  }
+  if (lane < octets) {
+    const int64_t slot = (static_cast<int64_t>(bh) * chunks + chunk) * dim + octet * 8;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      part_max[slot + i] = mx[i];
+      if constexpr (AFFINE) part_min[slot + i] = mn[i];
+    }
+  }
+}
+
+template <int DT, bool AFFINE>
+__global__ __launch_bounds__(256) void value_range_kernel(const void* __restrict__ v,
+                                                          float* __restrict__ part_max,
+                                                          float* __restrict__ part_min, int length,
+                                                          int dim, int heads, int chunks,
+                                                          int64_t stride_b, int64_t stride_h,
+                                                          int64_t stride_n) {
+  value_range_block<DT, AFFINE>(v, part_max, part_min, length, dim, heads, chunks, stride_b, stride_h,
+                                stride_n, blockIdx.x, blockIdx.y);
+}
+
+// grid (ceil(B*H*dim/8 / 4)), 256 threads: one wavefront per (batch, head, 8
+// channels); lanes stride over the partial ranges, xor shuffles combine them.
+template <bool AFFINE>
+__global__ __launch_bounds__(256) void value_params_kernel(const float* __restrict__ part_max,
+                                                           const float* __restrict__ part_min,
+                                                           float* __restrict__ scale,
+                                                           float* __restrict__ center,
+                                                           float* __restrict__ inverse,
+                                                           float* __restrict__ midpoint, int dim,
+                                                           int chunks, int groups) {
+  const int lane = threadIdx.x & 63;
+  const int group = blockIdx.x * 4 + (threadIdx.x >> 6);  // (b*H + h) * dim/8 + octet
+  if (group >= groups) return;
+  const int octets = dim / 8;
+  const int bh = group / octets, octet = group - bh * octets;
+  float mx[8], mn[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    mx[i] = AFFINE ? -FLT_MAX : 0.0f;
+    mn[i] = FLT_MAX;
+  }
+  for (int chunk = lane; chunk < chunks; chunk += 64) {
+    const int64_t slot = (static_cast<int64_t>(bh) * chunks + chunk) * dim + octet * 8;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      mx[i] = __builtin_fmaxf(mx[i], part_max[slot + i]);
+      if constexpr (AFFINE) mn[i] = __builtin_fminf(mn[i], part_min[slot + i]);
+    }
+  }
+#pragma unroll
+  for (int offset = 32; offset > 0; offset >>= 1) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      mx[i] = __builtin_fmaxf(mx[i], __shfl_xor(mx[i], offset));
+      if constexpr (AFFINE) mn[i] = __builtin_fminf(mn[i], __shfl_xor(mn[i], offset));
+    }
+  }
+  if (lane < 8) {
+    const int row = group * 8 + lane;
+    float hi = mx[0], lo = mn[0];
+#pragma unroll
+    for (int i = 1; i < 8; ++i) {
+      hi = lane == i ? mx[i] : hi;
+      lo = lane == i ? mn[i] : lo;
+    }
+    const float mid = AFFINE ? 0.5f * (lo + hi) : 0.0f;
+    const float radius = AFFINE ? 0.5f * (hi - lo) : hi;
+    const float sc = __builtin_fmaxf(radius * (1.0f / 127.0f), 1e-12f);
+    scale[row] = sc;
+    inverse[row] = 1.0f / sc;
+    midpoint[row] = mid;
+    if constexpr (!AFFINE) center[row] = 0.0f;
+  }
+}
+
+// grid (ceil(padded/256), B*H, dim/32), 256 threads.  Lane l of every wave owns the
+// four packed positions 256*blockIdx.x + 4*l .. +3 (four consecutive tokens); wave
+// w of the workgroup takes the eight channels 32*blockIdx.z + 8*w .. +7.
+//
+// PARAMS says where the per-channel scale and midpoint come from: kParamsStored reads
+// what value_params_kernel left; kParamsAbsmax / kParamsAffine reduce the partial
+// ranges (at most 64 of them, one per lane) inside every wavefront, which saves a
+// launch for short sequences; the workgroups of the first 256 positions also store
+// the parameters for the kernels that follow.
+constexpr int kParamsStored = 0, kParamsAbsmax = 1, kParamsAffine = 2;
+
+struct FusedParams {
+  const float* part_max;
+  const float* part_min;
+  float* scale;
+  float* center;
+  float* inverse;
+  float* midpoint;
+  int chunks;
+};
+
+template <int DT, int CTA_K, int PARAMS>
+__device__ __forceinline__ void value_codes_block(const void* __restrict__ v, int8_t* __restrict__ codes,
+                                                  int32_t* __restrict__ tile_sum,
+                                                  const float* __restrict__ inverse,
+                                                  const float* __restrict__ midpoint, int length,
+                                                  int padded, int dim, int heads, int64_t stride_b,
+                                                  int64_t stride_h, int64_t stride_n,
+                                                  const int32_t* __restrict__ permutation,
+                                                  const FusedParams& fused, int position_block, int bh,
+                                                  int channel_block) {
+  const int b = bh / heads, h = bh - b * heads;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int p0 = position_block * 256 + lane * 4;
+  const int n0 = first_token_of_positions(p0);
+  const int64_t base = static_cast<int64_t>(b) * stride_b + static_cast<int64_t>(h) * stride_h;
+  const int tiles = padded / CTA_K;
+  {
+    const int octet = channel_block * 4 + wave;
+    const int64_t row0 = static_cast<int64_t>(bh) * dim + octet * 8;
+    float inv[8], mid[8];
+    if constexpr (PARAMS == kParamsStored) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        inv[i] = inverse[row0 + i];
+        mid[i] = midpoint[row0 + i];
+      }
+    } else {
+      constexpr bool AFFINE = PARAMS == kParamsAffine;
+      float mx[8], mn[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        mx[i] = AFFINE ? -FLT_MAX : 0.0f;
+        mn[i] = FLT_MAX;
+      }
+      if (lane < fused.chunks) {
+        const int64_t slot = (static_cast<int64_t>(bh) * fused.chunks + lane) * dim + octet * 8;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          mx[i] = fused.part_max[slot + i];
+          if constexpr (AFFINE) mn[i] = fused.part_min[slot + i];
+        }
+      }
+#pragma unroll
+      for (int offset = 32; offset > 0; offset >>= 1) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          mx[i] = __builtin_fmaxf(mx[i], __shfl_xor(mx[i], offset));
+          if constexpr (AFFINE) mn[i] = __builtin_fminf(mn[i], __shfl_xor(mn[i], offset));
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        mid[i] = AFFINE ? 0.5f * (mn[i] + mx[i]) : 0.0f;
+        const float radius = AFFINE ? 0.5f * (mx[i] - mn[i]) : mx[i];
+        const float sc = __builtin_fmaxf(radius * (1.0f / 127.0f), 1e-12f);
+        inv[i] = 1.0f / sc;
+        if (position_block == 0 && lane == i) {
+          fused.scale[row0 + i] = sc;
+          fused.inverse[row0 + i] = inv[i];
+          fused.midpoint[row0 + i] = mid[i];
+          if constexpr (!AFFINE) fused.center[row0 + i] = 0.0f;
+        }
+      }
+    }
+    int q[8][4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int n = n0 + r;
+      if (n < length) {
+        const int from = permutation != nullptr ? permutation[static_cast<int64_t>(bh) * length + n] : n;
+        float x[8];
+        load8<DT>(v, base + static_cast<int64_t>(from) * stride_n + octet * 8, x);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) q[i][r] = quantize_s8((x[i] - mid[i]) * inv[i]);
+      } else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) q[i][r] = 0;
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      if (p0 < padded) {
+        *reinterpret_cast<uint32_t*>(codes + (row0 + i) * padded + p0) =
+            pack_s8x4(q[i][0], q[i][1], q[i][2], q[i][3]);
+      }
+      int sum = q[i][0] + q[i][1] + q[i][2] + q[i][3];
+#pragma unroll
+      for (int offset = CTA_K / 8; offset > 0; offset >>= 1) sum += __shfl_xor(sum, offset);
+      if ((lane & (CTA_K / 4 - 1)) == 0 && p0 < padded) {
+        tile_sum[(static_cast<int64_t>(bh) * tiles + p0 / CTA_K) * dim + octet * 8 + i] =
+            sum * 128 + kAccumulatorSeedBits;
+      }
+    }
+  }
+}
+
+template <int DT, int CTA_K, int PARAMS>
+__global__ __launch_bounds__(256) void value_codes_kernel(const void* __restrict__ v,
+                                                          int8_t* __restrict__ codes,
+                                                          int32_t* __restrict__ tile_sum,
+                                                          const float* __restrict__ inverse,
+                                                          const float* __restrict__ midpoint,
+                                                          int length, int padded, int dim, int heads,
+                                                          int64_t stride_b, int64_t stride_h,
+                                                          int64_t stride_n,
+                                                          const int32_t* __restrict__ permutation,
+                                                          FusedParams fused) {
+  value_codes_block<DT, CTA_K, PARAMS>(v, codes, tile_sum, inverse, midpoint, length, padded, dim,
+                                       heads, stride_b, stride_h, stride_n, permutation, fused,
+                                       blockIdx.x, blockIdx.y, blockIdx.z);
+}
+
+// grid (T / (256/octets), B*H), 256 threads: thread = (summation thread t, octet).
+template <int DT>
+__global__ __launch_bounds__(256) void value_residual_kernel(const void* __restrict__ v,
+                                                             float* __restrict__ partial,
+                                                             const float* __restrict__ inverse,
+                                                             const float* __restrict__ midpoint,
+                                                             int length, int dim, int heads,
+                                                             int threads, int64_t stride_b,
+                                                             int64_t stride_h, int64_t stride_n,
+                                                             const int32_t* __restrict__ permutation) {
+  const int bh = blockIdx.y;
+  const int b = bh / heads, h = bh - b * heads;
+  const int octets = dim / 8;
+  const int octet = threadIdx.x % octets;
+  const int t = blockIdx.x * (256 / octets) + threadIdx.x / octets;
+  const int64_t base = static_cast<int64_t>(b) * stride_b + static_cast<int64_t>(h) * stride_h;
+  const int64_t row0 = static_cast<int64_t>(bh) * dim + octet * 8;
+  float inv[8], mid[8], residual[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    inv[i] = inverse[row0 + i];
+    mid[i] = midpoint[row0 + i];
+    residual[i] = 0.0f;
+  }
+  for (int src = length - 1 - t; src >= 0; src -= threads) {
+    const int from = permutation != nullptr ? permutation[static_cast<int64_t>(bh) * length + src] : src;
+    float x[8];
+    load8<DT>(v, base + static_cast<int64_t>(from) * stride_n + octet * 8, x);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const float normalized = (x[i] - mid[i]) * inv[i];
+      const float code = static_cast<float>(quantize_s8(normalized));
+      residual[i] += normalized - code;
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < 8; ++i) partial[(row0 + i) * threads + t] = residual[i];
+}
+
+__global__ void value_center_kernel(const float* __restrict__ partial,
+                                    const float* __restrict__ inverse,
+                                    const float* __restrict__ midpoint, float* __restrict__ center,
+                                    int rows, int threads, int length) {
+  const int row = blockIdx.x * blockDim.x + threadIdx.x;
+  if (row >= rows) return;
+  const float* p = partial + static_cast<int64_t>(row) * threads;
+  float total = 0.0f;
+  for (int w = 0; w < threads / 32; ++w) {
+    float t[32];
+#pragma unroll
+    for (int i = 0; i < 32; ++i) t[i] = p[w * 32 + i];
+#pragma unroll
+    for (int offset = 16; offset > 0; offset >>= 1) {
+#pragma unroll
+      for (int i = 0; i < offset; ++i) t[i] = t[i] + t[i + offset];
+    }
+    total += t[0];
+  }
+  const float scale = 1.0f / inverse[row];
+  const float mean = total / static_cast<float>(length);
+  const float correction = scale * mean;
+  center[row] = midpoint[row] + correction;
+}
+
+// grid (ceil(padded/256), rows_bh), 256 threads: accumulator seeds of already packed codes.
+template <int CTA_K>
+__global__ __launch_bounds__(256) void value_tile_sum_kernel(const int8_t* __restrict__ codes,
+                                                             int32_t* __restrict__ tile_sum, int dim,
+                                                             int padded) {
+  const int bh = blockIdx.y;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int p0 = blockIdx.x * 256 + lane * 4;
+  const int tiles = padded / CTA_K;
+  for (int c = wave; c < dim; c += 4) {
+    int sum = 0;
+    if (p0 < padded) {
+      const uint32_t word =
+          *reinterpret_cast<const uint32_t*>(codes + (static_cast<int64_t>(bh) * dim + c) * padded + p0);
+      sum = static_cast<int8_t>(word & 0xff) + static_cast<int8_t>((word >> 8) & 0xff) +
+            static_cast<int8_t>((word >> 16) & 0xff) + static_cast<int8_t>(word >> 24);
+    }
+#pragma unroll
+    for (int offset = CTA_K / 8; offset > 0; offset >>= 1) sum += __shfl_xor(sum, offset);
+    if ((lane & (CTA_K / 4 - 1)) == 0 && p0 < padded) {
+      tile_sum[(static_cast<int64_t>(bh) * tiles + p0 / CTA_K) * dim + c] = sum * 128 + kAccumulatorSeedBits;
+    }
+  }
+}
+
+struct Workspace {
+  float* part_max;
+  float* part_min;
+  float* inverse;
+  float* midpoint;
+  float* partial;
+  size_t bytes;
+};
+
+Workspace carve(void* base, int batch, int heads, int length, int dim, bool affine) {
+  const size_t bh = static_cast<size_t>(batch) * heads;
+  const size_t chunks = range_chunks(length);
+  const size_t rows = bh * dim;
+  float* p = static_cast<float*>(base);
+  Workspace w{};
+  size_t offset = 0;
+  w.part_max = p + offset;
+  offset += bh * chunks * dim;
+  w.part_min = p + offset;
+  offset += affine ? bh * chunks * dim : 0;
+  w.inverse = p + offset;
+  offset += rows;
+  w.midpoint = p + offset;
+  offset += rows;
+  w.partial = p + offset;
+  offset += affine ? rows * summation_threads(length) : 0;
+  w.bytes = offset * sizeof(float);
+  return w;
+}
+
+}  // namespace
+}  // namespace risa
