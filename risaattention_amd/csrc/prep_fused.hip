@@ -87,16 +87,10 @@ void launch_stages(const FusedArgs& a, hipStream_t stream) {
   if (a.v.midpoint_affine) {
     prepare_stage1_kernel<DT, DK, ROT, true><<<stage1_blocks, 256, 0, stream>>>(a);
     prepare_stage2_kernel<DT, DK, CTA_K, ROT, kParamsAffine><<<stage2_blocks, 256, 0, stream>>>(a);
-    const int threads = summation_threads(a.v.length);
-    const int per_block = 256 / (a.v.head_dim / 8);
-    const int rows = a.kv * a.v.head_dim;
-    dim3 residual_grid(threads / per_block, a.kv);
-    value_residual_kernel<DT><<<residual_grid, 256, 0, stream>>>(
-        a.v.v, a.partial, a.inverse, a.midpoint, a.v.length,
-        a.v.head_dim, a.v.heads, threads, a.v.stride_b, a.v.stride_h, a.v.stride_n, nullptr);
-    value_center_kernel<<<(rows + 63) / 64, 64, 0, stream>>>(
-        a.partial, a.inverse, a.midpoint, a.v.center, rows, threads,
-        a.v.length);
+    dim3 center_grid(a.v.head_dim / 8, a.kv);
+    value_center_fused_kernel<DT><<<center_grid, summation_threads(a.v.length), 0, stream>>>(
+        a.v.v, a.inverse, a.midpoint, a.v.center, a.v.length, a.v.head_dim, a.v.heads, a.v.stride_b,
+        a.v.stride_h, a.v.stride_n, nullptr);
   } else {
     prepare_stage1_kernel<DT, DK, ROT, false><<<stage1_blocks, 256, 0, stream>>>(a);
     prepare_stage2_kernel<DT, DK, CTA_K, ROT, kParamsAbsmax><<<stage2_blocks, 256, 0, stream>>>(a);

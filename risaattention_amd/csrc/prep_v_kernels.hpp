@@ -13,9 +13,9 @@
 //   1. value_range_kernel     partial min/max per (wavefront chunk of 64+ tokens, channel)
 //   2. value_params_kernel    scale, midpoint and reciprocal per channel
 //   3. value_codes_kernel     codes + packed transposed store + tile sums
-//   4. value_residual_kernel  (affine) per-summation-thread residual sums in the
-//                             reference's order: thread t adds tokens L-1-t-k*T
-//   5. value_center_kernel    (affine) xor-tree per 32 threads, warps in order
+//   4. value_center_kernel    (affine) per-summation-thread residual sums in the
+//                             reference's order (thread t adds tokens L-1-t-k*T),
+//                             tree per 32 threads, warps in order
 // min/max are order independent, so 1-3 are exact for any split; 4-5 keep the
 // floating-point summation order explicitly.
 
@@ -40,6 +40,8 @@ __host__ __device__ inline int range_chunks(int length) {
 }
 
 __host__ __device__ inline int summation_threads(int length) { return length <= 256 ? 128 : 512; }
+// up to this many tokens the residual sums and the centre are one launch
+constexpr int kFusedCenterMaxLength = 4096;
 
 // Tokens held by the four consecutive packed positions starting at p0 (multiple of 4).
 __device__ __forceinline__ int first_token_of_positions(int p0) {
@@ -347,7 +349,7 @@ __global__ __launch_bounds__(256) void value_residual_kernel(const void* __restr
   for (int i = 0; i < 8; ++i) partial[(row0 + i) * threads + t] = residual[i];
 }
 
-__global__ void value_center_kernel(const float* __restrict__ partial,
+__global__ void value_center_from_partials_kernel(const float* __restrict__ partial,
                                     const float* __restrict__ inverse,
                                     const float* __restrict__ midpoint, float* __restrict__ center,
                                     int rows, int threads, int length) {
@@ -370,6 +372,63 @@ __global__ void value_center_kernel(const float* __restrict__ partial,
   const float mean = total / static_cast<float>(length);
   const float correction = scale * mean;
   center[row] = midpoint[row] + correction;
+}
+
+// One-launch form of the two kernels above for short sequences (a workgroup reads 16
+// bytes of every row, which wastes cache lines once the sequence is long).
+// Residual-corrected centre of the midpoint_affine mode (reference
+// quantize_v_impl.cuh:233-275).  grid (dim/8, B*H), `threads` threads (512, or 128
+// for at most 256 tokens): thread t is the reference's summation thread t for the
+// eight channels of the workgroup.  It adds the residuals of tokens L-1-t-k*threads
+// (k ascending); every 32 threads combine with the reference's tree (t[i] += t[i+16],
+// +8, +4, +2, +1: a shuffle-down), and the warp totals are added in warp order.
+template <int DT>
+__global__ __launch_bounds__(512) void value_center_fused_kernel(const void* __restrict__ v,
+                                                           const float* __restrict__ inverse,
+                                                           const float* __restrict__ midpoint,
+                                                           float* __restrict__ center, int length,
+                                                           int dim, int heads, int64_t stride_b,
+                                                           int64_t stride_h, int64_t stride_n,
+                                                           const int32_t* __restrict__ permutation) {
+  __shared__ float warp_total[8][16];
+  const int octet = blockIdx.x, bh = blockIdx.y;
+  const int b = bh / heads, h = bh - b * heads;
+  const int t = threadIdx.x, threads = blockDim.x;
+  const int64_t base = static_cast<int64_t>(b) * stride_b + static_cast<int64_t>(h) * stride_h;
+  const int64_t row0 = static_cast<int64_t>(bh) * dim + octet * 8;
+  float inv[8], mid[8], residual[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    inv[i] = inverse[row0 + i];
+    mid[i] = midpoint[row0 + i];
+    residual[i] = 0.0f;
+  }
+  for (int src = length - 1 - t; src >= 0; src -= threads) {
+    const int from = permutation != nullptr ? permutation[static_cast<int64_t>(bh) * length + src] : src;
+    float x[8];
+    load8<DT>(v, base + static_cast<int64_t>(from) * stride_n + octet * 8, x);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const float normalized = (x[i] - mid[i]) * inv[i];
+      const float code = static_cast<float>(quantize_s8(normalized));
+      residual[i] += normalized - code;
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+#pragma unroll
+    for (int offset = 16; offset > 0; offset >>= 1) residual[i] += __shfl_down(residual[i], offset, 32);
+    if ((t & 31) == 0) warp_total[i][t >> 5] = residual[i];
+  }
+  __syncthreads();
+  if (t < 8) {
+    float total = 0.0f;
+    for (int w = 0; w < threads / 32; ++w) total += warp_total[t][w];
+    const float scale = 1.0f / inverse[row0 + t];
+    const float mean = total / static_cast<float>(length);
+    const float correction = scale * mean;
+    center[row0 + t] = midpoint[row0 + t] + correction;
+  }
 }
 
 // grid (ceil(padded/256), rows_bh), 256 threads: accumulator seeds of already packed codes.
