@@ -280,13 +280,13 @@ def main():
     parser.add_argument("--no-cpu-baseline", action="store_true")
     parser.add_argument("--no-accuracy", action="store_true")
     parser.add_argument("--workload", default="dense", choices=["dense", "sweep", "masked", "sparse", "video"],
-                        help="dense = headline N=32K line (default); the others are the remaining BASELINE.json "
-                             "configurations, reported as one JSON line each")
+                        help="dense = headline N=32K line (default); the others are the remaining benchmark "
+                             "configurations of the reference, reported as one JSON line each")
     parser.add_argument("--calibrate-copy", action="store_true",
                         help="only run a 1 GiB device copy (reference point for rocprofv3 FETCH_SIZE/WRITE_SIZE)")
     args = parser.parse_args()
     if args.gpus != 1:
-        print("bench.py measures one MI355X; this path uses no second GPU (see DESIGN.md on sharding)",
+        print("bench.py measures one MI355X; this path uses no second GPU",
               file=sys.stderr)
         sys.exit(2)
 

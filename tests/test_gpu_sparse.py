@@ -16,7 +16,8 @@ pytestmark = pytest.mark.gpu
 
 
 def block_structured(batch, q_heads, kv_heads, length, dim, groups, seed, dtype=torch.bfloat16):
-    """Per-group centroid*3 plus unit noise for Q/K, unit-noise V (BASELINE sparse config)."""
+    """Per-group centroid*3 plus unit noise for Q/K, unit-noise V (the block-structured
+    inputs of the sparse-reuse benchmark)."""
     g = torch.Generator().manual_seed(seed)
     centroids = torch.randn(batch, kv_heads, groups, dim, generator=g) * 3
     per_token = centroids.repeat_interleave(length // groups, dim=2)
