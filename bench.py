@@ -7,7 +7,7 @@ include quantisation (reference README.md:102-106).  The JSON line reports
 dense-equivalent TOPS (4*B*Hq*Lq*Lk*D operations per call, reference
 benchmarks/plot_scaling.py:66-75), the roofline fraction of the attention
 kernel against the dense INT8 MFMA peak, and the numpy oracle timed on the host
-cores on a bounded sample (N=1024) as the CPU baseline.
+cores on a bounded sample (N=2048) as the CPU baseline.
 """
 
 from __future__ import annotations
@@ -236,8 +236,9 @@ def workload_video(torch, risa, args, device):
             "loop_speedup_vs_dense": round(10 * dense_ms / (construct_ms + sum(reuse)), 3)}
 
 
-def cpu_baseline(length=1024, calls=3):
-    """Oracle (numpy port of the quantised pipeline) on the host cores, N=1024."""
+def cpu_baseline(length=2048, calls=5):
+    """Oracle (numpy port of the quantised pipeline) on the host cores: a bounded sample
+    of the headline workload (same heads and head dim, N=2048; about ten seconds)."""
     import numpy as np
     import torch
 
