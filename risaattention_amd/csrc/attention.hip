@@ -13,6 +13,8 @@ namespace risa {
 template <> int launch_attention_variant<64>(const KernelParams&, int, bool, bool, bool, hipStream_t);
 template <> int launch_attention_variant<128>(const KernelParams&, int, bool, bool, bool, hipStream_t);
 template <> int launch_attention_variant<256>(const KernelParams&, int, bool, bool, bool, hipStream_t);
+int launch_attention_narrow(const KernelParams& p, int head_dim, int cta_k, hipStream_t stream);
+int narrow_attention_limit();
 
 namespace {
 
@@ -157,8 +159,15 @@ int launch_attention(const AttentionArgs& a, hipStream_t stream) {
   const bool indexed = p.index_mode != 0;
   const bool fast = a.mask == nullptr && !a.is_causal && a.sm_scale > 0.0f;
 
+  // A launch that cannot give every compute unit more than one workgroup runs the
+  // raw-score path with sixteen queries per wavefront (two wavefronts per SIMD).
+  const int64_t workgroups = static_cast<int64_t>(p.n_qb) * a.q_heads * a.batch;
+  const bool narrow = fast && !indexed && !capture && workgroups <= narrow_attention_limit();
+
   int status;
-  if (a.head_dim == 64)
+  if (narrow)
+    status = launch_attention_narrow(p, a.head_dim, a.cta_k, stream);
+  else if (a.head_dim == 64)
     status = launch_attention_variant<64>(p, a.cta_k, fast, indexed, capture, stream);
   else if (a.head_dim == 128)
     status = launch_attention_variant<128>(p, a.cta_k, fast, indexed, capture, stream);

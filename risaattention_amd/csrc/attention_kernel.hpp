@@ -39,6 +39,7 @@ namespace risa {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
+typedef float v4f __attribute__((ext_vector_type(4)));
 
 constexpr float kLog2e = 1.44269504088896340736f;
 constexpr float kU8Offset = 7.9943534f;
@@ -469,8 +470,11 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void attention_kernel(cons
 #pragma unroll
           for (int b4 = 0; b4 < 4; ++b4) {
             const int local = rb * 32 + b4 * 8 + half * 4;
-            const float4 bias = *reinterpret_cast<const float4*>(bias_row + local);
-            const float terms[4] = {bias.x, bias.y, bias.z, bias.w};
+            // A plain vector type on purpose: the compiler orders an LDS read it cannot
+            // classify (HIP's float4 is a struct) behind every outstanding copy into LDS,
+            // which would wait for the next tile in the middle of this one.
+            const v4f bias = *reinterpret_cast<const v4f*>(bias_row + local);
+            const float terms[4] = {bias[0], bias[1], bias[2], bias[3]};
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
               float value = static_cast<float>(s[rb][b4 * 4 + r]) * ((r & 2) ? sc1 : sc0) + terms[r];

@@ -1,0 +1,393 @@
+// Raw-score attention kernel for launches with fewer workgroups than compute units.
+//
+// Same arithmetic as risa::attention_kernel<D, CTA_K, true, false, false, -1>
+// (reference csrc/kernels/attention_int8.cuh:145-1026, unmasked non-causal path) on the
+// same operands, with the 128 queries of a workgroup spread over eight wavefronts of
+// sixteen queries instead of four of thirty-two.  A lone 256-thread workgroup leaves
+// one wavefront per SIMD, which issues a vector instruction only every other slot;
+// eight wavefronts put two on every SIMD with half the work each.  Measured on
+// B=1, H=16, D=128: 19 -> 17 us at 512 tokens, 29 -> 27.5 us at 1024, 47 -> 40.5 us at
+// 2048; what remains per tile is the dependent chain barrier -> LDS -> MFMA -> row
+// maximum -> exp2 -> MFMA.  On a full machine the wide kernel is the faster one (fewer
+// vector instructions per score, half the LDS operand traffic).
+//
+// Matrix instruction: v_mfma_i32_16x16x64_i8.  Lane l = 16*g + c feeds row/column c
+// with the sixteen bytes [16*g, 16*g + 16) of the 64-deep product and receives rows
+// 4*g .. 4*g + 3 of column c.
+//   * S^T = K · Q^T per 16-key block: A = 16 K rows from LDS, B = Q rows in registers.
+//     Row r of block (s, b) (s: 64-key step, b: 0..3) is key 64*s + 8*b + 32*(r/8) + r%8,
+//     so that lane group g ends up with keys 64*s + 32*(g/2) + 8*b + 4*(g%2) + i,
+//     i = 0..3: packing the four blocks b of a step gives sixteen bytes that sit at
+//     positions 16*g + 4*b + i of the step, exactly where the packed V matrix
+//     (risa::packed_value_position) keeps those tokens.
+//   * O^T = V^T · P^T per 16-channel block: A = 16 V rows (channels) from LDS, one
+//     16-byte read per 64-key step, B = the packed probabilities, no shuffle.
+#pragma once
+
+#include "attention_kernel.hpp"
+
+namespace risa {
+
+constexpr int kNarrowThreads = 512;
+
+// XOR applied to the 16-byte chunk index of K row `row` in LDS.  The sixteen rows a
+// matrix instruction reads are two runs of eight consecutive keys 32 apart; folding
+// bit 5 of the row into the swizzle keeps their sixteen chunks in distinct banks.
+template <int ROWBYTES> __device__ __forceinline__ int narrow_key_swizzle(int row) {
+  constexpr int CH = ROWBYTES / 16;
+  constexpr int ROWS_PER_256 = 256 / ROWBYTES;
+  return ((row / ROWS_PER_256) ^ ((row >> 5) * (8 / ROWS_PER_256))) & (CH - 1);
+}
+
+template <int D, int CTA_K>
+__global__ __launch_bounds__(kNarrowThreads) void attention_narrow_kernel(const KernelParams p) {
+  using Shape = TileShape<D, CTA_K>;
+  constexpr int KB = CTA_K / 16;  // 16-key blocks per tile
+  constexpr int SB = CTA_K / 64;  // 64-key steps of the P·V product
+  constexpr int CB = D / 16;      // 16-channel blocks
+  constexpr int KK = D / 64;      // 64-channel steps of the score product
+  constexpr int WAVES = kNarrowThreads / 64;
+  constexpr int COPIES = Shape::kTileBytes / 1024;  // 1 KB copy instructions per operand tile
+  constexpr int NC = (COPIES + WAVES - 1) / WAVES;
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int ql = lane & 15, grp = lane >> 4;
+
+  const int bx = blockIdx.x % p.n_qb;
+  const int rest = blockIdx.x / p.n_qb;
+  const int head = rest % p.q_heads;
+  const int batch = rest / p.q_heads;
+  const int kv_head = head / (p.q_heads / p.kv_heads);
+  const int64_t bhk = static_cast<int64_t>(batch) * p.kv_heads + kv_head;
+  const int64_t bhq = static_cast<int64_t>(batch) * p.q_heads + head;
+
+  const int8_t* k_base = p.k + bhk * p.k_len * D;
+  const int8_t* v_base = p.v + bhk * D * p.padded;
+  const int32_t* sum_base = p.v_tile_sum + bhk * p.n_kb * D;
+  const float* ks_base = p.k_scale + bhk * p.n_kb * 4;
+
+  const int query = bx * kQueryBlock + wave * 16 + ql;
+  const bool query_ok = query < p.q_len;
+  const int n_it = p.n_kb;
+
+  // --- copies HBM/L2 -> LDS ---------------------------------------------------------
+  // Copy instruction (wave*NC + i) fills LDS bytes [(wave*NC + i)*1024, +1024) of a
+  // tile; this lane supplies chunk `lane` of that kilobyte.
+  uint32_t k_src_offset[NC], v_src_offset[NC];
+#pragma unroll
+  for (int i = 0; i < NC; ++i) {
+    const int slot = (wave * NC + i) * 64 + lane;
+    {
+      constexpr int CH = D / 16;
+      const int row = slot / CH, phys = slot % CH;
+      k_src_offset[i] = row * D + ((phys ^ narrow_key_swizzle<D>(row)) << 4);
+    }
+    {
+      constexpr int CH = CTA_K / 16;
+      const int row = slot / CH, phys = slot % CH;
+      const int chunk = phys ^ ((row / (256 / CTA_K)) & (CH - 1));
+      v_src_offset[i] = static_cast<uint32_t>(row) * static_cast<uint32_t>(p.padded) + chunk * 16;
+    }
+  }
+  // The tail tile re-reads row 0 for keys past the end; those scores are masked by
+  // index.  The last two wavefronts add one copy each: the accumulator seeds and the
+  // four K scales of the tile.
+  const bool copies_tiles = wave * NC < COPIES;
+  auto issue_tile = [&](int tile, int stage) {
+    unsigned char* k_slot = lds + stage * Shape::kStageBytes + wave * (NC * 1024);
+    unsigned char* v_slot = k_slot + Shape::kTileBytes;
+    unsigned char* sl = lds + stage * Shape::kStageBytes + 2 * Shape::kTileBytes;
+    const int8_t* k_tile = k_base + static_cast<int64_t>(tile) * CTA_K * D;
+    const int8_t* v_tile = v_base + static_cast<int64_t>(tile) * CTA_K;
+    const int keys_left = p.k_len - tile * CTA_K;
+    if (copies_tiles) {
+      if (keys_left >= CTA_K) {
+#pragma unroll
+        for (int i = 0; i < NC; ++i) copy16_to_lds_uniform(k_tile, k_src_offset[i], k_slot + i * 1024);
+      } else {
+        const uint32_t bytes_left = static_cast<uint32_t>(keys_left) * D;
+#pragma unroll
+        for (int i = 0; i < NC; ++i) {
+          const uint32_t offset = k_src_offset[i] < bytes_left ? k_src_offset[i] : (k_src_offset[i] & (D - 1));
+          copy16_to_lds_uniform(k_tile, offset, k_slot + i * 1024);
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < NC; ++i) copy16_to_lds_uniform(v_tile, v_src_offset[i], v_slot + i * 1024);
+    }
+    if (wave == WAVES - 1) {
+      if (lane < D / 4) {
+        copy16_to_lds_uniform(reinterpret_cast<const int8_t*>(sum_base + static_cast<int64_t>(tile) * D),
+                              static_cast<uint32_t>(lane) * 16, sl);
+      }
+    } else if (wave == WAVES - 2) {
+      if (lane == 0) {
+        copy16_to_lds_uniform(reinterpret_cast<const int8_t*>(ks_base + static_cast<int64_t>(tile) * 4), 0u,
+                              sl + Shape::kSeedBytes);
+      }
+    }
+  };
+  // Read as a plain vector type: the compiler orders LDS reads it cannot classify
+  // behind every outstanding copy into LDS, i.e. behind the next tile.
+  auto tile_scales = [&](int stage, float& ks0, float& ks1) {
+    typedef float v2f __attribute__((ext_vector_type(2)));
+    const v2f pair = *reinterpret_cast<const v2f*>(lds + stage * Shape::kStageBytes + 2 * Shape::kTileBytes +
+                                                   Shape::kSeedBytes + 8 * (grp & 1));
+    ks0 = pair[0];
+    ks1 = pair[1];
+  };
+
+  // --- Q operand and scales ----------------------------------------------------------
+  v4i qreg[KK];
+  {
+    const int8_t* q_row = p.q + (bhq * p.q_len + query) * D;
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) {
+      qreg[kk] = query_ok ? *reinterpret_cast<const v4i*>(q_row + kk * 64 + grp * 16) : v4i{0, 0, 0, 0};
+    }
+  }
+  constexpr int W = D == 256 ? 16 : 32;
+  const int q_groups = (p.q_len + 127) / 128 * (128 / W) * 8;
+  const float q_scale = query_ok ? p.q_scale[bhq * q_groups + (query / W) * 8 + (query & 7)] : 1.0f;
+  const float qs2 = p.sm2;
+
+  float o_acc[CB][4];
+#pragma unroll
+  for (int cb = 0; cb < CB; ++cb)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) o_acc[cb][i] = 0.0f;
+  float m_run = kRowFloor;
+  float d_part = 0.0f;  // this lane's quarter of the row denominator
+  float seed_value;
+  asm volatile("v_mov_b32 %0, %1" : "=v"(seed_value) : "s"(kAccumulatorSeedBits));
+
+  // ---- S^T = K · Q^T ------------------------------------------------------------------
+  const int key_row = 32 * (ql >> 3) + (ql & 7);  // row of this lane inside block (s, b): + 64*s + 8*b
+  auto load_k_fragments = [&](const unsigned char* kl, int kk, v4i (&frag)[KB]) {
+#pragma unroll
+    for (int kb = 0; kb < KB; ++kb) {
+      const int row = (kb >> 2) * 64 + (kb & 3) * 8 + key_row;
+      frag[kb] = *reinterpret_cast<const v4i*>(
+          kl + row * D + (((kk * 4 + grp) ^ narrow_key_swizzle<D>(row)) << 4));
+    }
+  };
+  auto score_tile = [&](int stage, v4i (&first)[KB], v4i (&s)[KB]) {
+    const unsigned char* kl = lds + stage * Shape::kStageBytes;
+    v4i frag[2][KB];
+#pragma unroll
+    for (int kb = 0; kb < KB; ++kb) frag[0][kb] = first[kb];
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) {
+      if (kk + 1 < KK) load_k_fragments(kl, kk + 1, frag[(kk + 1) & 1]);
+#pragma unroll
+      for (int kb = 0; kb < KB; ++kb) {
+        if (kk == 0) {
+          const v4i zero = {0, 0, 0, 0};
+          s[kb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(frag[kk & 1][kb], qreg[kk], zero, 0, 0, 0);
+        } else {
+          s[kb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(frag[kk & 1][kb], qreg[kk], s[kb], 0, 0, 0);
+        }
+      }
+    }
+  };
+
+  // ---- scores -> U8 probabilities (as signed bytes) and the online-softmax state ------
+  // Element (kb, i) is key tile*CTA_K + (kb/4)*64 + 32*(grp/2) + (kb%4)*8 + 4*(grp%2) + i,
+  // K scale group (key % 8) / 2 = 2*(grp%2) + i/2.
+  constexpr float kRescaleSlack = 8.0f;
+  auto softmax_tile = [&](auto last_tag, int tile, float ks0, float ks1, v4i (&s)[KB], v4i (&pk)[SB]) -> float {
+    constexpr bool LAST = decltype(last_tag)::value;
+    const float sc0 = qs2 * (q_scale * ks0);
+    const float sc1 = qs2 * (q_scale * ks1);
+    float tile_m;
+    uint32_t row_sum = 0;
+    if constexpr (!LAST) {
+      int mx0 = s[0][0], mx1 = s[0][2];
+#pragma unroll
+      for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          if (i & 2)
+            mx1 = max(mx1, s[kb][i]);
+          else
+            mx0 = max(mx0, s[kb][i]);
+        }
+      tile_m = __builtin_fmaxf(__builtin_fmaf(static_cast<float>(mx0), sc0, -kU8Offset),
+                               __builtin_fmaf(static_cast<float>(mx1), sc1, -kU8Offset));
+    } else {
+      // Last tile: out-of-range keys become -1e30 and every scale group's maximum
+      // starts from -50000 before scaling.
+      const int key0 = tile * CTA_K + 32 * (grp >> 1) + 4 * (grp & 1);
+      float mx0 = kRowFloor, mx1 = kRowFloor;
+#pragma unroll
+      for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int key = key0 + (kb >> 2) * 64 + (kb & 3) * 8 + i;
+          const float raw = key < p.k_len ? static_cast<float>(s[kb][i]) : -1.0e30f;
+          s[kb][i] = __float_as_int(raw);
+          if (i & 2)
+            mx1 = __builtin_fmaxf(mx1, raw);
+          else
+            mx0 = __builtin_fmaxf(mx0, raw);
+        }
+      tile_m = __builtin_fmaxf(__builtin_fmaf(mx0, sc0, -kU8Offset), __builtin_fmaf(mx1, sc1, -kU8Offset));
+    }
+    tile_m = __builtin_fmaxf(tile_m, __shfl_xor(tile_m, 16));
+    tile_m = __builtin_fmaxf(tile_m, __shfl_xor(tile_m, 32));
+    const float neg_m = -tile_m;
+#pragma unroll
+    for (int kb = 0; kb < KB; ++kb) {
+      uint32_t packed = 0;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float raw = LAST ? __int_as_float(s[kb][i]) : static_cast<float>(s[kb][i]);
+        const float x = __builtin_fmaf(raw, (i & 2) ? sc1 : sc0, neg_m);
+        packed = __builtin_amdgcn_cvt_pk_u8_f32(__builtin_amdgcn_exp2f(x), i, packed);
+      }
+      row_sum = __builtin_amdgcn_udot4(packed, 0x01010101u, row_sum, false);
+      pk[kb >> 2][kb & 3] = static_cast<int>(packed ^ 0x80808080u);
+    }
+
+    // The running reference only moves when a tile maximum exceeds it by more than
+    // kRescaleSlack (the same deferred rescaling as the wide kernel).
+    const bool raise = tile_m > m_run + kRescaleSlack;
+    if (__builtin_amdgcn_ballot_w64(raise) != 0) {
+      const float o_scale = raise ? __builtin_amdgcn_exp2f(m_run - tile_m) : 1.0f;
+      m_run = raise ? tile_m : m_run;
+      d_part *= o_scale;
+#pragma unroll
+      for (int cb = 0; cb < CB; ++cb)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) o_acc[cb][i] *= o_scale;
+    }
+    const float t_scale = __builtin_amdgcn_exp2f(tile_m - m_run);
+    d_part = __builtin_fmaf(static_cast<float>(row_sum), t_scale, d_part);
+    return t_scale;
+  };
+
+  // ---- O^T += t_scale * (128*sum(V) + V^T · P_s8^T) -------------------------------------
+  // Channel blocks go through in groups of four independent accumulator chains; the
+  // seeds and V fragments of the next group are requested before this group's MFMAs.
+  constexpr int GROUP = 4;
+  constexpr int NG = CB / GROUP;
+  constexpr int SETS = NG > 2 ? 3 : 2;
+  auto load_group = [&](int stage, int g, v4i (&acc)[GROUP], v4i (&frag)[GROUP][SB]) {
+    const unsigned char* vl = lds + stage * Shape::kStageBytes + Shape::kTileBytes;
+    const int* sl = reinterpret_cast<const int*>(lds + stage * Shape::kStageBytes + 2 * Shape::kTileBytes);
+#pragma unroll
+    for (int j = 0; j < GROUP; ++j) {
+      const int cb = g * GROUP + j;
+      acc[j] = *reinterpret_cast<const v4i*>(sl + cb * 16 + grp * 4);
+#pragma unroll
+      for (int sb = 0; sb < SB; ++sb)
+        frag[j][sb] = *reinterpret_cast<const v4i*>(vl + swizzled<CTA_K>(cb * 16 + ql, sb * 4 + grp));
+    }
+  };
+  auto unseed = [&](int bits) { return __int_as_float(bits) - seed_value; };
+  auto fold_group = [&](int g, const v4i (&acc)[GROUP], float t_scale) {
+#pragma unroll
+    for (int j = 0; j < GROUP; ++j)
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        o_acc[g * GROUP + j][i] = __builtin_fmaf(unseed(acc[j][i]), t_scale, o_acc[g * GROUP + j][i]);
+  };
+  auto value_tile = [&](int stage, const v4i (&pk)[SB], v4i (&acc0)[GROUP], v4i (&frag0)[GROUP][SB], float t_scale) {
+    v4i acc[SETS][GROUP];
+    v4i frag[2][GROUP][SB];
+#pragma unroll
+    for (int j = 0; j < GROUP; ++j) {
+      acc[0][j] = acc0[j];
+#pragma unroll
+      for (int sb = 0; sb < SB; ++sb) frag[0][j][sb] = frag0[j][sb];
+    }
+#pragma unroll
+    for (int g = 0; g < NG; ++g) {
+      if (g + 1 < NG) load_group(stage, g + 1, acc[(g + 1) % SETS], frag[(g + 1) & 1]);
+#pragma unroll
+      for (int sb = 0; sb < SB; ++sb)
+#pragma unroll
+        for (int j = 0; j < GROUP; ++j)
+          acc[g % SETS][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(frag[g & 1][j][sb], pk[sb], acc[g % SETS][j], 0, 0, 0);
+      if (g > 0) fold_group(g - 1, acc[(g - 1) % SETS], t_scale);
+    }
+    fold_group(NG - 1, acc[(NG - 1) % SETS], t_scale);
+  };
+
+  // --- main loop: one barrier per tile ---------------------------------------------------
+  // At the barrier of iteration t every wave has finished tile t-1 (so stage (t+1)&1
+  // may be overwritten) and has seen its own share of tile t land.  A deeper pipeline
+  // (four stages, counted waits) was measured and gains nothing: the tile time is set
+  // by the dependent chain barrier -> LDS -> MFMA -> row maximum -> exp2 -> MFMA.
+  if (n_it > 0) {
+    v4i s[KB];
+    v4i pk[SB];
+    v4i k_first[KB];
+    v4i acc_first[GROUP];
+    v4i v_first[GROUP][SB];
+    float ks0, ks1;
+    issue_tile(0, 0);
+    for (int tile = 0; tile < n_it - 1; ++tile) {
+      const int stage = tile & 1;
+      __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
+      __syncthreads();
+      load_k_fragments(lds + stage * Shape::kStageBytes, 0, k_first);
+      tile_scales(stage, ks0, ks1);
+      issue_tile(tile + 1, stage ^ 1);
+      score_tile(stage, k_first, s);
+      load_group(stage, 0, acc_first, v_first);
+      __builtin_amdgcn_sched_barrier(0);
+      const float t_scale = softmax_tile(std::false_type{}, tile, ks0, ks1, s, pk);
+      __builtin_amdgcn_sched_barrier(0);
+      value_tile(stage, pk, acc_first, v_first, t_scale);
+    }
+    const int stage = (n_it - 1) & 1;
+    __builtin_amdgcn_s_waitcnt(0x0f70);
+    __syncthreads();
+    load_k_fragments(lds + stage * Shape::kStageBytes, 0, k_first);
+    tile_scales(stage, ks0, ks1);
+    score_tile(stage, k_first, s);
+    const float t_scale = softmax_tile(std::true_type{}, n_it - 1, ks0, ks1, s, pk);
+    load_group(stage, 0, acc_first, v_first);
+    value_tile(stage, pk, acc_first, v_first, t_scale);
+  }
+
+  // ---- epilogue ---------------------------------------------------------------------------
+  float d_total = d_part + __shfl_xor(d_part, 16);
+  d_total += __shfl_xor(d_total, 32);
+  const float inv_d = 1.0f / d_total;
+  if (query_ok) {
+    const float* vs = p.v_scale + bhk * D;
+    const float* vc = p.v_center + bhk * D;
+    unsigned char* out_row = static_cast<unsigned char*>(p.out) +
+                             2 * (batch * p.out_stride_b + head * p.out_stride_h +
+                                  static_cast<int64_t>(query) * p.out_stride_n);
+#pragma unroll
+    for (int cb = 0; cb < CB; ++cb) {
+      const int c = cb * 16 + grp * 4;
+      const float4 scale4 = *reinterpret_cast<const float4*>(vs + c);
+      const float4 center4 = *reinterpret_cast<const float4*>(vc + c);
+      float value[4];
+      value[0] = __builtin_fmaf(o_acc[cb][0] * inv_d, scale4.x, center4.x);
+      value[1] = __builtin_fmaf(o_acc[cb][1] * inv_d, scale4.y, center4.y);
+      value[2] = __builtin_fmaf(o_acc[cb][2] * inv_d, scale4.z, center4.z);
+      value[3] = __builtin_fmaf(o_acc[cb][3] * inv_d, scale4.w, center4.w);
+      uint32_t bits[4];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) bits[r] = p.out_dtype == kF16 ? to_f16_bits(value[r]) : to_bf16_bits(value[r]);
+      uint2 word;
+      word.x = bits[0] | (bits[1] << 16);
+      word.y = bits[2] | (bits[3] << 16);
+      *reinterpret_cast<uint2*>(out_row + 2 * c) = word;
+    }
+    if (p.lse != nullptr && grp == 0) {
+      p.lse[bhq * p.q_len + query] =
+          d_total > 0.0f ? (__builtin_amdgcn_logf(d_total) + m_run) / kLog2e : -__builtin_inff();
+    }
+  }
+}
+
+}  // namespace risa

@@ -239,3 +239,28 @@ def test_causal_launch_order_covers_every_block(risa):
     prepared = oracle_prequantize(q, k, v, is_causal=True)
     expected, _, _ = oracle_pipeline.attend(prepared)
     assert relative_l2(to_numpy(out), expected) < TOLERANCE
+
+
+@pytest.mark.parametrize("dim", [64, 128, 256])
+@pytest.mark.parametrize("k_len", [263, 1153])
+def test_both_unmasked_kernels_match_oracle(risa, dim, k_len):
+    """Unmasked launches with no more workgroups than the GPU has compute units run
+    sixteen queries per wavefront, larger ones thirty-two.  264 query heads go through
+    the second kernel, a slice of 66 of them through the first; both must agree with
+    the oracle on that slice and with each other everywhere."""
+    heads, kv_heads, q_len = 264, 4, 40
+    group = heads // kv_heads
+    assert heads > torch.cuda.get_device_properties(0).multi_processor_count >= group
+    q = seeded((1, heads, q_len, dim), torch.bfloat16, 61)
+    k = seeded((1, kv_heads, k_len, dim), torch.bfloat16, 62)
+    v = seeded((1, kv_heads, k_len, dim), torch.bfloat16, 63, offset=0.5)
+    wide, wide_lse = risa.int8_attention(q, k, v, return_lse=True)
+    for kv in range(kv_heads):
+        rows = slice(kv * group, (kv + 1) * group)
+        narrow, narrow_lse = risa.int8_attention(q[:, rows], k[:, kv:kv + 1], v[:, kv:kv + 1], return_lse=True)
+        assert relative_l2(to_numpy(narrow), to_numpy(wide[:, rows])) < 1e-4
+        assert relative_l2(to_numpy(narrow_lse), to_numpy(wide_lse[:, rows])) < 1e-6
+    prepared = oracle_prequantize(q[:, :group], k[:, :1], v[:, :1], return_lse=True)
+    expected, expected_lse, _ = oracle_pipeline.attend(prepared, return_lse=True)
+    assert relative_l2(to_numpy(wide[:, :group]), expected) < TOLERANCE
+    assert relative_l2(to_numpy(wide_lse[:, :group]), expected_lse) < TOLERANCE
