@@ -264,3 +264,19 @@ def test_both_unmasked_kernels_match_oracle(risa, dim, k_len):
     expected, expected_lse, _ = oracle_pipeline.attend(prepared, return_lse=True)
     assert relative_l2(to_numpy(wide[:, :group]), expected) < TOLERANCE
     assert relative_l2(to_numpy(wide_lse[:, :group]), expected_lse) < TOLERANCE
+
+
+@pytest.mark.parametrize("length,heads", [(4096, 16), (4422, 30), (4608, 32)])
+@pytest.mark.parametrize("mode", ["absmax", "midpoint_affine"])
+def test_lse_request_does_not_change_outputs(risa, length, heads, mode):
+    """reference tests/cuda/test_probability_mass.py:158-170 (image-sized query tiles):
+    the same packed tensors give bit-identical outputs with and without the LSE."""
+    torch.manual_seed(59)
+    q = torch.randn(1, heads, length, 128, device="cuda", dtype=torch.bfloat16)
+    k, v = [torch.randn(1, 2, length, 128, device="cuda", dtype=q.dtype) for _ in range(2)]
+    packed = risa.prequantize_int8_attention(q, k, v, v_quantization=mode, return_lse=True)
+    plain = risa.int8_attention_from_prequantized(packed)
+    with_lse, lse = risa.int8_attention_from_prequantized(packed, return_lse=True)
+    assert torch.equal(plain, with_lse)
+    assert torch.isfinite(lse).all()
+    assert torch.equal(plain, risa.int8_attention(q, k, v, v_quantization=mode))

@@ -142,3 +142,34 @@ def test_fused_permutation_matches_materialized_gather(risa, dtype, layout, mode
     out = risa.int8_attention(q, k, v, kv_permutation=permutation, v_quantization=mode)
     expected = risa.int8_attention_from_prequantized(plain)
     assert torch.equal(out, expected)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("layout", ["hnd", "token_major", "interleaved"])
+@pytest.mark.parametrize("length", [1490, 14850])
+def test_value_codes_do_not_depend_on_schedule(risa, dtype, layout, length):
+    """reference tests/cuda/test_probability_mass.py:111-145: V codes and scales of one
+    head are the same whether it is quantised alone or among 56 heads, for every memory
+    layout; the two lengths take the one-pass and the chunked range reduction."""
+    heads, channels = 56, 128
+    q = torch.randn(1, heads, 17, channels, device="cuda", dtype=dtype)
+    if layout == "hnd":
+        k, v = [torch.randn(1, heads, length, channels, device="cuda", dtype=dtype) for _ in range(2)]
+    elif layout == "token_major":
+        k, v = [torch.randn(1, length, heads, channels, device="cuda", dtype=dtype).transpose(1, 2)
+                for _ in range(2)]
+    else:
+        combined = torch.randn(1, length, 3, heads, channels, device="cuda", dtype=dtype)
+        k, v = (combined[:, :, index].transpose(1, 2) for index in (1, 2))
+    for mode in ("absmax", "midpoint_affine"):
+        wide = risa.prequantize_int8_attention(q, k, v, v_quantization=mode)
+        narrow = risa.prequantize_int8_attention(q[:, :1], k[:, :1], v[:, :1], v_quantization=mode)
+        padded = wide.v.shape[-1]
+        assert torch.equal(wide.v.reshape(1, heads, channels, padded)[:, :1],
+                           narrow.v.reshape(1, 1, channels, padded))
+        assert torch.equal(wide.v_scale.reshape(1, heads, channels)[:, :1],
+                           narrow.v_scale.reshape(1, 1, channels))
+        assert torch.equal(wide.v_center.reshape(1, heads, channels)[:, :1],
+                           narrow.v_center.reshape(1, 1, channels))
+        assert torch.equal(wide.k[:, :1], narrow.k)
+        assert torch.equal(wide.k_scale[:, :1], narrow.k_scale)

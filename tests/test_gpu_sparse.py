@@ -232,3 +232,91 @@ def test_full_size_invariants(risa):
     rows = slice(1000, 1128)
     scores = q[:, :4, rows].float() @ k[:, :1].float().transpose(-1, -2) / 128**0.5
     torch.testing.assert_close(lse[:, :4, rows], scores.logsumexp(-1), atol=0.02, rtol=0)
+
+
+@pytest.mark.parametrize("mode", ["absmax", "midpoint_affine"])
+def test_key_mask_skipping_stream_and_graph(risa, mode):
+    """reference tests/cuda/test_key_mask_tiles.py:57-76: constant V under a key mask that
+    hides whole tiles, on a side stream, eagerly and from a captured graph."""
+    q = torch.randn(1, 4, 513, 128, device="cuda", dtype=torch.float16)
+    k = torch.randn(1, 2, 2049, 128, device="cuda", dtype=q.dtype)
+    v = torch.full_like(k, 2.75)
+    mask = torch.ones(1, 1, 1, 2049, device="cuda", dtype=torch.bool)
+    mask[..., 128:1536] = False
+    stream = torch.cuda.Stream()
+    stream.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(stream):
+        for _ in range(3):
+            output = risa.int8_attention(q, k, v, attn_mask=mask, v_quantization=mode)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            captured = risa.int8_attention(q, k, v, attn_mask=mask, v_quantization=mode)
+        for _ in range(3):
+            captured.zero_()
+            graph.replay()
+            stream.synchronize()
+            assert torch.equal(captured, output)
+    torch.cuda.current_stream().wait_stream(stream)
+    assert torch.equal(output, v[..., :513, :].repeat_interleave(2, dim=1))
+
+
+@pytest.mark.parametrize("inference", [False, True])
+def test_key_mask_metadata_and_mask_mutation(risa, inference):
+    """reference tests/cuda/test_key_mask_tiles.py:79-104: the packed container keeps the
+    caller's mask tensor, not a copy; the tile list is rebuilt from its current
+    contents on every call."""
+    from risaattention_amd.key_mask import prepare_key_mask_tiles
+
+    q = torch.randn(1, 4, 257, 128, device="cuda", dtype=torch.bfloat16)
+    k = torch.randn(1, 2, 1153, 128, device="cuda", dtype=q.dtype)
+    v = torch.randn_like(k)
+    mask = torch.ones(1, 1, 1, 1153, device="cuda", dtype=torch.bool)
+    if inference:
+        with torch.inference_mode():
+            mask = mask.clone()
+    with torch.inference_mode():
+        mask[..., :512] = False
+    packed = risa.prequantize_int8_attention(q, k, v, attn_mask=mask)
+    tiles = prepare_key_mask_tiles(packed.attn_mask, packed.cta_k, 257, packed.attention_scale, False)
+    expected = torch.tensor([4, 5, 6, 7, 8, 9], device="cuda", dtype=torch.int32)
+    assert torch.equal(tiles[..., :6], expected.expand(1, 4, 6))
+    assert (tiles[..., -1] == 6).all()
+    with torch.inference_mode():
+        mask.fill_(True)
+    actual = risa.int8_attention_from_prequantized(packed)
+    generic = risa.int8_attention_from_prequantized(replace(packed, attn_mask=packed.attn_mask.clone()))
+    assert torch.equal(actual, generic)
+    # An all-true mask takes the pre-scaled path, no mask the raw-score path: same
+    # codes, different FP32 rounding order.
+    unmasked = risa.int8_attention_from_prequantized(replace(packed, attn_mask=None))
+    assert relative_l2(to_numpy(actual), to_numpy(unmasked)) < 1e-2
+
+
+@pytest.mark.parametrize("mode", ["absmax", "midpoint_affine"])
+def test_prequantized_mask_mutation_during_graph_replay(risa, mode):
+    """reference tests/cuda/test_key_mask_tiles.py:107-123: a mask emptied after capture
+    empties the replayed output."""
+    with torch.inference_mode():
+        q = torch.randn(1, 4, 257, 128, device="cuda", dtype=torch.bfloat16)
+        k = torch.randn(1, 2, 1153, 128, device="cuda", dtype=q.dtype)
+        v = torch.full_like(k, 2.75)
+        mask = torch.ones(1, 1, 1, 1153, device="cuda", dtype=torch.bool)
+        mask[..., :768] = False
+        packed = risa.prequantize_int8_attention(q, k, v, attn_mask=mask, v_quantization=mode)
+        for _ in range(3):
+            eager = risa.int8_attention_from_prequantized(packed)
+        assert torch.equal(eager, v[..., :257, :].repeat_interleave(2, dim=1))
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            captured = risa.int8_attention_from_prequantized(packed)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(captured, eager)
+        mask.fill_(False)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.count_nonzero(captured) == 0
+        mask[..., 900:] = True
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(captured, eager)
