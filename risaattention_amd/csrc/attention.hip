@@ -10,9 +10,9 @@
 
 namespace risa {
 
-template <> int launch_attention_variant<64>(const KernelParams&, int, bool, bool, bool, hipStream_t);
-template <> int launch_attention_variant<128>(const KernelParams&, int, bool, bool, bool, hipStream_t);
-template <> int launch_attention_variant<256>(const KernelParams&, int, bool, bool, bool, hipStream_t);
+template <> int launch_attention_variant<64>(const KernelParams&, int, bool, bool, bool, bool, hipStream_t);
+template <> int launch_attention_variant<128>(const KernelParams&, int, bool, bool, bool, bool, hipStream_t);
+template <> int launch_attention_variant<256>(const KernelParams&, int, bool, bool, bool, bool, hipStream_t);
 int launch_attention_narrow(const KernelParams& p, int head_dim, int cta_k, hipStream_t stream);
 int narrow_attention_limit();
 
@@ -111,6 +111,7 @@ int launch_attention(const AttentionArgs& a, hipStream_t stream) {
   p.mask_stride_q = a.mask_stride_q;
   p.mask_stride_k = a.mask_stride_k;
   p.mask_dtype = a.mask != nullptr ? a.mask_dtype : -1;
+  bool mask_vector = false;
   if (a.mask != nullptr) {
     // Groups of four keys start at multiples of four, so one load per group needs
     // unit key stride, the other strides multiples of four elements and the base
@@ -118,7 +119,7 @@ int launch_attention(const AttentionArgs& a, hipStream_t stream) {
     const int64_t element = a.mask_dtype == kF32 ? 4 : a.mask_dtype == kBool ? 1 : 2;
     const bool aligned = reinterpret_cast<uintptr_t>(a.mask) % (4 * element) == 0 &&
                          ((a.mask_stride_b | a.mask_stride_h | a.mask_stride_q) & 3) == 0;
-    p.mask_vector = a.mask_stride_k == 1 && aligned ? 1 : 0;
+    mask_vector = a.mask_stride_k == 1 && aligned;
     if (a.key_bias != nullptr) {
       if (a.mask_stride_q != 0) return fail("risa_attention: a key bias row needs a key-only mask");
       if (reinterpret_cast<uintptr_t>(a.key_bias) % 16 != 0 || (a.key_bias_stride_b | a.key_bias_stride_h) % 4 != 0)
@@ -168,11 +169,11 @@ int launch_attention(const AttentionArgs& a, hipStream_t stream) {
   if (narrow)
     status = launch_attention_narrow(p, a.head_dim, a.cta_k, stream);
   else if (a.head_dim == 64)
-    status = launch_attention_variant<64>(p, a.cta_k, fast, indexed, capture, stream);
+    status = launch_attention_variant<64>(p, a.cta_k, fast, indexed, capture, mask_vector, stream);
   else if (a.head_dim == 128)
-    status = launch_attention_variant<128>(p, a.cta_k, fast, indexed, capture, stream);
+    status = launch_attention_variant<128>(p, a.cta_k, fast, indexed, capture, mask_vector, stream);
   else if (a.head_dim == 256)
-    status = launch_attention_variant<256>(p, a.cta_k, fast, indexed, capture, stream);
+    status = launch_attention_variant<256>(p, a.cta_k, fast, indexed, capture, mask_vector, stream);
   else
     return fail("risa_attention: unsupported head_dim");
   if (status != 0) return status;

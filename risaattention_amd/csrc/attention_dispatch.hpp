@@ -6,13 +6,13 @@
 
 namespace risa {
 
-template <int D> int launch_attention_variant(const KernelParams& p, int cta_k, bool fast,
-                                              bool indexed, bool capture, hipStream_t stream);
+template <int D> int launch_attention_variant(const KernelParams& p, int cta_k, bool fast, bool indexed,
+                                              bool capture, bool mask_vector, hipStream_t stream);
 
-template <int D, int CTA_K, bool FAST, bool INDEXED, bool CAPTURE, int MASK_DT>
+template <int D, int CTA_K, bool FAST, bool INDEXED, bool CAPTURE, int MASK_DT, bool MASK_VEC = false>
 int launch_one(const KernelParams& p, hipStream_t stream) {
   using Shape = TileShape<D, CTA_K>;
-  auto kernel = attention_kernel<D, CTA_K, FAST, INDEXED, CAPTURE, MASK_DT>;
+  auto kernel = attention_kernel<D, CTA_K, FAST, INDEXED, CAPTURE, MASK_DT, MASK_VEC>;
   // The dynamic LDS limit is a per-device property of the function; setting it
   // again is cheap and keeps the launcher free of host-side caches.
   static thread_local int configured_device = -1;
@@ -32,25 +32,37 @@ int launch_one(const KernelParams& p, hipStream_t stream) {
   return 0;
 }
 
-template <int D, int CTA_K, int MASK_DT>
+template <int D, int CTA_K, int MASK_DT, bool MASK_VEC = false>
 int launch_general(const KernelParams& p, bool indexed, bool capture, hipStream_t stream) {
-  if (capture) return launch_one<D, CTA_K, false, false, true, MASK_DT>(p, stream);
-  if (indexed) return launch_one<D, CTA_K, false, true, false, MASK_DT>(p, stream);
-  return launch_one<D, CTA_K, false, false, false, MASK_DT>(p, stream);
+  if (capture) return launch_one<D, CTA_K, false, false, true, MASK_DT, MASK_VEC>(p, stream);
+  if (indexed) return launch_one<D, CTA_K, false, true, false, MASK_DT, MASK_VEC>(p, stream);
+  return launch_one<D, CTA_K, false, false, false, MASK_DT, MASK_VEC>(p, stream);
+}
+
+// Mask tensors read per score.  One load per group of four keys when the tensor allows
+// it (`vector`); only for 64-key tiles, the tile every query-dependent mask runs with
+// (a key-only mask given without its bias row still works, element by element).
+template <int D, int CTA_K, int MASK_DT>
+int launch_masked(const KernelParams& p, bool vector, bool indexed, bool capture, hipStream_t stream) {
+  if constexpr (CTA_K == 64) {
+    if (vector) return launch_general<D, CTA_K, MASK_DT, true>(p, indexed, capture, stream);
+  }
+  return launch_general<D, CTA_K, MASK_DT, false>(p, indexed, capture, stream);
 }
 
 template <int D, int CTA_K>
-int launch_tile(const KernelParams& p, bool fast, bool indexed, bool capture, hipStream_t stream) {
+int launch_tile(const KernelParams& p, bool fast, bool indexed, bool capture, bool mask_vector,
+                hipStream_t stream) {
   if (fast) {
     if (capture) return launch_one<D, CTA_K, true, false, true, -1>(p, stream);
     if (indexed) return launch_one<D, CTA_K, true, true, false, -1>(p, stream);
     return launch_one<D, CTA_K, true, false, false, -1>(p, stream);
   }
   switch (p.mask_dtype) {
-    case kBool: return launch_general<D, CTA_K, kBool>(p, indexed, capture, stream);
-    case kF32: return launch_general<D, CTA_K, kF32>(p, indexed, capture, stream);
-    case kF16: return launch_general<D, CTA_K, kF16>(p, indexed, capture, stream);
-    case kBF16: return launch_general<D, CTA_K, kBF16>(p, indexed, capture, stream);
+    case kBool: return launch_masked<D, CTA_K, kBool>(p, mask_vector, indexed, capture, stream);
+    case kF32: return launch_masked<D, CTA_K, kF32>(p, mask_vector, indexed, capture, stream);
+    case kF16: return launch_masked<D, CTA_K, kF16>(p, mask_vector, indexed, capture, stream);
+    case kBF16: return launch_masked<D, CTA_K, kBF16>(p, mask_vector, indexed, capture, stream);
     case kKeyBias: return launch_general<D, CTA_K, kKeyBias>(p, indexed, capture, stream);
     default: return launch_general<D, CTA_K, -1>(p, indexed, capture, stream);
   }
@@ -59,11 +71,12 @@ int launch_tile(const KernelParams& p, bool fast, bool indexed, bool capture, hi
 #define RISA_DEFINE_ATTENTION_VARIANT(DIM)                                                        \
   template <>                                                                                     \
   int launch_attention_variant<DIM>(const KernelParams& p, int cta_k, bool fast, bool indexed,    \
-                                    bool capture, hipStream_t stream) {                           \
+                                    bool capture, bool mask_vector, hipStream_t stream) {         \
     if constexpr (DIM != 64) {                                                                    \
-      if (cta_k == 128) return launch_tile<DIM, 128>(p, fast, indexed, capture, stream);          \
+      if (cta_k == 128)                                                                           \
+        return launch_tile<DIM, 128>(p, fast, indexed, capture, mask_vector, stream);             \
     }                                                                                             \
-    return launch_tile<DIM, 64>(p, fast, indexed, capture, stream);                               \
+    return launch_tile<DIM, 64>(p, fast, indexed, capture, mask_vector, stream);                  \
   }
 
 }  // namespace risa

@@ -59,7 +59,6 @@ struct KernelParams {
   const void* mask;
   int64_t mask_stride_b, mask_stride_h, mask_stride_q, mask_stride_k;
   int mask_dtype;  // -1: no mask
-  int mask_vector;  // keys are contiguous and groups of four keys aligned: one load per group
   const float* key_bias;  // key-only mask as an additive row [Bm,Hm,padded] (mask_dtype kKeyBias)
   int64_t key_bias_stride_b, key_bias_stride_h;
   int q_len, k_len, q_heads, kv_heads, padded, n_kb, n_qb, batch;
@@ -129,10 +128,14 @@ template <int D, int CTA_K> struct TileShape {
 
 // MASK_DT: element type of the mask tensor (risa::kBool, kF32, kF16, kBF16), kKeyBias
 // for a key-only mask prepared as an FP32 row, or -1 for none; FAST (raw-score path)
-// implies -1.
-template <int D, int CTA_K, bool FAST, bool INDEXED, bool CAPTURE, int MASK_DT>
+// implies -1.  MASK_VEC: the mask tensor allows one load per group of four keys (unit
+// key stride, aligned rows); a template parameter and not a run-time branch so that the
+// tile loop holds one unrolled mask path instead of two and stays inside the
+// instruction cache.
+template <int D, int CTA_K, bool FAST, bool INDEXED, bool CAPTURE, int MASK_DT, bool MASK_VEC>
 __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void attention_kernel(const KernelParams p) {
   static_assert(!FAST || MASK_DT < 0, "the raw-score path takes no mask");
+  static_assert(!MASK_VEC || (MASK_DT >= 0 && MASK_DT != kKeyBias), "vector loads need a mask tensor");
   using Shape = TileShape<D, CTA_K>;
   constexpr int RB = CTA_K / 32;  // 32-key blocks per tile
   constexpr int CB = D / 32;      // 32-channel blocks
@@ -330,6 +333,43 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void attention_kernel(cons
                 static_cast<int64_t>(query) * p.mask_stride_q
           : 0;
 
+  // Mask elements of a full tile, requested before the next tile's copies.  Vector
+  // memory operations complete in order: a mask load issued after the copies can only
+  // be consumed once they have landed, which stalls the softmax of this tile on the
+  // operands of the next one.  Requested first, it is waited for with the copies still
+  // in flight.  Used for query-dependent masks (always 64-key tiles, where the
+  // registers are there) that allow one load per group of four keys; not for FP32
+  // masks with head dim 64, where the 32 extra registers cost a resident wavefront.
+  constexpr bool PRELOAD = MASK_VEC && CTA_K == 64 && !(MASK_DT == kF32 && D == 64);
+  constexpr int WORDS = MASK_DT == kF32 ? 4 : MASK_DT == kBool ? 1 : 2;  // 32-bit words per four keys
+  constexpr bool LATE_COPIES = PRELOAD;
+  [[maybe_unused]] uint32_t mask_words[PRELOAD ? RB * 4 * WORDS : 1];
+  auto load_mask_words = [&](int tile) {
+    if constexpr (PRELOAD) {
+      constexpr int ES = MASK_DT == kF32 ? 4 : MASK_DT == kBool ? 1 : 2;
+      // Rows past the last query read the last row; their scores are discarded.
+      const int64_t row = mask_row - static_cast<int64_t>(query_ok ? 0 : query - (p.q_len - 1)) * p.mask_stride_q;
+      const unsigned char* base = static_cast<const unsigned char*>(p.mask) +
+                                  (row + tile * CTA_K + half * 4) * ES;
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+        for (int b4 = 0; b4 < 4; ++b4) {
+          const unsigned char* at = base + (rb * 32 + b4 * 8) * ES;
+          uint32_t* words = mask_words + (rb * 4 + b4) * WORDS;
+          if constexpr (WORDS == 1) {
+            words[0] = *reinterpret_cast<const uint32_t*>(at);
+          } else if constexpr (WORDS == 2) {
+            const uint2 w = *reinterpret_cast<const uint2*>(at);
+            words[0] = w.x, words[1] = w.y;
+          } else {
+            const uint4 w = *reinterpret_cast<const uint4*>(at);
+            words[0] = w.x, words[1] = w.y, words[2] = w.z, words[3] = w.w;
+          }
+        }
+    }
+  };
+
   // ---- S^T = K · Q^T for the tile staged in `stage` ---------------------------
   // The K fragments of k-step kk+1 are requested from LDS before the MFMAs of
   // k-step kk are issued, so the LDS latency hides behind RB matrix instructions.
@@ -462,33 +502,46 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void attention_kernel(cons
       } else if constexpr (MASK_DT == kKeyBias) {
         // Key-only mask: the tile's row of additive terms (already in the exp2
         // domain, -inf for hidden and out-of-range keys) sits in LDS next to the
-        // seeds; a lane reads the four consecutive keys of a group in one go.
+        // seeds; a lane reads the four consecutive keys of a group in one go.  The
+        // causal comparison is only compiled into the pass for tiles on the diagonal.
         const float* bias_row = reinterpret_cast<const float*>(
             lds + (it & 1) * Shape::kStageBytes + 2 * Shape::kTileBytes + Shape::kSeedBytes);
+        auto biased_scores = [&](auto diagonal_tag) {
+          constexpr bool DIAGONAL = decltype(diagonal_tag)::value;
 #pragma unroll
-        for (int rb = 0; rb < RB; ++rb)
+          for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
-          for (int b4 = 0; b4 < 4; ++b4) {
-            const int local = rb * 32 + b4 * 8 + half * 4;
-            // A plain vector type on purpose: the compiler orders an LDS read it cannot
-            // classify (HIP's float4 is a struct) behind every outstanding copy into LDS,
-            // which would wait for the next tile in the middle of this one.
-            const v4f bias = *reinterpret_cast<const v4f*>(bias_row + local);
-            const float terms[4] = {bias[0], bias[1], bias[2], bias[3]};
+            for (int b4 = 0; b4 < 4; ++b4) {
+              const int local = rb * 32 + b4 * 8 + half * 4;
+              // A plain vector type on purpose: the compiler orders an LDS read it cannot
+              // classify (HIP's float4 is a struct) behind every outstanding copy into LDS,
+              // which would wait for the next tile in the middle of this one.
+              const v4f bias = *reinterpret_cast<const v4f*>(bias_row + local);
+              const float terms[4] = {bias[0], bias[1], bias[2], bias[3]};
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-              float value = static_cast<float>(s[rb][b4 * 4 + r]) * ((r & 2) ? sc1 : sc0) + terms[r];
-              if (p.causal && tile * CTA_K + local + r > query) value = neg_inf;
-              s[rb][b4 * 4 + r] = __float_as_int(value);
-              mx = __builtin_fmaxf(mx, value);
+              for (int r = 0; r < 4; ++r) {
+                float value = static_cast<float>(s[rb][b4 * 4 + r]) * ((r & 2) ? sc1 : sc0) + terms[r];
+                if constexpr (DIAGONAL) {
+                  if (tile * CTA_K + local + r > query) value = neg_inf;
+                }
+                s[rb][b4 * 4 + r] = __float_as_int(value);
+                mx = __builtin_fmaxf(mx, value);
+              }
             }
-          }
+        };
+        if (on_diagonal) {
+          biased_scores(std::true_type{});
+        } else {
+          biased_scores(std::false_type{});
+        }
       } else {
         // DT: mask element type (-1: none, only the causal / key-range tests);
         // VEC: one load per group of four consecutive keys.
-        auto masked_scores = [&](auto dtype_tag, auto vector_tag) {
+        auto masked_scores = [&](auto dtype_tag, auto vector_tag, auto preloaded_tag, auto diagonal_tag) {
+          constexpr bool DIAGONAL = decltype(diagonal_tag)::value;  // causal comparison per score
           constexpr int DT = decltype(dtype_tag)::value;
           constexpr bool VEC = decltype(vector_tag)::value;
+          constexpr bool LOADED = decltype(preloaded_tag)::value;  // elements are in mask_words
           constexpr int ES = DT == kF32 ? 4 : DT == kBool ? 1 : 2;
           [[maybe_unused]] const unsigned char* lane_mask = nullptr;
           if constexpr (DT >= 0) {
@@ -504,7 +557,27 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void attention_kernel(cons
               bool keep[4] = {true, true, true, true};
               float bias[4] = {0.0f, 0.0f, 0.0f, 0.0f};
               if constexpr (DT >= 0) {
-                if (!query_ok) {
+                if constexpr (LOADED) {
+                  // Rows past the last query hold the last row's mask: they behave like
+                  // a valid row and are never stored.
+                  const uint32_t* words = mask_words + (rb * 4 + b4) * WORDS;
+                  if constexpr (DT == kBool) {
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) keep[r] = ((words[0] >> (8 * r)) & 0xffu) != 0;
+                  } else if constexpr (DT == kF32) {
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) bias[r] = __uint_as_float(words[r]);
+                  } else {
+                    const uint32_t bits16[4] = {words[0] & 0xffffu, words[0] >> 16, words[1] & 0xffffu,
+                                                words[1] >> 16};
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                      bias[r] = DT == kF16 ? static_cast<float>(__builtin_bit_cast(
+                                                 _Float16, static_cast<uint16_t>(bits16[r])))
+                                           : __uint_as_float(bits16[r] << 16);
+                    }
+                  }
+                } else if (!query_ok) {
 #pragma unroll
                   for (int r = 0; r < 4; ++r) keep[r] = false;
                 } else if (VEC && key + 3 < p.k_len) {
@@ -549,14 +622,16 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void attention_kernel(cons
               for (int r = 0; r < 4; ++r) {
                 float value = static_cast<float>(s[rb][b4 * 4 + r]) * ((r & 2) ? sc1 : sc0);
                 if constexpr (DT >= 0) value = keep[r] ? value + bias[r] * kLog2e : neg_inf;
-                if (p.causal && key + r > query) value = neg_inf;
+                if constexpr (DIAGONAL) {
+                  if (key + r > query) value = neg_inf;
+                }
                 if (LAST && key + r >= p.k_len) value = neg_inf;
                 s[rb][b4 * 4 + r] = __float_as_int(value);
                 mx = __builtin_fmaxf(mx, value);
               }
               // The mask loads of one key block at a time: all of a tile in flight
               // at once do not fit the register file.
-              if constexpr (DT >= 0) {
+              if constexpr (DT >= 0 && !LOADED) {
                 if (b4 == 3) {
                   asm volatile("" ::: "memory");
                   __builtin_amdgcn_sched_barrier(0);
@@ -565,10 +640,19 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void attention_kernel(cons
             }
         };
         using MaskType = std::integral_constant<int, MASK_DT>;
-        if (has_mask && p.mask_vector != 0) {
-          masked_scores(MaskType{}, std::true_type{});
+        auto mask_pass = [&](auto diagonal_tag) {
+          if constexpr (PRELOAD && !LAST) {
+            masked_scores(MaskType{}, std::true_type{}, std::true_type{}, diagonal_tag);
+          } else if constexpr (MASK_VEC) {
+            masked_scores(MaskType{}, std::true_type{}, std::false_type{}, diagonal_tag);
+          } else {
+            masked_scores(MaskType{}, std::false_type{}, std::false_type{}, diagonal_tag);
+          }
+        };
+        if (on_diagonal) {
+          mask_pass(std::true_type{});
         } else {
-          masked_scores(MaskType{}, std::false_type{});
+          mask_pass(std::false_type{});
         }
       }
       tile_m = mx - kU8Offset;
@@ -709,7 +793,11 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void attention_kernel(cons
       __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
       __syncthreads();
       load_k_fragments(lds + stage * Shape::kStageBytes, 0, k_first);
-      issue_tile(next_tile, stage ^ 1);
+      if constexpr (PRELOAD) {
+        load_mask_words(tile);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      if constexpr (!LATE_COPIES) issue_tile(next_tile, stage ^ 1);
       const int scale_pair = KEEP_OFFSETS ? 2 * half : (fresh_lane() >> 5) * 2;
       const float next_ks0 = ks_base[next_tile * 4 + scale_pair];
       const float next_ks1 = ks_base[next_tile * 4 + scale_pair + 1];
@@ -720,6 +808,10 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void attention_kernel(cons
         __builtin_amdgcn_sched_barrier(0);
       }
       const float t_scale = softmax_tile(std::false_type{}, it, tile, ks0, ks1, s, pk);
+      if constexpr (LATE_COPIES) {
+        __builtin_amdgcn_sched_barrier(0);
+        issue_tile(next_tile, stage ^ 1);
+      }
       if constexpr (PREFETCH) {
         __builtin_amdgcn_sched_barrier(0);
       } else {
