@@ -433,7 +433,7 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void attention_kernel(cons
         }
       tile_m = __builtin_fmaxf(__builtin_fmaf(static_cast<float>(mx0), sc0, -kU8Offset),
                                __builtin_fmaf(static_cast<float>(mx1), sc1, -kU8Offset));
-      tile_m = __builtin_fmaxf(tile_m, __shfl_xor(tile_m, 32));
+      tile_m = max_across_halves(tile_m);
       const float neg_m = -tile_m;
 #pragma unroll
       for (int rb = 0; rb < RB; ++rb)
@@ -465,7 +465,7 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void attention_kernel(cons
             mx0 = __builtin_fmaxf(mx0, raw);
         }
       tile_m = __builtin_fmaxf(__builtin_fmaf(mx0, sc0, -kU8Offset), __builtin_fmaf(mx1, sc1, -kU8Offset));
-      tile_m = __builtin_fmaxf(tile_m, __shfl_xor(tile_m, 32));
+      tile_m = max_across_halves(tile_m);
       const float neg_m = -tile_m;
 #pragma unroll
       for (int rb = 0; rb < RB; ++rb)
@@ -656,7 +656,7 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void attention_kernel(cons
         }
       }
       tile_m = mx - kU8Offset;
-      tile_m = __builtin_fmaxf(tile_m, __shfl_xor(tile_m, 32));
+      tile_m = max_across_halves(tile_m);
 #pragma unroll
       for (int rb = 0; rb < RB; ++rb)
 #pragma unroll

@@ -236,8 +236,7 @@ __global__ __launch_bounds__(kNarrowThreads) void attention_narrow_kernel(const 
         }
       tile_m = __builtin_fmaxf(__builtin_fmaf(mx0, sc0, -kU8Offset), __builtin_fmaf(mx1, sc1, -kU8Offset));
     }
-    tile_m = __builtin_fmaxf(tile_m, __shfl_xor(tile_m, 16));
-    tile_m = __builtin_fmaxf(tile_m, __shfl_xor(tile_m, 32));
+    tile_m = max_across_halves(max_across_row_pairs(tile_m));
     const float neg_m = -tile_m;
 #pragma unroll
     for (int kb = 0; kb < KB; ++kb) {

@@ -141,6 +141,21 @@ __device__ __forceinline__ uint32_t pack_s8x4(int a, int b, int c, int d) {
          ((static_cast<uint32_t>(c) & 0xffu) << 16) | ((static_cast<uint32_t>(d) & 0xffu) << 24);
 }
 
+// Maximum over lanes l and l ^ 32 (max_across_halves) or l and l ^ 16
+// (max_across_row_pairs), in both lanes, with the gfx950 lane-swap instructions: one
+// vector instruction instead of a round trip through the LDS crossbar.  With both
+// operands equal, v_permlane32_swap leaves the lower half's value in both halves of the
+// first result and the upper half's in both halves of the second; v_permlane16_swap
+// does the same for the even and odd 16-lane rows of each pair.
+__device__ __forceinline__ float max_across_halves(float x) {
+  const auto both = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return __builtin_fmaxf(__uint_as_float(both[0]), __uint_as_float(both[1]));
+}
+__device__ __forceinline__ float max_across_row_pairs(float x) {
+  const auto both = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return __builtin_fmaxf(__uint_as_float(both[0]), __uint_as_float(both[1]));
+}
+
 // Accumulator seed of the P·V product.  The matrix cores add integers to whatever
 // 32-bit pattern they start from; starting from the bits of 1.5 * 2^23 (plus the
 // zero-point term) leaves the bits of the float 12582912 + n for every result
