@@ -1,15 +1,18 @@
-// Q/K/V preparation in two launches for short sequences.
+// Q/K/V preparation in two launches (three beyond 4096 tokens).
 //
 // The separate preparation kernels (prep_qk.hip, prep_v.hip) are five to seven
 // launches whose order is fixed by data: anchor -> K codes, V range -> V parameters
 // -> V codes.  Up to a few thousand tokens every one of them runs for about five
 // microseconds however little it does, and the chain is longer than the attention
-// kernel.  The work has only two levels of dependence, so two launches are enough:
-//   stage 1  Q codes | K anchor | V partial ranges      (independent workgroups)
+// kernel; for long sequences the tail of each launch leaves most of the GPU idle.
+// The work has only two levels of dependence, so two launches are enough:
+//   stage 1  K anchor | Q codes | V partial ranges      (independent workgroups)
 //   stage 2  K codes (needs the anchor) | V codes (reduce the partial ranges themselves)
+// With more than 64 partial ranges per channel (beyond 4096 tokens) the small
+// parameter kernel runs between the stages instead of inside every code workgroup.
 // A workgroup finds its role from its index; every role runs the same device
-// function as the stand-alone kernel, so results are bit-identical.  Used when the
-// V range has at most 64 partial chunks (4096 tokens) and no permutation is given.
+// function as the stand-alone kernel, so results are bit-identical.  Used when no
+// permutation is given and K and V have the same extents.
 
 #include "prep_qk_kernels.hpp"
 #include "prep_v_kernels.hpp"
@@ -32,7 +35,15 @@ struct FusedArgs {
 
 template <int DT, int DK, int ROT, bool AFFINE>
 __global__ __launch_bounds__(256) void prepare_stage1_kernel(const FusedArgs a) {
+  // The anchor detectors go first: each is one long-running workgroup.
   int block = blockIdx.x;
+  if (block < a.anchor_blocks) {
+    detect_anchor_block<DT>(a.qk.k, a.qk.anchors, a.qk.k_len, a.qk.head_dim, a.qk.kv_heads,
+                            a.qk.k_stride_b, a.qk.k_stride_h, a.qk.k_stride_n, nullptr,
+                            block % a.qk.kv_heads, block / a.qk.kv_heads);
+    return;
+  }
+  block -= a.anchor_blocks;
   if (block < a.q_blocks) {
     const int slice = block % a.q_slices;
     const int rest = block / a.q_slices;
@@ -42,13 +53,6 @@ __global__ __launch_bounds__(256) void prepare_stage1_kernel(const FusedArgs a) 
     return;
   }
   block -= a.q_blocks;
-  if (block < a.anchor_blocks) {
-    detect_anchor_block<DT>(a.qk.k, a.qk.anchors, a.qk.k_len, a.qk.head_dim, a.qk.kv_heads,
-                            a.qk.k_stride_b, a.qk.k_stride_h, a.qk.k_stride_n, nullptr,
-                            block % a.qk.kv_heads, block / a.qk.kv_heads);
-    return;
-  }
-  block -= a.anchor_blocks;
   value_range_block<DT, AFFINE>(a.v.v, a.part_max, a.part_min, a.v.length, a.v.head_dim, a.v.heads,
                                 a.chunks, a.v.stride_b, a.v.stride_h, a.v.stride_n,
                                 block % a.range_groups, block / a.range_groups);
@@ -84,16 +88,42 @@ template <int DT, int DK, int CTA_K, int ROT>
 void launch_stages(const FusedArgs& a, hipStream_t stream) {
   const int stage1_blocks = a.q_blocks + a.anchor_blocks + a.range_groups * a.kv;
   const int stage2_blocks = a.key_blocks + a.code_blocks_x * a.kv * (a.v.head_dim / 32);
+  const bool stored_params = a.chunks > 64;
+  const int groups = a.kv * a.v.head_dim / 8;
   if (a.v.midpoint_affine) {
     prepare_stage1_kernel<DT, DK, ROT, true><<<stage1_blocks, 256, 0, stream>>>(a);
-    prepare_stage2_kernel<DT, DK, CTA_K, ROT, kParamsAffine><<<stage2_blocks, 256, 0, stream>>>(a);
-    dim3 center_grid(a.v.head_dim / 8, a.kv);
-    value_center_fused_kernel<DT><<<center_grid, summation_threads(a.v.length), 0, stream>>>(
-        a.v.v, a.inverse, a.midpoint, a.v.center, a.v.length, a.v.head_dim, a.v.heads, a.v.stride_b,
-        a.v.stride_h, a.v.stride_n, nullptr);
+    if (stored_params) {
+      value_params_kernel<true><<<(groups + 3) / 4, 256, 0, stream>>>(
+          a.part_max, a.part_min, a.v.scale, a.v.center, a.inverse, a.midpoint, a.v.head_dim, a.chunks, groups);
+      prepare_stage2_kernel<DT, DK, CTA_K, ROT, kParamsStored><<<stage2_blocks, 256, 0, stream>>>(a);
+    } else {
+      prepare_stage2_kernel<DT, DK, CTA_K, ROT, kParamsAffine><<<stage2_blocks, 256, 0, stream>>>(a);
+    }
+    if (a.v.length <= kFusedCenterMaxLength) {
+      dim3 center_grid(a.v.head_dim / 8, a.kv);
+      value_center_fused_kernel<DT><<<center_grid, summation_threads(a.v.length), 0, stream>>>(
+          a.v.v, a.inverse, a.midpoint, a.v.center, a.v.length, a.v.head_dim, a.v.heads, a.v.stride_b,
+          a.v.stride_h, a.v.stride_n, nullptr);
+    } else {
+      const int threads = summation_threads(a.v.length);
+      const int per_block = 256 / (a.v.head_dim / 8);
+      const int rows = a.kv * a.v.head_dim;
+      dim3 residual_grid(threads / per_block, a.kv);
+      value_residual_kernel<DT><<<residual_grid, 256, 0, stream>>>(
+          a.v.v, a.partial, a.inverse, a.midpoint, a.v.length, a.v.head_dim, a.v.heads, threads,
+          a.v.stride_b, a.v.stride_h, a.v.stride_n, nullptr);
+      value_center_from_partials_kernel<<<(rows + 63) / 64, 64, 0, stream>>>(
+          a.partial, a.inverse, a.midpoint, a.v.center, rows, threads, a.v.length);
+    }
   } else {
     prepare_stage1_kernel<DT, DK, ROT, false><<<stage1_blocks, 256, 0, stream>>>(a);
-    prepare_stage2_kernel<DT, DK, CTA_K, ROT, kParamsAbsmax><<<stage2_blocks, 256, 0, stream>>>(a);
+    if (stored_params) {
+      value_params_kernel<false><<<(groups + 3) / 4, 256, 0, stream>>>(
+          a.part_max, a.part_min, a.v.scale, a.v.center, a.inverse, a.midpoint, a.v.head_dim, a.chunks, groups);
+      prepare_stage2_kernel<DT, DK, CTA_K, ROT, kParamsStored><<<stage2_blocks, 256, 0, stream>>>(a);
+    } else {
+      prepare_stage2_kernel<DT, DK, CTA_K, ROT, kParamsAbsmax><<<stage2_blocks, 256, 0, stream>>>(a);
+    }
   }
 }
 
@@ -134,11 +164,11 @@ template <int DT> void launch_by_dim(const FusedArgs& a, hipStream_t stream) {
 bool can_prepare_fused(const QkArgs& qk, const ValueArgs& v) {
   return qk.permutation == nullptr && v.permutation == nullptr && qk.k_len == v.length &&
          qk.batch == v.batch && qk.kv_heads == v.heads && qk.head_dim == v.head_dim &&
-         qk.cta_k == v.cta_k && qk.dtype == v.dtype && range_chunks(v.length) <= 64;
+         qk.cta_k == v.cta_k && qk.dtype == v.dtype;
 }
 
 int launch_prepare_fused(const QkArgs& qk, const ValueArgs& v, hipStream_t stream) {
-  if (!can_prepare_fused(qk, v)) return fail("risa_sdpa: operands do not qualify for the two-launch preparation");
+  if (!can_prepare_fused(qk, v)) return fail("risa_sdpa: operands do not qualify for the fused preparation");
   if (v.workspace_bytes < value_workspace_bytes(v.batch, v.heads, v.length, v.head_dim, v.midpoint_affine))
     return fail("risa_quantize_v: workspace is too small");
   const Workspace w = carve(v.workspace, v.batch, v.heads, v.length, v.head_dim, v.midpoint_affine);
