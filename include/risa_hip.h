@@ -78,6 +78,23 @@ int risa_quantize_v(const void* v, void* out, float* scale, float* center, int32
                     const int32_t* kv_permutation, void* stream);
 
 /*
+ * Q, K and V preparation in one call.  Replaces risa_sdpa_quantize (reference
+ * csrc/bindings.cpp:195-272), which also prepares all three operands at once.
+ * Arguments as for risa_quantize_qk and risa_quantize_v (padded length =
+ * ceil(k_len / cta_k) * cta_k; the workspace is the V workspace).  Same results as
+ * the two separate calls; when no permutation is given the work runs in two
+ * launches (three beyond 4096 tokens) instead of five to seven.
+ */
+int risa_sdpa_quantize(const void* q, void* q_int8, float* q_scale, const void* k, void* k_int8,
+                       float* k_scale, const void* v, void* v_int8, float* v_scale, float* v_center,
+                       int32_t* v_tile_sum, void* v_workspace, size_t v_workspace_bytes, int batch,
+                       int q_heads, int q_len, int kv_heads, int k_len, int head_dim, int cta_k,
+                       int64_t q_stride_b, int64_t q_stride_h, int64_t q_stride_n, int64_t k_stride_b,
+                       int64_t k_stride_h, int64_t k_stride_n, int64_t v_stride_b, int64_t v_stride_h,
+                       int64_t v_stride_n, int input_dtype, int midpoint_affine,
+                       int32_t* anchor_indices, const int32_t* kv_permutation, void* stream);
+
+/*
  * Zero-point terms (128 x tile sums) of an already packed V matrix (for callers that build packed V
  * themselves, as reference tests/cuda/test_large_offsets.py:35-36 does).
  */

@@ -151,6 +151,33 @@ int risa_quantize_v(const void* v, void* out, float* scale, float* center, int32
   return risa::launch_quantize_v(a, static_cast<hipStream_t>(stream));
 }
 
+int risa_sdpa_quantize(const void* q, void* q_int8, float* q_scale, const void* k, void* k_int8,
+                       float* k_scale, const void* v, void* v_int8, float* v_scale, float* v_center,
+                       int32_t* v_tile_sum, void* v_workspace, size_t v_workspace_bytes, int batch,
+                       int q_heads, int q_len, int kv_heads, int k_len, int head_dim, int cta_k,
+                       int64_t q_stride_b, int64_t q_stride_h, int64_t q_stride_n, int64_t k_stride_b,
+                       int64_t k_stride_h, int64_t k_stride_n, int64_t v_stride_b, int64_t v_stride_h,
+                       int64_t v_stride_n, int input_dtype, int midpoint_affine,
+                       int32_t* anchor_indices, const int32_t* kv_permutation, void* stream) {
+  if (cta_k != 64 && cta_k != 128) return risa::fail("risa_sdpa_quantize: cta_k must be 64 or 128");
+  const int padded = (k_len + cta_k - 1) / cta_k * cta_k;
+  risa::QkArgs qk{};
+  int status = checked_qk_args(qk, q, q_int8, q_scale, k, k_int8, k_scale, batch, q_heads, q_len, kv_heads,
+                               k_len, head_dim, cta_k, q_stride_b, q_stride_h, q_stride_n, k_stride_b,
+                               k_stride_h, k_stride_n, input_dtype, anchor_indices, kv_permutation);
+  if (status != 0) return status;
+  risa::ValueArgs value{};
+  status = checked_v_args(value, v, v_int8, v_scale, v_center, v_tile_sum, v_workspace, v_workspace_bytes,
+                          batch, kv_heads, k_len, head_dim, padded, cta_k, v_stride_b, v_stride_h,
+                          v_stride_n, input_dtype, midpoint_affine, kv_permutation);
+  if (status != 0) return status;
+  hipStream_t hip_stream = static_cast<hipStream_t>(stream);
+  if (risa::can_prepare_fused(qk, value)) return risa::launch_prepare_fused(qk, value, hip_stream);
+  status = risa::launch_quantize_qk(qk, hip_stream);
+  if (status != 0) return status;
+  return risa::launch_quantize_v(value, hip_stream);
+}
+
 int risa_value_tile_sums(const void* v_int8, int32_t* tile_sum, int batch_heads, int head_dim,
                          int padded_length, int cta_k, void* stream) {
   if ((cta_k != 64 && cta_k != 128) || padded_length % cta_k != 0 || head_dim <= 0)

@@ -38,6 +38,10 @@ SIGNATURES = {
         _c_int,
         [_c_ptr] * 6 + [_c_size] + [_c_int] * 6 + [_c_i64] * 3 + [_c_int, _c_int, _c_ptr, _c_ptr],
     ),
+    "risa_sdpa_quantize": (
+        _c_int,
+        [_c_ptr] * 12 + [_c_size] + [_c_int] * 7 + [_c_i64] * 9 + [_c_int, _c_int, _c_ptr, _c_ptr, _c_ptr],
+    ),
     "risa_value_tile_sums": (_c_int, [_c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr]),
     "risa_unpack_order": (None, [_c_ptr]),
     "risa_attention": (

@@ -102,21 +102,15 @@ def quantize_inputs(q, k, v, attn_mask, scale, use_midpoint_affine: bool,
     stream = native.current_stream(device)
     code = DTYPE_CODES[input_dtype]
     native.check(
-        lib.risa_quantize_qk(
+        lib.risa_sdpa_quantize(
             q.data_ptr(), q_codes.data_ptr(), q_scale.data_ptr(),
             k.data_ptr(), k_codes.data_ptr(), k_scale.data_ptr(),
-            batch, q_heads, q_len, kv_heads, k_len, dim, cta_k,
-            q.stride(0), q.stride(1), q.stride(2), k.stride(0), k.stride(1), k.stride(2),
-            code, anchors.data_ptr(), native.pointer(kv_permutation), stream,
-        )
-    )
-    native.check(
-        lib.risa_quantize_v(
             v.data_ptr(), v_codes.data_ptr(), v_scale.data_ptr(), v_center.data_ptr(),
             v_tile_sum.data_ptr(), workspace.data_ptr(), workspace.numel(),
-            batch, kv_heads, k_len, dim, padded, cta_k,
+            batch, q_heads, q_len, kv_heads, k_len, dim, cta_k,
+            q.stride(0), q.stride(1), q.stride(2), k.stride(0), k.stride(1), k.stride(2),
             v.stride(0), v.stride(1), v.stride(2), code, int(use_midpoint_affine),
-            native.pointer(kv_permutation), stream,
+            anchors.data_ptr(), native.pointer(kv_permutation), stream,
         )
     )
     return PreparedBuffers(q_codes, k_codes, v_codes, q_scale, k_scale, v_scale, v_center,
