@@ -82,8 +82,8 @@ int risa_quantize_v(const void* v, void* out, float* scale, float* center, int32
  * csrc/bindings.cpp:195-272), which also prepares all three operands at once.
  * Arguments as for risa_quantize_qk and risa_quantize_v (padded length =
  * ceil(k_len / cta_k) * cta_k; the workspace is the V workspace).  Same results as
- * the two separate calls; when no permutation is given the work runs in two
- * launches (three beyond 4096 tokens) instead of five to seven.
+ * the two separate calls, in two launches (three beyond 4096 tokens) instead of
+ * five to seven.
  */
 int risa_sdpa_quantize(const void* q, void* q_int8, float* q_scale, const void* k, void* k_int8,
                        float* k_scale, const void* v, void* v_int8, float* v_scale, float* v_center,

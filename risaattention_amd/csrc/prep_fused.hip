@@ -11,8 +11,8 @@
 // With more than 64 partial ranges per channel (beyond 4096 tokens) the small
 // parameter kernel runs between the stages instead of inside every code workgroup.
 // A workgroup finds its role from its index; every role runs the same device
-// function as the stand-alone kernel, so results are bit-identical.  Used when no
-// permutation is given and K and V have the same extents.
+// function as the stand-alone kernel, so results are bit-identical.  Used when K and V
+// have the same extents (always, for callers of the attention API).
 
 #include "prep_qk_kernels.hpp"
 #include "prep_v_kernels.hpp"
@@ -39,7 +39,7 @@ __global__ __launch_bounds__(256) void prepare_stage1_kernel(const FusedArgs a) 
   int block = blockIdx.x;
   if (block < a.anchor_blocks) {
     detect_anchor_block<DT>(a.qk.k, a.qk.anchors, a.qk.k_len, a.qk.head_dim, a.qk.kv_heads,
-                            a.qk.k_stride_b, a.qk.k_stride_h, a.qk.k_stride_n, nullptr,
+                            a.qk.k_stride_b, a.qk.k_stride_h, a.qk.k_stride_n, a.qk.permutation,
                             block % a.qk.kv_heads, block / a.qk.kv_heads);
     return;
   }
@@ -70,7 +70,7 @@ __global__ __launch_bounds__(256) void prepare_stage2_kernel(const FusedArgs a) 
     if (tile < a.key_tiles) {
       quantize_k_block<DT, DK, CTA_K, ROT>(a.qk.k, a.qk.k_codes, a.qk.k_scale, a.qk.anchors, a.qk.k_len,
                                            a.qk.kv_heads, a.key_tiles * 4, a.qk.k_stride_b,
-                                           a.qk.k_stride_h, a.qk.k_stride_n, a.k_wide, nullptr, tile,
+                                           a.qk.k_stride_h, a.qk.k_stride_n, a.k_wide, a.qk.permutation, tile,
                                            half % 4, rest % a.qk.kv_heads, rest / a.qk.kv_heads);
     }
     return;
@@ -81,7 +81,7 @@ __global__ __launch_bounds__(256) void prepare_stage2_kernel(const FusedArgs a) 
   const int rest = block / a.code_blocks_x;
   value_codes_block<DT, CTA_K, PARAMS>(a.v.v, a.v.codes, a.v.tile_sum, a.inverse, a.midpoint, a.v.length,
                                        a.v.padded, a.v.head_dim, a.v.heads, a.v.stride_b, a.v.stride_h,
-                                       a.v.stride_n, nullptr, fused, x, rest % a.kv, rest / a.kv);
+                                       a.v.stride_n, a.v.permutation, fused, x, rest % a.kv, rest / a.kv);
 }
 
 template <int DT, int DK, int CTA_K, int ROT>
@@ -103,7 +103,7 @@ void launch_stages(const FusedArgs& a, hipStream_t stream) {
       dim3 center_grid(a.v.head_dim / 8, a.kv);
       value_center_fused_kernel<DT><<<center_grid, summation_threads(a.v.length), 0, stream>>>(
           a.v.v, a.inverse, a.midpoint, a.v.center, a.v.length, a.v.head_dim, a.v.heads, a.v.stride_b,
-          a.v.stride_h, a.v.stride_n, nullptr);
+          a.v.stride_h, a.v.stride_n, a.v.permutation);
     } else {
       const int threads = summation_threads(a.v.length);
       const int per_block = 256 / (a.v.head_dim / 8);
@@ -111,7 +111,7 @@ void launch_stages(const FusedArgs& a, hipStream_t stream) {
       dim3 residual_grid(threads / per_block, a.kv);
       value_residual_kernel<DT><<<residual_grid, 256, 0, stream>>>(
           a.v.v, a.partial, a.inverse, a.midpoint, a.v.length, a.v.head_dim, a.v.heads, threads,
-          a.v.stride_b, a.v.stride_h, a.v.stride_n, nullptr);
+          a.v.stride_b, a.v.stride_h, a.v.stride_n, a.v.permutation);
       value_center_from_partials_kernel<<<(rows + 63) / 64, 64, 0, stream>>>(
           a.partial, a.inverse, a.midpoint, a.v.center, rows, threads, a.v.length);
     }
@@ -162,7 +162,7 @@ template <int DT> void launch_by_dim(const FusedArgs& a, hipStream_t stream) {
 }  // namespace
 
 bool can_prepare_fused(const QkArgs& qk, const ValueArgs& v) {
-  return qk.permutation == nullptr && v.permutation == nullptr && qk.k_len == v.length &&
+  return qk.k_len == v.length &&
          qk.batch == v.batch && qk.kv_heads == v.heads && qk.head_dim == v.head_dim &&
          qk.cta_k == v.cta_k && qk.dtype == v.dtype;
 }

@@ -175,22 +175,30 @@ def test_value_codes_do_not_depend_on_schedule(risa, dtype, layout, length):
         assert torch.equal(wide.k_scale[:, :1], narrow.k_scale)
 
 
+@pytest.mark.parametrize("permuted", [False, True])
 @pytest.mark.parametrize("dtype,dim,length,mode", [
     (torch.bfloat16, 128, 1500, "absmax"),
     (torch.float16, 128, 6000, "midpoint_affine"),
     (torch.bfloat16, 64, 700, "midpoint_affine"),
     (torch.float32, 256, 4300, "absmax"),
 ])
-def test_separate_entry_points_match_one_call_preparation(risa, dtype, dim, length, mode):
+def test_separate_entry_points_match_one_call_preparation(risa, dtype, dim, length, mode, permuted):
     """risa_quantize_qk + risa_quantize_v (one launch per kernel) against
-    risa_sdpa_quantize (merged launches) on the same inputs: every output bit-equal."""
+    risa_sdpa_quantize (merged launches) on the same inputs, with and without a K/V
+    permutation: every output bit-equal."""
     from risaattention_amd import native
     from risaattention_amd.policy import DTYPE_CODES
 
     q = seeded((2, 4, 333, dim), dtype, 81)
     k = seeded((2, 2, length, dim), dtype, 82, offset=3.0)
     v = seeded((2, 2, length, dim), dtype, 83, offset=-1.0)
-    packed = risa.prequantize_int8_attention(q, k, v, v_quantization=mode)
+    extra, order = {}, None
+    if permuted:
+        generator = torch.Generator(device="cpu").manual_seed(84)
+        order = torch.stack([torch.randperm(length, generator=generator) for _ in range(4)])
+        order = order.reshape(2, 2, length).to("cuda", torch.int32)
+        extra = {"kv_permutation": risa.prepare_kv_permutation(order), "fuse_gather": True}
+    packed = risa.prequantize_int8_attention(q, k, v, v_quantization=mode, **extra)
     lib = native.library()
     affine = int(mode == "midpoint_affine")
     q_codes, k_codes, v_codes = (torch.empty_like(t) for t in (packed.q, packed.k, packed.v))
@@ -205,11 +213,11 @@ def test_separate_entry_points_match_one_call_preparation(risa, dtype, dim, leng
     native.check(lib.risa_quantize_qk(
         q.data_ptr(), q_codes.data_ptr(), q_scale.data_ptr(), k.data_ptr(), k_codes.data_ptr(),
         k_scale.data_ptr(), 2, 4, 333, 2, length, dim, packed.cta_k, *q.stride()[:3], *k.stride()[:3],
-        code, anchors.data_ptr(), None, stream))
+        code, anchors.data_ptr(), native.pointer(order), stream))
     native.check(lib.risa_quantize_v(
         v.data_ptr(), v_codes.data_ptr(), v_scale.data_ptr(), v_center.data_ptr(), tile_sum.data_ptr(),
         workspace.data_ptr(), workspace.numel(), 2, 2, length, dim, packed.v.shape[-1], packed.cta_k,
-        *v.stride()[:3], code, affine, None, stream))
+        *v.stride()[:3], code, affine, native.pointer(order), stream))
     for ours, theirs in ((q_codes, packed.q), (k_codes, packed.k), (v_codes, packed.v),
                          (q_scale, packed.q_scale), (k_scale, packed.k_scale), (v_scale, packed.v_scale),
                          (v_center, packed.v_center), (tile_sum, packed.v_tile_sum)):
