@@ -197,6 +197,52 @@ def workload_sparse(torch, risa, args, device):
     return rows
 
 
+def workload_prepare(torch, risa, args, device):
+    """Q/K/V preparation alone at the headline head counts: the one-call entry point
+    (merged launches) against risa_quantize_qk + risa_quantize_v (one launch per kernel)."""
+    from risaattention_amd import native
+    from risaattention_amd.policy import DTYPE_CODES
+
+    lib = native.library()
+    rows = []
+    batch, q_heads, kv_heads, dim = SHAPE["batch"], SHAPE["q_heads"], SHAPE["kv_heads"], SHAPE["head_dim"]
+    for length in ([args.length] if args.length else (1024, 4096, 32768)):
+        q, k, v = make_inputs(torch, length, 0, device)
+        for mode in ("absmax", "midpoint_affine"):
+            affine = int(mode == "midpoint_affine")
+            packed = risa.prequantize_int8_attention(q, k, v, v_quantization=mode)
+            anchors = torch.empty(batch, kv_heads, dtype=torch.int32, device=device)
+            workspace = torch.empty(max(1, lib.risa_quantize_v_workspace_bytes(batch, kv_heads, length, dim, affine)),
+                                    dtype=torch.uint8, device=device)
+            stream = native.current_stream(device)
+            code = DTYPE_CODES[q.dtype]
+            qk_args = (q.data_ptr(), packed.q.data_ptr(), packed.q_scale.data_ptr(), k.data_ptr(),
+                       packed.k.data_ptr(), packed.k_scale.data_ptr())
+            v_args = (v.data_ptr(), packed.v.data_ptr(), packed.v_scale.data_ptr(), packed.v_center.data_ptr(),
+                      packed.v_tile_sum.data_ptr(), workspace.data_ptr(), workspace.numel())
+
+            def separate():
+                native.check(lib.risa_quantize_qk(*qk_args, batch, q_heads, length, kv_heads, length, dim,
+                                                  packed.cta_k, *q.stride()[:3], *k.stride()[:3], code,
+                                                  anchors.data_ptr(), None, stream))
+                native.check(lib.risa_quantize_v(*v_args, batch, kv_heads, length, dim, packed.v.shape[-1],
+                                                 packed.cta_k, *v.stride()[:3], code, affine, None, stream))
+
+            def merged():
+                native.check(lib.risa_sdpa_quantize(*qk_args, *v_args, batch, q_heads, length, kv_heads, length,
+                                                    dim, packed.cta_k, *q.stride()[:3], *k.stride()[:3],
+                                                    *v.stride()[:3], code, affine, anchors.data_ptr(), None, stream))
+
+            in_bytes = (q.numel() + k.numel() + v.numel()) * q.element_size()
+            out_bytes = q.numel() + k.numel() + v.numel()
+            merged_ms = time_calls(torch, merged, 20)
+            rows.append({"N": length, "v_quantization": mode,
+                         "separate_ms": round(time_calls(torch, separate, 20), 4),
+                         "merged_ms": round(merged_ms, 4),
+                         "merged_gb_per_s": round((in_bytes + out_bytes) / (merged_ms * 1e-3) / 1e9, 1)})
+    return rows
+
+
 def workload_video(torch, risa, args, device):
     """Video-DiT-scale sampling loop: one construction, nine drifting reuses, packed-operand replay."""
     frames, per_frame, heads, dim = 21, 1560, 40, 128
@@ -280,7 +326,7 @@ def main():
     parser.add_argument("--mode", default="absmax", choices=["absmax", "midpoint_affine"])
     parser.add_argument("--no-cpu-baseline", action="store_true")
     parser.add_argument("--no-accuracy", action="store_true")
-    parser.add_argument("--workload", default="dense", choices=["dense", "sweep", "masked", "sparse", "video"],
+    parser.add_argument("--workload", default="dense", choices=["dense", "sweep", "masked", "sparse", "video", "prepare"],
                         help="dense = headline N=32K line (default); the others are the remaining benchmark "
                              "configurations of the reference, reported as one JSON line each")
     parser.add_argument("--calibrate-copy", action="store_true",
@@ -310,7 +356,7 @@ def main():
         return
     if args.workload != "dense":
         runner = {"sweep": workload_sweep, "masked": workload_masked, "sparse": workload_sparse,
-                  "video": workload_video}[args.workload]
+                  "video": workload_video, "prepare": workload_prepare}[args.workload]
         wall = time.perf_counter()
         rows = runner(torch, risa, args, device)
         print(json.dumps({"metric": f"{args.workload} workload (see config.rows)", "value": None, "unit": "ms",

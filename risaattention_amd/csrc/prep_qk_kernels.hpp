@@ -137,19 +137,22 @@ __device__ __forceinline__ float half_wave_max(float value) {
   return value;
 }
 
-// One scale group handled by one 32-lane half: NTOK tokens x DK channels, two
-// tokens at a time (one per 16-lane row).  `token_of(i)` gives the i-th token of
-// the group.  `wide` says rows are 16-byte aligned, so 16-bit inputs are read
-// eight channels per load.
-template <int DT, int DK, int ROT, int NTOK, typename TokenOf>
+// One scale group handled by LANES lanes (a 32-lane half or a whole wavefront): NTOK
+// tokens x DK channels, LANES / 16 tokens at a time (one per 16-lane row).
+// `token_of(i)` gives the i-th token of the group, `sub` the lane's index inside the
+// LANES.  `wide` says rows are 16-byte aligned, so 16-bit inputs are read eight
+// channels per load.
+template <int DT, int DK, int ROT, int NTOK, int LANES = 32, typename TokenOf>
 __device__ __forceinline__ void quantize_group(const void* in, int64_t in_base, int64_t stride_n,
                                                int8_t* out, float* scale_slot, int length, int sub,
                                                const void* bias_row, bool wide, TokenOf token_of,
                                                const int32_t* source = nullptr) {
   constexpr int BLOCKS = DK == 256 ? 2 : 1;   // 128-channel rotation blocks
   constexpr int GROUPS = DK == 64 ? 1 : 2;    // runs of four channels per lane and block
-  constexpr int STEPS = NTOK / 2;
-  static_assert(NTOK % 2 == 0, "two tokens per 32-lane half and step");
+  constexpr int PER_STEP = LANES / 16;
+  constexpr int STEPS = NTOK / PER_STEP;
+  static_assert(LANES == 32 || LANES == 64, "a half or a whole wavefront");
+  static_assert(NTOK % PER_STEP == 0, "whole steps");
   const int j = sub & 15, row = sub >> 4;
   auto channel_of = [&](int block, int g) { return block * 128 + (GROUPS * j + g) * 4; };
 
@@ -174,7 +177,7 @@ __device__ __forceinline__ void quantize_group(const void* in, int64_t in_base, 
   float v[STEPS][BLOCKS][GROUPS][4];
 #pragma unroll
   for (int i = 0; i < STEPS; ++i) {
-    const int n = token_of(2 * i + row);
+    const int n = token_of(PER_STEP * i + row);
     if (n < length) {
       // with a permutation, token n of the gathered sequence is source row source[n]
       const int from = source != nullptr ? source[n] : n;
@@ -208,12 +211,13 @@ __device__ __forceinline__ void quantize_group(const void* in, int64_t in_base, 
         for (int c = 0; c < 4; ++c) mx = __builtin_fmaxf(mx, __builtin_fabsf(v[i][block][g][c]));
     }
   mx = half_wave_max(mx);
+  if constexpr (LANES == 64) mx = max_across_halves(mx);
   const float scale = mx / 127.0f + 1e-7f;
   const float inverse = 1.0f / scale;
   if (sub == 0) *scale_slot = scale;
 #pragma unroll
   for (int i = 0; i < STEPS; ++i) {
-    const int n = token_of(2 * i + row);
+    const int n = token_of(PER_STEP * i + row);
     if (n < length) {
 #pragma unroll
       for (int block = 0; block < BLOCKS; ++block) {
@@ -269,7 +273,8 @@ __global__ __launch_bounds__(256) void quantize_q_kernel(const void* __restrict_
 }
 
 // One scale group ((token mod 8) / 2 = `group`) of key tile `tile`, handled by the
-// calling 32-lane half.
+// calling wavefront: four tokens per step keep the per-lane working set at half the
+// registers of a 32-lane group and put twice the wavefronts behind every tile.
 template <int DT, int DK, int CTA_K, int ROT>
 __device__ __forceinline__ void quantize_k_block(const void* __restrict__ k, int8_t* __restrict__ codes,
                                                  float* __restrict__ scales,
@@ -279,7 +284,7 @@ __device__ __forceinline__ void quantize_k_block(const void* __restrict__ k, int
                                                  const int32_t* __restrict__ permutation, int tile,
                                                  int group, int h, int b) {
   constexpr int NTOK = CTA_K / 4;
-  const int sub = threadIdx.x & 31;
+  const int sub = threadIdx.x & 63;
   const int64_t in_base = static_cast<int64_t>(b) * stride_b + static_cast<int64_t>(h) * stride_h;
   const int64_t bh = static_cast<int64_t>(b) * heads + h;
   const int anchor = anchors[b * heads + h];
@@ -288,16 +293,16 @@ __device__ __forceinline__ void quantize_k_block(const void* __restrict__ k, int
   const int anchor_row = anchor >= 0 && source != nullptr ? source[anchor] : anchor;
   const int64_t anchor_offset = static_cast<int64_t>(anchor_row) * stride_n;
   const int first = tile * CTA_K + group * 2;
-  quantize_group<DT, DK, ROT, NTOK>(k, in_base, stride_n, codes + bh * length * DK,
+  quantize_group<DT, DK, ROT, NTOK, 64>(k, in_base, stride_n, codes + bh * length * DK,
                                     scales + bh * scales_per_head + tile * 4 + group, length, sub,
                                     anchor >= 0 ? &anchor_offset : nullptr, wide != 0,
                                     [first](int i) { return first + (i >> 1) * 8 + (i & 1); }, source);
 }
 
-// grid (key tiles, Hkv, B), 128 threads: four 32-lane halves = the four scale
-// groups of one key tile of CTA_K tokens.
+// grid (key tiles, Hkv, B), 256 threads: four wavefronts = the four scale groups of
+// one key tile of CTA_K tokens.
 template <int DT, int DK, int CTA_K, int ROT>
-__global__ __launch_bounds__(128) void quantize_k_kernel(const void* __restrict__ k,
+__global__ __launch_bounds__(256) void quantize_k_kernel(const void* __restrict__ k,
                                                          int8_t* __restrict__ codes,
                                                          float* __restrict__ scales,
                                                          const int* __restrict__ anchors, int length,
@@ -307,7 +312,7 @@ __global__ __launch_bounds__(128) void quantize_k_kernel(const void* __restrict_
                                                          const int32_t* __restrict__ permutation) {
   quantize_k_block<DT, DK, CTA_K, ROT>(k, codes, scales, anchors, length, heads, scales_per_head,
                                        stride_b, stride_h, stride_n, wide, permutation, blockIdx.x,
-                                       threadIdx.x >> 5, blockIdx.y, blockIdx.z);
+                                       threadIdx.x >> 6, blockIdx.y, blockIdx.z);
 }
 
 // ---------------------------------------------------------------------------
