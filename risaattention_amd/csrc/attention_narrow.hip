@@ -4,11 +4,13 @@
 
 namespace risa {
 
+int narrow_attention_limit();
+
 namespace {
 
-template <int D, int CTA_K> int launch_narrow(const KernelParams& p, hipStream_t stream) {
+template <int D, int CTA_K, int WAVES> int launch_block(const KernelParams& p, hipStream_t stream) {
   using Shape = TileShape<D, CTA_K>;
-  auto kernel = attention_narrow_kernel<D, CTA_K>;
+  auto kernel = attention_narrow_kernel<D, CTA_K, WAVES>;
   static thread_local int configured_device = -1;
   int device = -1;
   if (hipGetDevice(&device) != hipSuccess) return fail("risa_attention: hipGetDevice failed");
@@ -21,9 +23,21 @@ template <int D, int CTA_K> int launch_narrow(const KernelParams& p, hipStream_t
     }
     configured_device = device;
   }
-  const dim3 grid(static_cast<unsigned>(p.n_qb) * p.q_heads * p.batch);
-  kernel<<<grid, kNarrowThreads, Shape::kLdsBytes, stream>>>(p);
+  constexpr int QUERIES = 16 * WAVES;
+  const unsigned query_blocks = static_cast<unsigned>((p.q_len + QUERIES - 1) / QUERIES);
+  const dim3 grid(query_blocks * p.q_heads * p.batch);
+  kernel<<<grid, 64 * WAVES, Shape::kLdsBytes, stream>>>(p);
   return 0;
+}
+
+// Queries per workgroup: 128, or 64 / 32 when that still leaves compute units without
+// a workgroup (every SIMD then runs one wavefront with a quarter of the usual work).
+template <int D, int CTA_K> int launch_narrow(const KernelParams& p, hipStream_t stream) {
+  const int64_t workgroups = static_cast<int64_t>(p.n_qb) * p.q_heads * p.batch;
+  const int compute_units = narrow_attention_limit();
+  if (workgroups * 4 <= compute_units) return launch_block<D, CTA_K, 2>(p, stream);
+  if (workgroups * 2 <= compute_units) return launch_block<D, CTA_K, 4>(p, stream);
+  return launch_block<D, CTA_K, 8>(p, stream);
 }
 
 }  // namespace

@@ -28,7 +28,6 @@
 
 namespace risa {
 
-constexpr int kNarrowThreads = 512;
 
 // XOR applied to the 16-byte chunk index of K row `row` in LDS.  The sixteen rows a
 // matrix instruction reads are two runs of eight consecutive keys 32 apart; folding
@@ -39,14 +38,17 @@ template <int ROWBYTES> __device__ __forceinline__ int narrow_key_swizzle(int ro
   return ((row / ROWS_PER_256) ^ ((row >> 5) * (8 / ROWS_PER_256))) & (CH - 1);
 }
 
-template <int D, int CTA_K>
-__global__ __launch_bounds__(kNarrowThreads) void attention_narrow_kernel(const KernelParams p) {
+// WAVES wavefronts of sixteen queries per workgroup (8, 4 or 2: 128, 64 or 32 queries).
+// The launcher picks the largest workgroup that still gives every compute unit one.
+template <int D, int CTA_K, int WAVES>
+__global__ __launch_bounds__(64 * WAVES) void attention_narrow_kernel(const KernelParams p) {
+  static_assert(WAVES == 8 || WAVES == 4 || WAVES == 2, "seeds and scales are copied by two different wavefronts");
+  constexpr int QUERIES = 16 * WAVES;
   using Shape = TileShape<D, CTA_K>;
   constexpr int KB = CTA_K / 16;  // 16-key blocks per tile
   constexpr int SB = CTA_K / 64;  // 64-key steps of the P·V product
   constexpr int CB = D / 16;      // 16-channel blocks
   constexpr int KK = D / 64;      // 64-channel steps of the score product
-  constexpr int WAVES = kNarrowThreads / 64;
   constexpr int COPIES = Shape::kTileBytes / 1024;  // 1 KB copy instructions per operand tile
   constexpr int NC = (COPIES + WAVES - 1) / WAVES;
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
@@ -56,8 +58,9 @@ __global__ __launch_bounds__(kNarrowThreads) void attention_narrow_kernel(const 
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int ql = lane & 15, grp = lane >> 4;
 
-  const int bx = blockIdx.x % p.n_qb;
-  const int rest = blockIdx.x / p.n_qb;
+  const int query_blocks = (p.q_len + QUERIES - 1) / QUERIES;
+  const int bx = blockIdx.x % query_blocks;
+  const int rest = blockIdx.x / query_blocks;
   const int head = rest % p.q_heads;
   const int batch = rest / p.q_heads;
   const int kv_head = head / (p.q_heads / p.kv_heads);
@@ -69,7 +72,7 @@ __global__ __launch_bounds__(kNarrowThreads) void attention_narrow_kernel(const 
   const int32_t* sum_base = p.v_tile_sum + bhk * p.n_kb * D;
   const float* ks_base = p.k_scale + bhk * p.n_kb * 4;
 
-  const int query = bx * kQueryBlock + wave * 16 + ql;
+  const int query = bx * QUERIES + wave * 16 + ql;
   const bool query_ok = query < p.q_len;
   const int n_it = p.n_kb;
 

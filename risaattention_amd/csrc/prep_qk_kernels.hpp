@@ -129,11 +129,14 @@ template <int ROT, int GROUPS> __device__ __forceinline__ void rotate(float (&v)
     for (int c = 0; c < 4; ++c) v[g][c] *= factor;
 }
 
+// Maximum over the 32 lanes of a half wavefront, in every lane: one lane swap for the
+// two 16-lane rows, DPP moves inside a row, no LDS round trips.
 __device__ __forceinline__ float half_wave_max(float value) {
-#pragma unroll
-  for (int offset = 16; offset > 0; offset >>= 1) {
-    value = __builtin_fmaxf(value, __shfl_xor(value, offset));
-  }
+  value = max_across_row_pairs(value);
+  value = __builtin_fmaxf(value, dpp_partner<8>(value));
+  value = __builtin_fmaxf(value, dpp_partner<4>(value));
+  value = __builtin_fmaxf(value, dpp_partner<2>(value));
+  value = __builtin_fmaxf(value, dpp_partner<1>(value));
   return value;
 }
 
@@ -323,17 +326,20 @@ __global__ __launch_bounds__(256) void quantize_k_kernel(const void* __restrict_
 // ---------------------------------------------------------------------------
 constexpr int kSamples = 9;
 
+// Sum / maximum of a 32-lane segment as lane 0 of the segment gets it from a
+// shuffle-down tree with offsets 16, 8, 4, 2, 1 (the reference's order).  An exchange
+// butterfly gives lane 0 the same additions in the same order (x + y = y + x exactly),
+// and needs one lane swap plus four DPP moves instead of five trips through LDS.
 __device__ __forceinline__ float segment_down_sum(float value) {
-#pragma unroll
-  for (int offset = 16; offset > 0; offset >>= 1) value += __shfl_down(value, offset, 32);
+  const auto rows = __builtin_amdgcn_permlane16_swap(__float_as_uint(value), __float_as_uint(value), false, false);
+  value = __uint_as_float(rows[0]) + __uint_as_float(rows[1]);
+  value += dpp_partner<8>(value);
+  value += dpp_partner<4>(value);
+  value += dpp_partner<2>(value);
+  value += dpp_partner<1>(value);
   return value;
 }
-__device__ __forceinline__ float segment_down_max(float value) {
-#pragma unroll
-  for (int offset = 16; offset > 0; offset >>= 1)
-    value = __builtin_fmaxf(value, __shfl_down(value, offset, 32));
-  return value;
-}
+__device__ __forceinline__ float segment_down_max(float value) { return half_wave_max(value); }
 
 template <int DT>
 __device__ __forceinline__ void detect_anchor_block(const void* __restrict__ k, int* __restrict__ anchors,
