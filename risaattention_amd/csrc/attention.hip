@@ -10,9 +10,9 @@
 
 namespace risa {
 
-template <> int launch_attention_variant<64>(const KernelParams&, int, bool, bool, bool, bool, hipStream_t);
-template <> int launch_attention_variant<128>(const KernelParams&, int, bool, bool, bool, bool, hipStream_t);
-template <> int launch_attention_variant<256>(const KernelParams&, int, bool, bool, bool, bool, hipStream_t);
+template <> int launch_attention_variant<64>(const KernelParams&, int, bool, bool, bool, int, hipStream_t);
+template <> int launch_attention_variant<128>(const KernelParams&, int, bool, bool, bool, int, hipStream_t);
+template <> int launch_attention_variant<256>(const KernelParams&, int, bool, bool, bool, int, hipStream_t);
 int launch_attention_narrow(const KernelParams& p, int head_dim, int cta_k, hipStream_t stream);
 int narrow_attention_limit();
 
@@ -111,15 +111,23 @@ int launch_attention(const AttentionArgs& a, hipStream_t stream) {
   p.mask_stride_q = a.mask_stride_q;
   p.mask_stride_k = a.mask_stride_k;
   p.mask_dtype = a.mask != nullptr ? a.mask_dtype : -1;
-  bool mask_vector = false;
+  int mask_mode = kMaskScalar;
   if (a.mask != nullptr) {
     // Groups of four keys start at multiples of four, so one load per group needs
     // unit key stride, the other strides multiples of four elements and the base
-    // aligned to four elements.
-    const int64_t element = a.mask_dtype == kF32 ? 4 : a.mask_dtype == kBool ? 1 : 2;
-    const bool aligned = reinterpret_cast<uintptr_t>(a.mask) % (4 * element) == 0 &&
-                         ((a.mask_stride_b | a.mask_stride_h | a.mask_stride_q) & 3) == 0;
-    mask_vector = a.mask_stride_k == 1 && aligned;
+    // aligned to four elements.  Staging the mask tile in LDS copies 16 bytes per lane:
+    // everything 16-byte aligned, rows not overlapping backwards, and the 128 rows of a
+    // query block within reach of a 32-bit byte offset.
+    const int64_t element = mask_element_bytes(a.mask_dtype);
+    const auto address = reinterpret_cast<uintptr_t>(a.mask);
+    const int64_t strides = a.mask_stride_b | a.mask_stride_h | a.mask_stride_q;
+    if (a.mask_stride_k == 1 && address % (4 * element) == 0 && (strides & 3) == 0) {
+      mask_mode = kMaskVector;
+      if (address % 16 == 0 && (strides * element) % 16 == 0 && a.mask_stride_q >= 0 &&
+          a.mask_stride_q * element * kQueryBlock < (int64_t{1} << 31)) {
+        mask_mode = kMaskStaged;
+      }
+    }
     if (a.key_bias != nullptr) {
       if (a.mask_stride_q != 0) return fail("risa_attention: a key bias row needs a key-only mask");
       if (reinterpret_cast<uintptr_t>(a.key_bias) % 16 != 0 || (a.key_bias_stride_b | a.key_bias_stride_h) % 4 != 0)
@@ -169,11 +177,11 @@ int launch_attention(const AttentionArgs& a, hipStream_t stream) {
   if (narrow)
     status = launch_attention_narrow(p, a.head_dim, a.cta_k, stream);
   else if (a.head_dim == 64)
-    status = launch_attention_variant<64>(p, a.cta_k, fast, indexed, capture, mask_vector, stream);
+    status = launch_attention_variant<64>(p, a.cta_k, fast, indexed, capture, mask_mode, stream);
   else if (a.head_dim == 128)
-    status = launch_attention_variant<128>(p, a.cta_k, fast, indexed, capture, mask_vector, stream);
+    status = launch_attention_variant<128>(p, a.cta_k, fast, indexed, capture, mask_mode, stream);
   else if (a.head_dim == 256)
-    status = launch_attention_variant<256>(p, a.cta_k, fast, indexed, capture, mask_vector, stream);
+    status = launch_attention_variant<256>(p, a.cta_k, fast, indexed, capture, mask_mode, stream);
   else
     return fail("risa_attention: unsupported head_dim");
   if (status != 0) return status;

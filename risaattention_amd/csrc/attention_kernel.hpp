@@ -117,26 +117,54 @@ __device__ __forceinline__ int fresh_lane() {
   return lane_id;
 }
 
-template <int D, int CTA_K> struct TileShape {
+// MASK_BYTES: bytes of the mask tile kept next to K and V in each of the two stages;
+// SHARED_MASK_BYTES: bytes of a single mask tile behind both stages (0 unless staged).
+template <int D, int CTA_K, int MASK_BYTES = 0, int SHARED_MASK_BYTES = 0> struct TileShape {
   static constexpr int kTileBytes = CTA_K * D;
   static constexpr int kCopiesPerWave = kTileBytes / 16 / 256;  // 1 KB copy instructions per wave
   static constexpr int kSeedBytes = D * 4;                       // accumulator seeds of the tile
   static constexpr int kBiasBytes = CTA_K * 4;                   // key-only mask row of the tile
-  static constexpr int kStageBytes = 2 * kTileBytes + kSeedBytes + kBiasBytes;
-  static constexpr int kLdsBytes = 2 * kStageBytes;
+  static constexpr int kMaskOffset = 2 * kTileBytes + kSeedBytes + kBiasBytes;
+  static constexpr int kStageBytes = kMaskOffset + MASK_BYTES;
+  static constexpr int kSharedMaskOffset = 2 * kStageBytes;
+  static constexpr int kLdsBytes = 2 * kStageBytes + SHARED_MASK_BYTES;
 };
+
+// How the kernel reads a mask tensor (template parameter MASK_MODE).
+constexpr int kMaskScalar = 0;  // element by element: any strides
+constexpr int kMaskVector = 1;  // one load per four keys: unit key stride, aligned rows
+constexpr int kMaskStaged = 2;  // mask tile copied to LDS with K and V: 16-byte aligned rows, 64-key tiles
+
+constexpr int mask_element_bytes(int mask_dtype) { return mask_dtype == kF32 ? 4 : mask_dtype == kBool ? 1 : 2; }
+// LDS bytes of a staged mask tile (128 queries x CTA_K keys).
+// 1- and 2-byte masks keep one tile per stage (requested a tile ahead, like K and V).
+// A 4-byte mask tile is 32 KB: it is kept once, which leaves room for two workgroups
+// per compute unit, and is requested after the softmax of the previous tile.  That
+// needs no barrier: every wavefront copies and reads only the rows of its own queries.
+constexpr bool staged_mask_is_shared(int mask_dtype) { return mask_dtype == kF32; }
+constexpr int staged_mask_bytes(int mask_dtype, int mask_mode, int cta_k, bool shared) {
+  return mask_mode == kMaskStaged && staged_mask_is_shared(mask_dtype) == shared
+             ? kQueryBlock * cta_k * mask_element_bytes(mask_dtype)
+             : 0;
+}
+template <int D, int CTA_K, int MASK_DT, int MASK_MODE>
+using AttentionTileShape = TileShape<D, CTA_K, staged_mask_bytes(MASK_DT, MASK_MODE, CTA_K, false),
+                                     staged_mask_bytes(MASK_DT, MASK_MODE, CTA_K, true)>;
 
 // MASK_DT: element type of the mask tensor (risa::kBool, kF32, kF16, kBF16), kKeyBias
 // for a key-only mask prepared as an FP32 row, or -1 for none; FAST (raw-score path)
-// implies -1.  MASK_VEC: the mask tensor allows one load per group of four keys (unit
-// key stride, aligned rows); a template parameter and not a run-time branch so that the
-// tile loop holds one unrolled mask path instead of two and stays inside the
-// instruction cache.
-template <int D, int CTA_K, bool FAST, bool INDEXED, bool CAPTURE, int MASK_DT, bool MASK_VEC>
+// implies -1.  MASK_MODE: kMaskScalar / kMaskVector / kMaskStaged; a template parameter
+// and not a run-time branch so that the tile loop holds one unrolled mask path and
+// stays inside the instruction cache.
+template <int D, int CTA_K, bool FAST, bool INDEXED, bool CAPTURE, int MASK_DT, int MASK_MODE>
 __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void attention_kernel(const KernelParams p) {
   static_assert(!FAST || MASK_DT < 0, "the raw-score path takes no mask");
-  static_assert(!MASK_VEC || (MASK_DT >= 0 && MASK_DT != kKeyBias), "vector loads need a mask tensor");
-  using Shape = TileShape<D, CTA_K>;
+  static_assert(MASK_MODE == kMaskScalar || (MASK_DT >= 0 && MASK_DT != kKeyBias), "vector loads need a mask tensor");
+  static_assert(MASK_MODE != kMaskStaged || CTA_K == 64, "staged masks: 64-key tiles");
+  constexpr bool MASK_VEC = MASK_MODE != kMaskScalar;
+  constexpr bool STAGED = MASK_MODE == kMaskStaged;
+  constexpr bool SHARED_MASK = STAGED && staged_mask_is_shared(MASK_DT);
+  using Shape = AttentionTileShape<D, CTA_K, MASK_DT, MASK_MODE>;
   constexpr int RB = CTA_K / 32;  // 32-key blocks per tile
   constexpr int CB = D / 32;      // 32-channel blocks
   constexpr int KK = D / 32;      // k-steps of the score product
@@ -238,6 +266,41 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void attention_kernel(cons
       v_kept[i] = v_source_offset(i, lane);
     }
   }
+  // Staged masks: the mask tile of the workgroup's 128 queries (64 * ES bytes per row,
+  // 16-byte chunks XOR-swizzled by row so that the 32 rows a half-wave reads spread over
+  // the banks) is copied like K and V.  Source offsets are relative to the first row of
+  // the query block; rows past the last query re-read the last one.
+  constexpr int MASK_ES = MASK_DT >= 0 && MASK_DT != kKeyBias ? mask_element_bytes(MASK_DT) : 1;
+  constexpr int MASK_ROW_BYTES = CTA_K * MASK_ES;
+  constexpr int MASK_CH = MASK_ROW_BYTES / 16;                       // chunks per row
+  constexpr int NM = STAGED ? kQueryBlock * MASK_CH / 256 : 1;       // copy instructions per wave
+  auto mask_swizzle = [](int row) { return (row / (256 / MASK_ROW_BYTES)) & (MASK_CH - 1); };
+  [[maybe_unused]] const int8_t* mask_block = nullptr;
+  if constexpr (STAGED) {
+    mask_block = static_cast<const int8_t*>(p.mask) +
+                 (static_cast<int64_t>(batch) * p.mask_stride_b + static_cast<int64_t>(head) * p.mask_stride_h +
+                  static_cast<int64_t>(bx) * kQueryBlock * p.mask_stride_q) * MASK_ES;
+  }
+  auto mask_region = [&](int stage) -> unsigned char* {
+    if constexpr (SHARED_MASK) return lds + Shape::kSharedMaskOffset;
+    return lds + stage * Shape::kStageBytes + Shape::kMaskOffset;
+  };
+  auto issue_mask_tile = [&](int tile, int stage) {
+    if constexpr (STAGED) {
+      unsigned char* slot = mask_region(stage) + wave * (NM * 1024);
+      const int8_t* source = mask_block + static_cast<int64_t>(tile) * MASK_ROW_BYTES;
+      const int lane_id = fresh_lane();
+      const int last_row = p.q_len - 1 - bx * kQueryBlock;
+#pragma unroll
+      for (int i = 0; i < NM; ++i) {
+        const int index = (wave * NM + i) * 64 + lane_id;
+        const int row = index / MASK_CH, chunk = (index % MASK_CH) ^ mask_swizzle(row);
+        const uint32_t offset = static_cast<uint32_t>(min(row, last_row)) *
+                                    static_cast<uint32_t>(p.mask_stride_q * MASK_ES) + chunk * 16;
+        copy16_to_lds_uniform(source, offset, slot + i * 1024);
+      }
+    }
+  };
   auto issue_tile = [&](int tile, int stage) {
     unsigned char* k_slot = lds + stage * Shape::kStageBytes + wave * (NC * 1024);
     unsigned char* v_slot = k_slot + Shape::kTileBytes;
@@ -340,7 +403,7 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void attention_kernel(cons
   // in flight.  Used for query-dependent masks (always 64-key tiles, where the
   // registers are there) that allow one load per group of four keys; not for FP32
   // masks with head dim 64, where the 32 extra registers cost a resident wavefront.
-  constexpr bool PRELOAD = MASK_VEC && CTA_K == 64 && !(MASK_DT == kF32 && D == 64);
+  constexpr bool PRELOAD = MASK_MODE == kMaskVector && CTA_K == 64 && !(MASK_DT == kF32 && D == 64);
   constexpr int WORDS = MASK_DT == kF32 ? 4 : MASK_DT == kBool ? 1 : 2;  // 32-bit words per four keys
   constexpr bool LATE_COPIES = PRELOAD;
   [[maybe_unused]] uint32_t mask_words[PRELOAD ? RB * 4 * WORDS : 1];
@@ -560,7 +623,28 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void attention_kernel(cons
                 if constexpr (LOADED) {
                   // Rows past the last query hold the last row's mask: they behave like
                   // a valid row and are never stored.
+                  [[maybe_unused]] uint32_t staged_words[4];
                   const uint32_t* words = mask_words + (rb * 4 + b4) * WORDS;
+                  if constexpr (STAGED) {
+                    // This lane's four keys of the group: bytes [offset, offset + 4 * ES) of its row.
+                    const int row = wave * 32 + l32;
+                    const int offset = (local + half * 4) * MASK_ES;
+                    const unsigned char* at = mask_region(it & 1) + row * MASK_ROW_BYTES +
+                                              (((offset >> 4) ^ mask_swizzle(row)) << 4) + (offset & 15);
+                    if constexpr (MASK_ES == 1) {
+                      staged_words[0] = *reinterpret_cast<const uint32_t*>(at);
+                    } else if constexpr (MASK_ES == 4) {
+                      typedef uint32_t v4u __attribute__((ext_vector_type(4)));
+                      const v4u quad = *reinterpret_cast<const v4u*>(at);
+                      staged_words[0] = quad[0], staged_words[1] = quad[1];
+                      staged_words[2] = quad[2], staged_words[3] = quad[3];
+                    } else {
+                      typedef uint32_t v2u __attribute__((ext_vector_type(2)));
+                      const v2u pair = *reinterpret_cast<const v2u*>(at);
+                      staged_words[0] = pair[0], staged_words[1] = pair[1];
+                    }
+                    words = staged_words;
+                  }
                   if constexpr (DT == kBool) {
 #pragma unroll
                     for (int r = 0; r < 4; ++r) keep[r] = ((words[0] >> (8 * r)) & 0xffu) != 0;
@@ -641,7 +725,7 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void attention_kernel(cons
         };
         using MaskType = std::integral_constant<int, MASK_DT>;
         auto mask_pass = [&](auto diagonal_tag) {
-          if constexpr (PRELOAD && !LAST) {
+          if constexpr ((PRELOAD || STAGED) && !LAST) {
             masked_scores(MaskType{}, std::true_type{}, std::true_type{}, diagonal_tag);
           } else if constexpr (MASK_VEC) {
             masked_scores(MaskType{}, std::true_type{}, std::false_type{}, diagonal_tag);
@@ -785,6 +869,8 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void attention_kernel(cons
     v16i seed[2];
     int tile = tile_at(0);
     issue_tile(tile, 0);
+    // The last listed tile reads its mask elements directly (it may be partial).
+    if (n_it > 1) issue_mask_tile(tile, 0);
     float ks0 = ks_base[tile * 4 + 2 * half];
     float ks1 = ks_base[tile * 4 + 2 * half + 1];
     for (int it = 0; it < n_it - 1; ++it) {
@@ -798,6 +884,9 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void attention_kernel(cons
         __builtin_amdgcn_sched_barrier(0);
       }
       if constexpr (!LATE_COPIES) issue_tile(next_tile, stage ^ 1);
+      if constexpr (!SHARED_MASK) {
+        if (it + 2 < n_it) issue_mask_tile(next_tile, stage ^ 1);
+      }
       const int scale_pair = KEEP_OFFSETS ? 2 * half : (fresh_lane() >> 5) * 2;
       const float next_ks0 = ks_base[next_tile * 4 + scale_pair];
       const float next_ks1 = ks_base[next_tile * 4 + scale_pair + 1];
@@ -811,6 +900,11 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void attention_kernel(cons
       if constexpr (LATE_COPIES) {
         __builtin_amdgcn_sched_barrier(0);
         issue_tile(next_tile, stage ^ 1);
+      }
+      if constexpr (SHARED_MASK) {
+        // this wavefront has consumed its rows of the one mask tile: refill them
+        __builtin_amdgcn_sched_barrier(0);
+        if (it + 2 < n_it) issue_mask_tile(next_tile, stage ^ 1);
       }
       if constexpr (PREFETCH) {
         __builtin_amdgcn_sched_barrier(0);

@@ -280,3 +280,39 @@ def test_lse_request_does_not_change_outputs(risa, length, heads, mode):
     assert torch.equal(plain, with_lse)
     assert torch.isfinite(lse).all()
     assert torch.equal(plain, risa.int8_attention(q, k, v, v_quantization=mode))
+
+
+@pytest.mark.parametrize("mask_dtype", [torch.bool, torch.float16, torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("dim", [64, 128, 256])
+@pytest.mark.parametrize("causal", [False, True])
+def test_staged_mask_tiles_match_oracle(risa, mask_dtype, dim, causal):
+    """Query-dependent masks whose rows are 16-byte aligned are copied to LDS tile by
+    tile.  330 queries (a ragged last query block) x 400 keys (a ragged last key tile),
+    two batch entries with a mask per batch entry and head; a mask view with an
+    unaligned base takes the other load path and must give the same answer."""
+    q_len, k_len = 330, 400
+    q = seeded((2, 2, q_len, dim), torch.float16, 71)
+    k = seeded((2, 1, k_len, dim), torch.float16, 72)
+    v = seeded((2, 1, k_len, dim), torch.float16, 73)
+    generator = torch.Generator(device="cpu").manual_seed(74)
+    if mask_dtype == torch.bool:
+        mask = torch.rand((2, 2, q_len, k_len), generator=generator) > 0.4
+        mask[0, 1, 129] = False  # a fully hidden row
+    else:
+        mask = torch.randn((2, 2, q_len, k_len), generator=generator).to(mask_dtype)
+        mask[..., 3::7] = float("-inf")
+    mask = mask.cuda()
+    out, lse = risa.int8_attention(q, k, v, attn_mask=mask, is_causal=causal, return_lse=True)
+    prepared = oracle_prequantize(q, k, v, attn_mask=mask, is_causal=causal, return_lse=True)
+    expected, expected_lse, _ = oracle_pipeline.attend(prepared, return_lse=True)
+    assert relative_l2(to_numpy(out), expected) < TOLERANCE
+    finite = np.isfinite(expected_lse)
+    assert np.array_equal(np.isfinite(to_numpy(lse)), finite)
+    assert relative_l2(to_numpy(lse)[finite], expected_lse[finite]) < TOLERANCE
+    # same values behind a base address that is not 16-byte aligned
+    storage = torch.empty(mask.numel() + 16, dtype=mask.dtype, device="cuda")
+    shifted = storage[4:4 + mask.numel()].view_as(mask).copy_(mask)
+    assert shifted.data_ptr() % 16 != 0 or mask.element_size() == 4
+    out_shifted, lse_shifted = risa.int8_attention(q, k, v, attn_mask=shifted, is_causal=causal, return_lse=True)
+    assert torch.equal(out_shifted, out)
+    assert torch.equal(lse_shifted, lse)
