@@ -8,36 +8,50 @@ int narrow_attention_limit();
 
 namespace {
 
-template <int D, int CTA_K, int WAVES> int launch_block(const KernelParams& p, hipStream_t stream) {
+template <int D, int CTA_K, int WAVES, int KSPLIT> int launch_block(const KernelParams& p, hipStream_t stream) {
   using Shape = TileShape<D, CTA_K>;
-  auto kernel = attention_narrow_kernel<D, CTA_K, WAVES>;
+  constexpr int kLdsBytes = Shape::kLdsBytes * KSPLIT;
+  auto kernel = attention_narrow_kernel<D, CTA_K, WAVES, KSPLIT>;
   static thread_local int configured_device = -1;
   int device = -1;
   if (hipGetDevice(&device) != hipSuccess) return fail("risa_attention: hipGetDevice failed");
   if (device != configured_device) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                            hipFuncAttributeMaxDynamicSharedMemorySize,
-                            Shape::kLdsBytes) != hipSuccess) {
-      return fail("risa_attention: cannot reserve " + std::to_string(Shape::kLdsBytes) +
-                  " bytes of LDS");
+                            hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes) != hipSuccess) {
+      return fail("risa_attention: cannot reserve " + std::to_string(kLdsBytes) + " bytes of LDS");
     }
     configured_device = device;
   }
   constexpr int QUERIES = 16 * WAVES;
   const unsigned query_blocks = static_cast<unsigned>((p.q_len + QUERIES - 1) / QUERIES);
   const dim3 grid(query_blocks * p.q_heads * p.batch);
-  kernel<<<grid, 64 * WAVES, Shape::kLdsBytes, stream>>>(p);
+  kernel<<<grid, 64 * WAVES * KSPLIT, kLdsBytes, stream>>>(p);
   return 0;
 }
 
 // Queries per workgroup: 128, or 64 / 32 when that still leaves compute units without
 // a workgroup (every SIMD then runs one wavefront with a quarter of the usual work).
+// Those smaller workgroups also split the key tiles over two sets of wavefronts when
+// the tile count is even: the launch is short of work, not of hardware.
 template <int D, int CTA_K> int launch_narrow(const KernelParams& p, hipStream_t stream) {
   const int64_t workgroups = static_cast<int64_t>(p.n_qb) * p.q_heads * p.batch;
   const int compute_units = narrow_attention_limit();
-  if (workgroups * 4 <= compute_units) return launch_block<D, CTA_K, 2>(p, stream);
-  if (workgroups * 2 <= compute_units) return launch_block<D, CTA_K, 4>(p, stream);
-  return launch_block<D, CTA_K, 8>(p, stream);
+  // two sets of stages must fit the 160 KB of LDS of a compute unit
+  constexpr bool kSplitFits = 2 * TileShape<D, CTA_K>::kLdsBytes <= 160 * 1024;
+  const bool split = kSplitFits && p.n_kb >= 4 && p.n_kb % 2 == 0;
+  if (workgroups * 4 <= compute_units) {
+    if constexpr (kSplitFits) {
+      if (split) return launch_block<D, CTA_K, 2, 2>(p, stream);
+    }
+    return launch_block<D, CTA_K, 2, 1>(p, stream);
+  }
+  if (workgroups * 2 <= compute_units) {
+    if constexpr (kSplitFits) {
+      if (split) return launch_block<D, CTA_K, 4, 2>(p, stream);
+    }
+    return launch_block<D, CTA_K, 4, 1>(p, stream);
+  }
+  return launch_block<D, CTA_K, 8, 1>(p, stream);
 }
 
 }  // namespace

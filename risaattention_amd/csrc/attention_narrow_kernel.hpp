@@ -40,9 +40,15 @@ template <int ROWBYTES> __device__ __forceinline__ int narrow_key_swizzle(int ro
 
 // WAVES wavefronts of sixteen queries per workgroup (8, 4 or 2: 128, 64 or 32 queries).
 // The launcher picks the largest workgroup that still gives every compute unit one.
-template <int D, int CTA_K, int WAVES>
-__global__ __launch_bounds__(64 * WAVES) void attention_narrow_kernel(const KernelParams p) {
+// KSPLIT = 2 doubles the wavefronts: two parts of WAVES wavefronts walk the first and the
+// second half of the key tiles of the same queries (each with its own LDS stages) and
+// the first part merges the two partial results through LDS at the end, which halves
+// the chain of dependent tiles of a short sequence.  The merge is the online-softmax
+// update applied once more, so only the FP32 rounding order differs.
+template <int D, int CTA_K, int WAVES, int KSPLIT = 1>
+__global__ __launch_bounds__(64 * WAVES * KSPLIT) void attention_narrow_kernel(const KernelParams p) {
   static_assert(WAVES == 8 || WAVES == 4 || WAVES == 2, "seeds and scales are copied by two different wavefronts");
+  static_assert(KSPLIT == 1 || (KSPLIT == 2 && WAVES <= 4), "at most eight wavefronts per workgroup");
   constexpr int QUERIES = 16 * WAVES;
   using Shape = TileShape<D, CTA_K>;
   constexpr int KB = CTA_K / 16;  // 16-key blocks per tile
@@ -51,12 +57,15 @@ __global__ __launch_bounds__(64 * WAVES) void attention_narrow_kernel(const Kern
   constexpr int KK = D / 64;      // 64-channel steps of the score product
   constexpr int COPIES = Shape::kTileBytes / 1024;  // 1 KB copy instructions per operand tile
   constexpr int NC = (COPIES + WAVES - 1) / WAVES;
-  extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds_all[];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int workgroup_wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int part = workgroup_wave / WAVES;  // which half of the key tiles (0 when KSPLIT == 1)
+  const int wave = workgroup_wave % WAVES;  // which sixteen queries
   const int ql = lane & 15, grp = lane >> 4;
+  unsigned char* lds = lds_all + part * Shape::kLdsBytes;
 
   const int query_blocks = (p.q_len + QUERIES - 1) / QUERIES;
   const int bx = blockIdx.x % query_blocks;
@@ -74,7 +83,8 @@ __global__ __launch_bounds__(64 * WAVES) void attention_narrow_kernel(const Kern
 
   const int query = bx * QUERIES + wave * 16 + ql;
   const bool query_ok = query < p.q_len;
-  const int n_it = p.n_kb;
+  const int n_it = p.n_kb / KSPLIT;  // the launcher splits even tile counts only
+  const int first_tile = part * n_it;
 
   // --- copies HBM/L2 -> LDS ---------------------------------------------------------
   // Copy instruction (wave*NC + i) fills LDS bytes [(wave*NC + i)*1024, +1024) of a
@@ -331,9 +341,10 @@ __global__ __launch_bounds__(64 * WAVES) void attention_narrow_kernel(const Kern
     v4i acc_first[GROUP];
     v4i v_first[GROUP][SB];
     float ks0, ks1;
-    issue_tile(0, 0);
-    for (int tile = 0; tile < n_it - 1; ++tile) {
-      const int stage = tile & 1;
+    issue_tile(first_tile, 0);
+    for (int step = 0; step < n_it - 1; ++step) {
+      const int stage = step & 1;
+      const int tile = first_tile + step;
       __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
       __syncthreads();
       load_k_fragments(lds + stage * Shape::kStageBytes, 0, k_first);
@@ -347,14 +358,52 @@ __global__ __launch_bounds__(64 * WAVES) void attention_narrow_kernel(const Kern
       value_tile(stage, pk, acc_first, v_first, t_scale);
     }
     const int stage = (n_it - 1) & 1;
+    const int tile = first_tile + n_it - 1;
     __builtin_amdgcn_s_waitcnt(0x0f70);
     __syncthreads();
     load_k_fragments(lds + stage * Shape::kStageBytes, 0, k_first);
     tile_scales(stage, ks0, ks1);
     score_tile(stage, k_first, s);
-    const float t_scale = softmax_tile(std::true_type{}, n_it - 1, ks0, ks1, s, pk);
+    // Only the last tile of the sequence takes the last-tile formulas.
+    float t_scale;
+    if (KSPLIT == 1 || part == KSPLIT - 1) {
+      t_scale = softmax_tile(std::true_type{}, tile, ks0, ks1, s, pk);
+    } else {
+      t_scale = softmax_tile(std::false_type{}, tile, ks0, ks1, s, pk);
+    }
     load_group(stage, 0, acc_first, v_first);
     value_tile(stage, pk, acc_first, v_first, t_scale);
+  }
+
+  // ---- merge of the two key halves ----------------------------------------------------------
+  // Part 1 leaves (O, m, d) of every lane in LDS, value-major so that lanes are
+  // contiguous; the wavefront of part 0 with the same queries folds them in.
+  if constexpr (KSPLIT == 2) {
+    constexpr int VALUES = CB * 4 + 2;
+    __syncthreads();  // every wavefront is done with its stages
+    float* exchange = reinterpret_cast<float*>(lds_all) + wave * (VALUES * 64) + lane;
+    if (part == 1) {
+#pragma unroll
+      for (int cb = 0; cb < CB; ++cb)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) exchange[(cb * 4 + i) * 64] = o_acc[cb][i];
+      exchange[(CB * 4) * 64] = m_run;
+      exchange[(CB * 4 + 1) * 64] = d_part;
+    }
+    __syncthreads();
+    if (part == 1) return;
+    const float other_m = exchange[(CB * 4) * 64];
+    const float other_d = exchange[(CB * 4 + 1) * 64];
+    const float merged_m = __builtin_fmaxf(m_run, other_m);
+    const float mine = __builtin_amdgcn_exp2f(m_run - merged_m);
+    const float theirs = __builtin_amdgcn_exp2f(other_m - merged_m);
+    d_part = __builtin_fmaf(other_d, theirs, d_part * mine);
+#pragma unroll
+    for (int cb = 0; cb < CB; ++cb)
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        o_acc[cb][i] = __builtin_fmaf(exchange[(cb * 4 + i) * 64], theirs, o_acc[cb][i] * mine);
+    m_run = merged_m;
   }
 
   // ---- epilogue ---------------------------------------------------------------------------
