@@ -316,3 +316,26 @@ def test_staged_mask_tiles_match_oracle(risa, mask_dtype, dim, causal):
     out_shifted, lse_shifted = risa.int8_attention(q, k, v, attn_mask=shifted, is_causal=causal, return_lse=True)
     assert torch.equal(out_shifted, out)
     assert torch.equal(lse_shifted, lse)
+
+
+@pytest.mark.parametrize("heads", [4, 80, 200])
+@pytest.mark.parametrize("dim,k_len", [(64, 500), (128, 500), (128, 1400), (256, 444)])
+def test_small_launches_match_oracle(risa, heads, dim, k_len):
+    """Unmasked launches below one workgroup per compute unit: 4 heads run 32 queries per
+    workgroup and 80 heads 64, both with the key tiles split over two sets of wavefronts
+    (8, 22 and 8 tiles: even counts, ragged last tile); 200 heads run 128 queries per
+    workgroup without the split.  444 keys are 7 tiles: an odd count is not split."""
+    assert 128 < torch.cuda.get_device_properties(0).multi_processor_count <= 256
+    q = seeded((1, heads, 100, dim), torch.bfloat16, 91)
+    k = seeded((1, 4, k_len, dim), torch.bfloat16, 92)
+    v = seeded((1, 4, k_len, dim), torch.bfloat16, 93, offset=-0.5)
+    out, lse = risa.int8_attention(q, k, v, return_lse=True)
+    keep = slice(0, heads, max(1, heads // 8))  # the oracle checks every eighth head
+    group = heads // 4
+    kv_of = [h // group for h in range(heads)][keep]
+    picked_k = k[:, kv_of]
+    picked_v = v[:, kv_of]
+    prepared = oracle_prequantize(q[:, keep], picked_k, picked_v, return_lse=True)
+    expected, expected_lse, _ = oracle_pipeline.attend(prepared, return_lse=True)
+    assert relative_l2(to_numpy(out[:, keep]), expected) < TOLERANCE
+    assert relative_l2(to_numpy(lse[:, keep]), expected_lse) < TOLERANCE
