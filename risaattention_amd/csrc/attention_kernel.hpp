@@ -771,7 +771,7 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void attention_kernel(cons
     d_part = __builtin_fmaf(static_cast<float>(row_sum), t_scale, d_part);
 
     if constexpr (CAPTURE) {
-      const uint32_t numerator = row_sum + __shfl_xor(row_sum, 32);
+      const uint32_t numerator = sum_across_halves(row_sum);
       if (half == 0 && query_ok) {
         if constexpr (!LAST) {
           // Tile-major: the 32 queries of a half-wave store 256 contiguous bytes.

@@ -156,6 +156,12 @@ __device__ __forceinline__ float max_across_row_pairs(float x) {
   return __builtin_fmaxf(__uint_as_float(both[0]), __uint_as_float(both[1]));
 }
 
+// Integer sum over lanes l and l ^ 32, in both lanes (exact, so the order is free).
+__device__ __forceinline__ uint32_t sum_across_halves(uint32_t x) {
+  const auto both = __builtin_amdgcn_permlane32_swap(x, x, false, false);
+  return both[0] + both[1];
+}
+
 // Accumulator seed of the P·V product.  The matrix cores add integers to whatever
 // 32-bit pattern they start from; starting from the bits of 1.5 * 2^23 (plus the
 // zero-point term) leaves the bits of the float 12582912 + n for every result
