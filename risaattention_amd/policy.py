@@ -74,6 +74,9 @@ def is_available(device: torch.device | int | None = None) -> bool:
     return native.is_available(device)
 
 
+_CHECKED_DEVICES: set[int] = set()  # CUDA device indices that passed is_available()
+
+
 def validate_inputs(q, k, v, attn_mask):
     """Check shapes/dtypes/devices and return the mask broadcast to [B,Hq,Lq,Lk]."""
     if q.ndim != 4 or k.ndim != 4 or v.ndim != 4:
@@ -86,8 +89,13 @@ def validate_inputs(q, k, v, attn_mask):
         )
     if not q.is_cuda or q.device != k.device or q.device != v.device:
         raise ValueError("q, k, and v must be on the same CUDA device")
-    if not is_available(q.device):
-        raise RuntimeError(UNAVAILABLE)
+    # the device check costs several microseconds: done once per device
+    index = q.device.index
+    if index is None or index not in _CHECKED_DEVICES:
+        if not is_available(q.device):
+            raise RuntimeError(UNAVAILABLE)
+        if index is not None:
+            _CHECKED_DEVICES.add(index)
 
     batch, q_heads, q_len, head_dim = q.shape
     k_batch, kv_heads, k_len, k_dim = k.shape
