@@ -890,13 +890,21 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void attention_kernel(cons
       const int scale_pair = KEEP_OFFSETS ? 2 * half : (fresh_lane() >> 5) * 2;
       const float next_ks0 = ks_base[next_tile * 4 + scale_pair];
       const float next_ks1 = ks_base[next_tile * 4 + scale_pair + 1];
+      // Wave priorities by phase: when one wavefront of a SIMD is in its softmax and
+      // the other in a matrix phase, the vector instructions go first.  Matrix and
+      // vector instructions do not overlap on a SIMD; a matrix instruction issued
+      // ahead of short vector work delays a whole dependent chain, the other way
+      // round it costs the matrix phase one issue slot (3 % on the dense kernel).
+      __builtin_amdgcn_s_setprio(0);
       score_tile(stage, k_first, s);
       if constexpr (PREFETCH) {
         load_seed_pair(stage, 0, seed);
         load_v_pair(stage, 0, 0, v_first);
         __builtin_amdgcn_sched_barrier(0);
       }
+      __builtin_amdgcn_s_setprio(2);
       const float t_scale = softmax_tile(std::false_type{}, it, tile, ks0, ks1, s, pk);
+      __builtin_amdgcn_s_setprio(1);
       if constexpr (LATE_COPIES) {
         __builtin_amdgcn_sched_barrier(0);
         issue_tile(next_tile, stage ^ 1);

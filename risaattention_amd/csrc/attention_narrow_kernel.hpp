@@ -350,10 +350,13 @@ __global__ __launch_bounds__(64 * WAVES * KSPLIT) void attention_narrow_kernel(c
       load_k_fragments(lds + stage * Shape::kStageBytes, 0, k_first);
       tile_scales(stage, ks0, ks1);
       issue_tile(tile + 1, stage ^ 1);
+      __builtin_amdgcn_s_setprio(0);  // vector phases before matrix phases, as in the wide kernel
       score_tile(stage, k_first, s);
       load_group(stage, 0, acc_first, v_first);
       __builtin_amdgcn_sched_barrier(0);
+      __builtin_amdgcn_s_setprio(2);
       const float t_scale = softmax_tile(std::false_type{}, tile, ks0, ks1, s, pk);
+      __builtin_amdgcn_s_setprio(1);
       __builtin_amdgcn_sched_barrier(0);
       value_tile(stage, pk, acc_first, v_first, t_scale);
     }
