@@ -1,8 +1,9 @@
-"""``int8_attention`` and its ``torch.compile``-visible operator registration.
+"""``int8_attention`` and the two operators ``torch.compile`` sees.
 
-Counterpart of reference src/risa_attention/dense.py:14-146: the same two
-operators (``risa_attention::int8_attention`` and ``::int8_attention_masked``)
-with fake implementations that only propagate the query shape.
+Operator names and schemas follow reference src/risa_attention/dense.py:14-77
+(``risa_attention::int8_attention`` and ``::int8_attention_masked``, fake
+implementations that only propagate the query shape), so graphs traced against the
+reference keep working.  Eager calls on plain tensors do not go through them.
 """
 
 from __future__ import annotations
@@ -16,28 +17,36 @@ from .prepare import prequantize_int8_attention
 OP_NAMESPACE = "risa_attention"
 
 
-@torch.library.custom_op(f"{OP_NAMESPACE}::int8_attention", mutates_args=())
-def _dense_op(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float | None,
-              use_midpoint_affine: bool, is_causal: bool) -> torch.Tensor:
-    return execute_dense_attention(q, k, v, scale=scale, attn_mask=None,
+def _run(q, k, v, attn_mask, scale, use_midpoint_affine, is_causal):
+    return execute_dense_attention(q, k, v, scale=scale, attn_mask=attn_mask,
                                    use_midpoint_affine=use_midpoint_affine, is_causal=is_causal)
 
 
-@_dense_op.register_fake
-def _(q, k, v, scale, use_midpoint_affine, is_causal):
+def _same_shape_as_query(q, *unused):
     return q.new_empty(q.shape)
+
+
+@torch.library.custom_op(f"{OP_NAMESPACE}::int8_attention", mutates_args=())
+def _dense_op(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float | None,
+              use_midpoint_affine: bool, is_causal: bool) -> torch.Tensor:
+    return _run(q, k, v, None, scale, use_midpoint_affine, is_causal)
 
 
 @torch.library.custom_op(f"{OP_NAMESPACE}::int8_attention_masked", mutates_args=())
 def _masked_op(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, attn_mask: torch.Tensor,
                scale: float | None, use_midpoint_affine: bool, is_causal: bool) -> torch.Tensor:
-    return execute_dense_attention(q, k, v, scale=scale, attn_mask=attn_mask,
-                                   use_midpoint_affine=use_midpoint_affine, is_causal=is_causal)
+    return _run(q, k, v, attn_mask, scale, use_midpoint_affine, is_causal)
 
 
-@_masked_op.register_fake
-def _(q, k, v, attn_mask, scale, use_midpoint_affine, is_causal):
-    return q.new_empty(q.shape)
+_dense_op.register_fake(_same_shape_as_query)
+_masked_op.register_fake(_same_shape_as_query)
+
+
+def _plain_eager(*tensors) -> bool:
+    """Ordinary tensors outside tracing: nothing needs to see an operator boundary."""
+    if torch.compiler.is_compiling():
+        return False
+    return all(t is None or type(t) is torch.Tensor for t in tensors)
 
 
 def int8_attention(
@@ -67,23 +76,22 @@ def int8_attention(
     (taken from the same rounded U8 probabilities as P·V) and V dequantisation
     are FP32.  ``return_lse=True`` also returns natural-log normalisers.
     """
-    if return_lse or kv_permutation is not None:
+    needs_packed_route = return_lse or kv_permutation is not None
+    if needs_packed_route:
+        # the LSE and the permuted order live in the packed container
         packed = prequantize_int8_attention(
             q, k, v, scale=scale, attn_mask=attn_mask, v_quantization=v_quantization,
             is_causal=is_causal, return_lse=return_lse, kv_permutation=kv_permutation,
             fuse_gather=fuse_gather,
         )
         return int8_attention_from_prequantized(packed, return_lse=return_lse)
-    use_midpoint_affine = uses_centered_values(v_quantization)
+    centered = uses_centered_values(v_quantization)
     # Plain eager tensors skip the operator dispatch (about 10 us per call, a third of a
     # short sequence's whole step); tracing, fake and wrapped tensors go through the
     # registered operators so that torch.compile sees them.
-    if (type(q) is torch.Tensor and type(k) is torch.Tensor and type(v) is torch.Tensor
-            and (attn_mask is None or type(attn_mask) is torch.Tensor)
-            and not torch.compiler.is_compiling()):
-        return execute_dense_attention(q, k, v, scale=scale, attn_mask=attn_mask,
-                                       use_midpoint_affine=use_midpoint_affine, is_causal=is_causal)
-    ops = getattr(torch.ops, OP_NAMESPACE)
+    if _plain_eager(q, k, v, attn_mask):
+        return _run(q, k, v, attn_mask, scale, centered, is_causal)
+    operators = getattr(torch.ops, OP_NAMESPACE)
     if attn_mask is None:
-        return ops.int8_attention(q, k, v, scale, use_midpoint_affine, is_causal)
-    return ops.int8_attention_masked(q, k, v, attn_mask, scale, use_midpoint_affine, is_causal)
+        return operators.int8_attention(q, k, v, scale, centered, is_causal)
+    return operators.int8_attention_masked(q, k, v, attn_mask, scale, centered, is_causal)

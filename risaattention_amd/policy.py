@@ -1,8 +1,10 @@
 """Input contracts, mask helpers and the key-tile policy.
 
-Same rules, error types and messages as reference
-src/risa_attention/_validation.py:11-148; the device requirement reads
-"ROCm/gfx950" instead of "CUDA/SM80+".
+The rules, the exception types and the message texts are the contract of reference
+src/risa_attention/_validation.py:11-148 (callers and tests match on them); the device
+requirement reads "HIP extension / gfx950" instead of "CUDA extension / SM80+".  The
+checks are table-driven here: one entry per rule, applied in the reference's order so
+that the first violated rule is the one reported.
 """
 
 from __future__ import annotations
@@ -12,47 +14,76 @@ import torch
 from . import native
 
 DTYPE_CODES = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}
-MASK_DTYPE_CODES = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2, torch.bool: 3}
-SUPPORTED_DTYPES = (torch.float32, torch.float16, torch.bfloat16)
+MASK_DTYPE_CODES = {**DTYPE_CODES, torch.bool: 3}
+SUPPORTED_DTYPES = tuple(DTYPE_CODES)
+QUERY_BLOCK_SIZE = 128
 KEY_BLOCK_SIZE = 64
 LARGE_KEY_BLOCK_SIZE = 128
-QUERY_BLOCK_SIZE = 128
 MIN_PATTERN_SPARSITY = 0.05
 OUTPUT_LAYOUTS = ("hnd", "nhd")
 VALUE_QUANTIZATION_MODES = ("midpoint_affine", "absmax")
 
 UNAVAILABLE = "INT8 attention requires the risaattention_amd HIP extension and a gfx950 (MI355X) GPU"
 
+# rule -> (exception type, message template)
+_RULES = {
+    "rank": (ValueError, "q, k, and v must have shape [batch, heads, sequence, head_dim]"),
+    "dtype": (TypeError, "q, k, and v must be float32, float16, or bfloat16, got {dtype}"),
+    "same_dtype": (TypeError, "q, k, and v must have the same dtype, got {q}, {k}, and {v}"),
+    "device": (ValueError, "q, k, and v must be on the same CUDA device"),
+    "unavailable": (RuntimeError, UNAVAILABLE),
+    "v_shape": (ValueError, "v must have shape [q.batch, k.heads, k.sequence, q.head_dim], got {shape}"),
+    "qk_shape": (ValueError, "q and k batch/head dimensions must match, got {q} and {k}"),
+    "empty": (ValueError, "batch, head counts, and sequence lengths must be positive"),
+    "groups": (ValueError, "q head count ({q}) must be divisible by k/v head count ({kv})"),
+    "head_dim": (ValueError, "head_dim must be in [1, 256], got {head_dim}"),
+    "stride": (ValueError, "the last dimension of q, k, and v must be contiguous"),
+    "mask_device": (ValueError, "attn_mask must be on the same CUDA device as q, k, and v"),
+    "mask_dtype": (TypeError, "attn_mask must be bool, float16, bfloat16, or float32"),
+    "mask_shape": (ValueError, "attn_mask must be broadcastable to [{b}, {h}, {lq}, {lk}], got {shape}"),
+    "v_mode": (ValueError, "v_quantization must be one of {modes}, got {mode!r}"),
+}
+
+
+def _violation(rule: str, **values) -> Exception:
+    kind, template = _RULES[rule]
+    return kind(template.format(**values))
+
 
 def uses_centered_values(v_quantization: str) -> bool:
+    """True for ``midpoint_affine``, False for ``absmax``; anything else is an error."""
     if v_quantization not in VALUE_QUANTIZATION_MODES:
-        raise ValueError(
-            f"v_quantization must be one of {VALUE_QUANTIZATION_MODES}, got {v_quantization!r}"
-        )
-    return v_quantization == "midpoint_affine"
+        raise _violation("v_mode", modes=VALUE_QUANTIZATION_MODES, mode=v_quantization)
+    return v_quantization == VALUE_QUANTIZATION_MODES[0]
 
 
 def mask_signature(mask: torch.Tensor | None) -> tuple | None:
-    """Identity of a mask's storage and contents version (None for no mask)."""
+    """What identifies a mask for a retained pattern: its storage, layout and contents version.
+
+    Inference tensors have no version counter (reading it raises); their entry is None and
+    the caller must leave them unchanged while a pattern built under them is in use.
+    """
     if mask is None:
         return None
     try:
         version = mask._version
-    except RuntimeError:  # inference tensors carry no version counter
+    except RuntimeError:
         version = None
-    return (mask.data_ptr(), version, tuple(mask.shape), tuple(mask.stride()), mask.dtype, mask.device)
+    layout = (tuple(mask.shape), tuple(mask.stride()), mask.dtype, mask.device)
+    return (mask.data_ptr(), version, *layout)
 
 
 def apply_score_mask(scores, attn_mask, is_causal, start):
-    """FP32 masking of a block of score rows beginning at query ``start``."""
-    rows = scores.shape[-2]
+    """Mask FP32 score rows ``start .. start + rows`` the way the kernels do: boolean masks
+    hide, floating-point masks add, the causal rule hides keys after the query."""
+    rows, keys = scores.shape[-2], scores.shape[-1]
     if attn_mask is not None:
-        window = attn_mask[..., start : start + rows, :]
-        scores = scores.masked_fill(~window, -torch.inf) if window.dtype == torch.bool else scores + window
+        window = attn_mask.narrow(-2, start, rows)
+        scores = scores + window if window.dtype != torch.bool else scores.masked_fill(window.logical_not(), -torch.inf)
     if is_causal:
-        q_index = torch.arange(start, start + rows, device=scores.device)[:, None]
-        k_index = torch.arange(scores.shape[-1], device=scores.device)[None, :]
-        scores = scores.masked_fill(k_index > q_index, -torch.inf)
+        query_index = torch.arange(start, start + rows, device=scores.device).unsqueeze(1)
+        future = torch.arange(keys, device=scores.device).unsqueeze(0) > query_index
+        scores = scores.masked_fill(future, -torch.inf)
     return scores
 
 
@@ -61,7 +92,8 @@ def pad_key_length(length: int, key_block_size: int = KEY_BLOCK_SIZE) -> int:
 
 
 def kernel_head_dim(head_dim: int) -> int:
-    return 64 if head_dim <= 64 else 128 if head_dim <= 128 else 256
+    """Head dim the kernels run with: the next of 64, 128, 256."""
+    return next(width for width in (64, 128, 256) if head_dim <= width)
 
 
 def select_key_block_size(kernel_dim: int, key_length: int, *, has_mask: bool) -> int:
@@ -74,59 +106,55 @@ def is_available(device: torch.device | int | None = None) -> bool:
     return native.is_available(device)
 
 
-_CHECKED_DEVICES: set[int] = set()  # CUDA device indices that passed is_available()
+_CHECKED_DEVICES: set[int] = set()  # device indices that passed is_available(): it costs microseconds per call
+
+
+def _require_device(device: torch.device) -> None:
+    index = device.index
+    if index is not None and index in _CHECKED_DEVICES:
+        return
+    if not is_available(device):
+        raise _violation("unavailable")
+    if index is not None:
+        _CHECKED_DEVICES.add(index)
 
 
 def validate_inputs(q, k, v, attn_mask):
-    """Check shapes/dtypes/devices and return the mask broadcast to [B,Hq,Lq,Lk]."""
-    if q.ndim != 4 or k.ndim != 4 or v.ndim != 4:
-        raise ValueError("q, k, and v must have shape [batch, heads, sequence, head_dim]")
-    if q.dtype not in SUPPORTED_DTYPES:
-        raise TypeError(f"q, k, and v must be float32, float16, or bfloat16, got {q.dtype}")
-    if q.dtype != k.dtype or q.dtype != v.dtype:
-        raise TypeError(
-            f"q, k, and v must have the same dtype, got {q.dtype}, {k.dtype}, and {v.dtype}"
-        )
-    if not q.is_cuda or q.device != k.device or q.device != v.device:
-        raise ValueError("q, k, and v must be on the same CUDA device")
-    # the device check costs several microseconds: done once per device
-    index = q.device.index
-    if index is None or index not in _CHECKED_DEVICES:
-        if not is_available(q.device):
-            raise RuntimeError(UNAVAILABLE)
-        if index is not None:
-            _CHECKED_DEVICES.add(index)
+    """Check Q, K, V and the mask; return the mask as a ``[B, Hq, Lq, Lk]`` broadcast view."""
+    operands = (q, k, v)
+    if any(t.ndim != 4 for t in operands):
+        raise _violation("rank")
+    if q.dtype not in DTYPE_CODES:
+        raise _violation("dtype", dtype=q.dtype)
+    if any(t.dtype != q.dtype for t in operands):
+        raise _violation("same_dtype", q=q.dtype, k=k.dtype, v=v.dtype)
+    if not q.is_cuda or any(t.device != q.device for t in operands):
+        raise _violation("device")
+    _require_device(q.device)
 
     batch, q_heads, q_len, head_dim = q.shape
-    k_batch, kv_heads, k_len, k_dim = k.shape
-    if v.shape != (batch, kv_heads, k_len, head_dim):
-        raise ValueError(
-            f"v must have shape [q.batch, k.heads, k.sequence, q.head_dim], got {tuple(v.shape)}"
-        )
-    if k_batch != batch or k_dim != head_dim:
-        raise ValueError(
-            f"q and k batch/head dimensions must match, got {tuple(q.shape)} and {tuple(k.shape)}"
-        )
-    if 0 in (batch, q_heads, kv_heads, q_len, k_len):
-        raise ValueError("batch, head counts, and sequence lengths must be positive")
-    if q_heads % kv_heads != 0:
-        raise ValueError(
-            f"q head count ({q_heads}) must be divisible by k/v head count ({kv_heads})"
-        )
-    if head_dim <= 0 or head_dim > 256:
-        raise ValueError(f"head_dim must be in [1, 256], got {head_dim}")
-    if q.stride(-1) != 1 or k.stride(-1) != 1 or v.stride(-1) != 1:
-        raise ValueError("the last dimension of q, k, and v must be contiguous")
+    kv_heads, k_len = k.shape[1], k.shape[2]
+    if tuple(v.shape) != (batch, kv_heads, k_len, head_dim):
+        raise _violation("v_shape", shape=tuple(v.shape))
+    if (k.shape[0], k.shape[3]) != (batch, head_dim):
+        raise _violation("qk_shape", q=tuple(q.shape), k=tuple(k.shape))
+    if min(batch, q_heads, kv_heads, q_len, k_len) == 0:
+        raise _violation("empty")
+    if q_heads % kv_heads:
+        raise _violation("groups", q=q_heads, kv=kv_heads)
+    if not 1 <= head_dim <= 256:
+        raise _violation("head_dim", head_dim=head_dim)
+    if any(t.stride(-1) != 1 for t in operands):
+        raise _violation("stride")
+
     if attn_mask is None:
         return None
     if attn_mask.device != q.device:
-        raise ValueError("attn_mask must be on the same CUDA device as q, k, and v")
+        raise _violation("mask_device")
     if attn_mask.dtype not in MASK_DTYPE_CODES:
-        raise TypeError("attn_mask must be bool, float16, bfloat16, or float32")
+        raise _violation("mask_dtype")
     try:
-        return torch.broadcast_to(attn_mask, (batch, q_heads, q_len, k_len))
+        return attn_mask.broadcast_to((batch, q_heads, q_len, k_len))
     except RuntimeError as error:
-        raise ValueError(
-            "attn_mask must be broadcastable to "
-            f"[{batch}, {q_heads}, {q_len}, {k_len}], got {tuple(attn_mask.shape)}"
-        ) from error
+        raise _violation("mask_shape", b=batch, h=q_heads, lq=q_len, lk=k_len,
+                         shape=tuple(attn_mask.shape)) from error
