@@ -197,6 +197,41 @@ def workload_sparse(torch, risa, args, device):
     return rows
 
 
+def workload_sparse_blocks(torch, risa, args, device):
+    """The sparse table of the reference's README: Q/K = N(0,1) + one of two prototypes of
+    norm 8 per 128-token block (alternating), theta = 0.99, construction on the clean
+    tensors, reuse on tensors drifted by 0.05 (reference benchmarks/sparse.py:30-60,
+    README.md:127-142).  About half of the key tiles carry the mass of every query block."""
+    rows = []
+    dim, kv_heads, q_heads = SHAPE["head_dim"], SHAPE["kv_heads"], SHAPE["q_heads"]
+    for length in ([args.length] if args.length else (1024, 2048, 4096, 8192, 16384, 32768)):
+        generator = torch.Generator(device=device).manual_seed(0)
+        draw = lambda *shape: torch.randn(shape, generator=generator, device=device)
+        clean_q, clean_k, v32 = draw(1, q_heads, length, dim), draw(1, kv_heads, length, dim), draw(1, kv_heads, length, dim)
+        prototypes = draw(1, kv_heads, 2, dim)
+        prototypes = prototypes * (8.0 / prototypes.norm(dim=-1, keepdim=True))
+        block = (torch.arange(length, device=device) // 128) % 2
+        clean_k = clean_k + prototypes[:, :, block]
+        clean_q = clean_q + prototypes.repeat_interleave(q_heads // kv_heads, 1)[:, :, block]
+        drifted_q = (clean_q + 0.05 * draw(*clean_q.shape)).bfloat16()
+        drifted_k = (clean_k + 0.05 * draw(*clean_k.shape)).bfloat16()
+        q0, k0, v = clean_q.bfloat16(), clean_k.bfloat16(), v32.bfloat16()
+        reference = fp32_reference(torch, drifted_q, drifted_k, v)
+        for mode in ("absmax", "midpoint_affine"):
+            build = lambda: risa.construct_sparse_int8_attention(q0, k0, v, theta=0.99, v_quantization=mode)
+            construct_ms = time_calls(torch, build, 5, 2)
+            _, pattern = build()
+            dense = lambda: risa.int8_attention(drifted_q, drifted_k, v, v_quantization=mode)
+            sparse = lambda: risa.sparse_int8_attention(drifted_q, drifted_k, v, pattern, v_quantization=mode)
+            dense_ms, sparse_ms = time_calls(torch, dense, 20, 3), time_calls(torch, sparse, 20, 3)
+            rows.append({"N": length, "v_quantization": mode, "construct_ms": round(construct_ms, 4),
+                         "dense_ms": round(dense_ms, 4), "sparse_ms": round(sparse_ms, 4),
+                         "speedup": round(dense_ms / sparse_ms, 3), "coverage": round(pattern.coverage, 4),
+                         "sparse_sqnr_db": round(sqnr_db(torch, sparse(), reference), 2),
+                         "dense_sqnr_db": round(sqnr_db(torch, dense(), reference), 2)})
+    return rows
+
+
 def workload_prepare(torch, risa, args, device):
     """Q/K/V preparation alone at the headline head counts: the one-call entry point
     (merged launches) against risa_quantize_qk + risa_quantize_v (one launch per kernel)."""
@@ -326,7 +361,7 @@ def main():
     parser.add_argument("--mode", default="absmax", choices=["absmax", "midpoint_affine"])
     parser.add_argument("--no-cpu-baseline", action="store_true")
     parser.add_argument("--no-accuracy", action="store_true")
-    parser.add_argument("--workload", default="dense", choices=["dense", "sweep", "masked", "sparse", "video", "prepare"],
+    parser.add_argument("--workload", default="dense", choices=["dense", "sweep", "masked", "sparse", "sparse_blocks", "video", "prepare"],
                         help="dense = headline N=32K line (default); the others are the remaining benchmark "
                              "configurations of the reference, reported as one JSON line each")
     parser.add_argument("--calibrate-copy", action="store_true",
@@ -356,7 +391,8 @@ def main():
         return
     if args.workload != "dense":
         runner = {"sweep": workload_sweep, "masked": workload_masked, "sparse": workload_sparse,
-                  "video": workload_video, "prepare": workload_prepare}[args.workload]
+                  "video": workload_video, "prepare": workload_prepare,
+                  "sparse_blocks": workload_sparse_blocks}[args.workload]
         wall = time.perf_counter()
         rows = runner(torch, risa, args, device)
         print(json.dumps({"metric": f"{args.workload} workload (see config.rows)", "value": None, "unit": "ms",

@@ -154,7 +154,10 @@ int risa_attention(const void* q_int8, const void* k_int8, const void* v_int8, v
  * aligned).  q/k/v are [B,H,L,D] with element strides, head_dim 64, 128 or 256;
  * out and the mask as for risa_attention; mask_batch / mask_heads are the mask's
  * own extents (1 where it broadcasts).  key_only_mask in the size query says
- * whether a mask with query stride 0 will be passed.
+ * whether a mask with query stride 0 will be passed.  sparse_row_offsets /
+ * sparse_block_indices (both or neither, as for risa_attention) restrict the
+ * attention to a retained-mass pattern: the reuse call of the sparse path
+ * (reference src/risa_attention/sparse.py:150-191) in one call as well.
  */
 size_t risa_sdpa_workspace_bytes(int batch, int q_heads, int q_len, int kv_heads, int k_len,
                                  int head_dim, int cta_k, int midpoint_affine, int key_only_mask);
@@ -166,7 +169,8 @@ int risa_sdpa(const void* q, const void* k, const void* v, void* out, void* work
               int64_t out_stride_h, float sm_scale, int input_dtype, int output_dtype,
               int midpoint_affine, const void* mask, int64_t mask_stride_b, int64_t mask_stride_h,
               int64_t mask_stride_q, int64_t mask_stride_k, int mask_dtype, int mask_batch,
-              int mask_heads, int is_causal, void* stream);
+              int mask_heads, int is_causal, const int32_t* sparse_row_offsets,
+              const int32_t* sparse_block_indices, void* stream);
 
 /*
  * Retained-mass selection over masses already sorted in descending order.

@@ -170,10 +170,15 @@ def execute_dense_attention(
     attn_mask: torch.Tensor | None = None,
     use_midpoint_affine: bool = False,
     is_causal: bool = False,
+    sparse_pattern: RetainedMassPattern | None = None,
+    output_layout: str = "hnd",
 ) -> torch.Tensor:
     """Quantize and attend in one native call; the intermediate buffers are sections of
     one workspace that lives only for the call (reference _execution.py:28-134 over
-    ``_C.risa_sdpa``)."""
+    ``_C.risa_sdpa``).  With ``sparse_pattern`` the attention walks the pattern's key tiles
+    (the reuse call of the sparse path); a pattern under 5 % sparsity runs dense."""
+    if output_layout not in OUTPUT_LAYOUTS:
+        raise ValueError(f"output_layout must be one of {OUTPUT_LAYOUTS}, got {output_layout!r}")
     attn_mask = validate_inputs(q, k, v, attn_mask)
     original_dim, input_dtype = q.shape[-1], q.dtype
     q, k, v, dim = pad_head_dim(q, k, v)
@@ -184,7 +189,18 @@ def execute_dense_attention(
     key_only = attn_mask is not None and not query_mask
     cta_k = select_key_block_size(dim, k_len, has_mask=query_mask)
     lib = native.library()
-    output = torch.empty(batch, q_heads, q_len, dim, dtype=output_dtype_for(input_dtype), device=q.device)
+    csr = (None, None)
+    if sparse_pattern is not None:
+        check_pattern_for(sparse_pattern, batch=batch, q_heads=q_heads, q_len=q_len, k_len=k_len, cta_k=cta_k,
+                          attention_scale=attention_scale, is_causal=bool(is_causal), attn_mask=attn_mask,
+                          device=q.device)
+        if sparse_pattern.sparsity >= MIN_PATTERN_SPARSITY:
+            csr = (sparse_pattern.row_offsets.data_ptr(), sparse_pattern.block_indices.data_ptr())
+    out_dtype = output_dtype_for(input_dtype)
+    if output_layout == "nhd":
+        output = torch.empty(batch, q_len, q_heads, dim, dtype=out_dtype, device=q.device).permute(0, 2, 1, 3)
+    else:
+        output = torch.empty(batch, q_heads, q_len, dim, dtype=out_dtype, device=q.device)
     workspace = torch.empty(
         lib.risa_sdpa_workspace_bytes(batch, q_heads, q_len, kv_heads, k_len, dim, cta_k,
                                       int(use_midpoint_affine), int(key_only)),
@@ -201,7 +217,7 @@ def execute_dense_attention(
             q.stride(0), q.stride(1), q.stride(2), k.stride(0), k.stride(1), k.stride(2),
             v.stride(0), v.stride(1), v.stride(2), output.stride(0), output.stride(2), output.stride(1),
             attention_scale, DTYPE_CODES[input_dtype], DTYPE_CODES[output.dtype],
-            int(use_midpoint_affine), *mask_args, int(bool(is_causal)),
+            int(use_midpoint_affine), *mask_args, int(bool(is_causal)), *csr,
             native.current_stream(q.device),
         )
     )
@@ -210,28 +226,38 @@ def execute_dense_attention(
     return output.float() if input_dtype == torch.float32 else output
 
 
-def check_pattern(quantized: PrequantizedInt8Attention, pattern: RetainedMassPattern) -> None:
+def check_pattern_for(pattern: RetainedMassPattern, *, batch, q_heads, q_len, k_len, cta_k,
+                      attention_scale, is_causal, attn_mask, device) -> None:
+    """A pattern may only drive the attention problem it was built for
+    (reference _execution.py:180-228)."""
     if not isinstance(pattern, RetainedMassPattern):
         raise TypeError("sparse_pattern must be returned by build_retained_mass_pattern")
-    if pattern.is_causal != quantized.is_causal:
+    if pattern.is_causal != is_causal:
         raise ValueError("sparse pattern and attention call must use the same is_causal")
-    if pattern.mask_signature != mask_signature(quantized.attn_mask):
+    if pattern.mask_signature != mask_signature(attn_mask):
         raise ValueError("sparse pattern mask has changed; rebuild the pattern")
-    expected = (*quantized.q.shape[:3], quantized.k.shape[2], QUERY_BLOCK_SIZE, quantized.cta_k)
+    expected = (batch, q_heads, q_len, k_len, QUERY_BLOCK_SIZE, cta_k)
     actual = (pattern.batch_size, pattern.q_heads, pattern.q_length, pattern.kv_length,
               pattern.query_block_size, pattern.key_block_size)
     if actual != expected:
         raise ValueError(
             f"sparse pattern metadata does not match packed attention: expected {expected}, got {actual}"
         )
-    if not math.isclose(pattern.attention_scale, quantized.attention_scale, rel_tol=1e-7, abs_tol=0.0):
+    if not math.isclose(pattern.attention_scale, attention_scale, rel_tol=1e-7, abs_tol=0.0):
         raise ValueError("sparse pattern and attention call must use the same scale")
-    device = quantized.q.device
     if pattern.row_offsets.device != device or pattern.block_indices.device != device:
         raise ValueError("sparse pattern and packed tensors must be on the same CUDA device")
     for index in (pattern.row_offsets, pattern.block_indices):
         if index.dtype != torch.int32 or not index.is_contiguous():
             raise TypeError("sparse CSR row offsets and block indices must be contiguous int32")
+
+
+def check_pattern(quantized: PrequantizedInt8Attention, pattern: RetainedMassPattern) -> None:
+    batch, q_heads, q_len = quantized.q.shape[:3]
+    check_pattern_for(pattern, batch=batch, q_heads=q_heads, q_len=q_len, k_len=quantized.k.shape[2],
+                      cta_k=quantized.cta_k, attention_scale=quantized.attention_scale,
+                      is_causal=quantized.is_causal, attn_mask=quantized.attn_mask,
+                      device=quantized.q.device)
 
 
 def int8_attention_from_prequantized(

@@ -365,7 +365,8 @@ int risa_sdpa(const void* q, const void* k, const void* v, void* out, void* work
               int64_t out_stride_h, float sm_scale, int input_dtype, int output_dtype,
               int midpoint_affine, const void* mask, int64_t mask_stride_b, int64_t mask_stride_h,
               int64_t mask_stride_q, int64_t mask_stride_k, int mask_dtype, int mask_batch,
-              int mask_heads, int is_causal, void* stream) {
+              int mask_heads, int is_causal, const int32_t* sparse_row_offsets,
+              const int32_t* sparse_block_indices, void* stream) {
   using risa::fail;
   if (batch <= 0 || q_heads <= 0 || q_len <= 0 || kv_heads <= 0 || k_len <= 0 ||
       (cta_k != 64 && cta_k != 128))
@@ -419,7 +420,7 @@ int risa_sdpa(const void* q, const void* k, const void* v, void* out, void* work
     bias_stride_h = mask_heads > 1 ? padded : 0;
     bias_stride_b = mask_batch > 1 ? static_cast<int64_t>(mask_heads) * padded : 0;
     // tile lists pay off under the conditions of reference _key_mask.py:9-28
-    if (k_len > 1024 && q_len >= 256 && sm_scale > 0.0f && is_causal == 0) {
+    if (k_len > 1024 && q_len >= 256 && sm_scale > 0.0f && is_causal == 0 && sparse_row_offsets == nullptr) {
       auto* list = reinterpret_cast<int32_t*>(base + l.key_tiles);
       status = risa_prepare_key_mask_tiles(mask, list, batch, q_heads, k_len, cta_k, mask_stride_b,
                                            mask_stride_h, mask_stride_k, mask_dtype, stream);
@@ -431,8 +432,8 @@ int risa_sdpa(const void* q, const void* k, const void* v, void* out, void* work
                         v_scale, v_center, tile_sum, mask, mask_stride_b, mask_stride_h,
                         mask_stride_q, mask_stride_k, mask_dtype, cta_k, batch, q_len, k_len,
                         q_heads, kv_heads, head_dim, out_stride_b, out_stride_n, out_stride_h,
-                        sm_scale, output_dtype, nullptr, nullptr, nullptr, is_causal, nullptr,
-                        key_tiles, key_bias, bias_stride_b, bias_stride_h, stream);
+                        sm_scale, output_dtype, sparse_row_offsets, sparse_block_indices, nullptr,
+                        is_causal, nullptr, key_tiles, key_bias, bias_stride_b, bias_stride_h, stream);
 }
 
 }  // extern "C"

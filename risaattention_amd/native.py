@@ -61,7 +61,7 @@ SIGNATURES = {
     "risa_sdpa": (
         _c_int,
         [_c_ptr] * 5 + [_c_size] + [_c_int] * 7 + [_c_i64] * 12 + [_c_f32, _c_int, _c_int, _c_int]
-        + [_c_ptr] + [_c_i64] * 4 + [_c_int] * 4 + [_c_ptr],
+        + [_c_ptr] + [_c_i64] * 4 + [_c_int] * 4 + [_c_ptr, _c_ptr, _c_ptr],
     ),
     "risa_selector_workspace_size": (_c_size, [_c_int]),
     "risa_select_retained_mass": (_c_int, [_c_ptr] * 8 + [_c_int, _c_int, _c_f64, _c_ptr]),

@@ -10,8 +10,8 @@ import math
 import torch
 
 from . import native
-from .attend import int8_attention_from_prequantized
-from .policy import QUERY_BLOCK_SIZE, mask_signature
+from .attend import execute_dense_attention, int8_attention_from_prequantized
+from .policy import QUERY_BLOCK_SIZE, mask_signature, uses_centered_values
 from .prepare import prequantize_int8_attention
 from .types import PrequantizedInt8Attention, RetainedMassPattern
 
@@ -126,8 +126,9 @@ def sparse_int8_attention(
     is_causal: bool = False,
     attn_mask: torch.Tensor | None = None,
 ) -> torch.Tensor:
-    """INT8 attention over a frozen pattern; Q/K/V are quantised again on every call."""
-    packed = prequantize_int8_attention(q, k, v, scale=scale, v_quantization=v_quantization,
-                                        is_causal=is_causal, attn_mask=attn_mask)
-    return int8_attention_from_prequantized(packed, sparse_pattern=sparse_pattern,
-                                            output_layout=output_layout)
+    """INT8 attention over a frozen pattern; Q/K/V are quantised again on every call
+    (one native call: preparation and the walk over the pattern's key tiles)."""
+    return execute_dense_attention(q, k, v, scale=scale, attn_mask=attn_mask,
+                                   use_midpoint_affine=uses_centered_values(v_quantization),
+                                   is_causal=is_causal, sparse_pattern=sparse_pattern,
+                                   output_layout=output_layout)
