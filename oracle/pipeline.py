@@ -43,9 +43,9 @@ def _expand_mask(mask, batch, heads, q_len, k_len):
     mask = np.asarray(mask)
     while mask.ndim < 4:
         mask = mask[None]
+    # Callers that hold the broadcast view's strides override this (a contiguous
+    # [..., 1, Lk] mask over one query has a non-zero query stride in the reference).
     query_dependent = mask.shape[2] != 1
-    if mask.shape[2] == 1 and q_len == 1:
-        query_dependent = False
     target_q = q_len if query_dependent else 1
     return np.broadcast_to(mask, (batch, heads, target_q, k_len)), query_dependent
 

@@ -28,6 +28,12 @@ def mask_to_numpy(mask: torch.Tensor | None):
 
 
 def oracle_prequantize(q, k, v, *, attn_mask=None, **kwargs):
+    if attn_mask is not None and "query_dependent_mask" not in kwargs:
+        # The key tile policy looks at the broadcast view's query stride (reference
+        # src/risa_attention/_quantization.py:90), which numpy's copy of the mask loses: a
+        # contiguous [..., 1, Lk] mask over a single query keeps a non-zero stride there.
+        view = attn_mask.broadcast_to((q.shape[0], q.shape[1], q.shape[2], k.shape[2]))
+        kwargs["query_dependent_mask"] = view.stride(-2) != 0
     return oracle_pipeline.prequantize(
         to_numpy(q), to_numpy(k), to_numpy(v), mask=mask_to_numpy(attn_mask),
         dtype_name=DTYPE_NAMES[q.dtype], **kwargs,
