@@ -44,6 +44,13 @@ typedef float v4f __attribute__((ext_vector_type(4)));
 constexpr float kLog2e = 1.44269504088896340736f;
 constexpr float kU8Offset = 7.9943534f;
 constexpr float kRowFloor = -50000.0f;
+// The score accumulators start at the bit pattern of 1.5 * 2^23 instead of zero: with
+// |Q.K| < 2^22 (at most 256 products of signed bytes) the INT32 result, read as FP32, is
+// exactly 1.5 * 2^23 + Q.K, so one exact subtraction replaces the slower integer-to-float
+// conversion.  Integer comparisons of seeded accumulators order like the raw scores.
+constexpr int kScoreSeedBits = 0x4B400000;
+constexpr float kScoreSeed = 12582912.0f;
+__device__ __forceinline__ float score_value(int seeded) { return __int_as_float(seeded) - kScoreSeed; }
 constexpr int kQueryBlock = 128;
 
 struct KernelParams {
@@ -441,6 +448,9 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void attention_kernel(cons
     for (int rb = 0; rb < RB; ++rb)
       frag[rb] = *reinterpret_cast<const v4i*>(kl + swizzled<D>(rb * 32 + l32, kk * 2 + half));
   };
+  v16i score_seed;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) score_seed[i] = kScoreSeedBits;
   auto score_tile = [&](int stage, v4i (&first)[RB], v16i (&s)[RB]) {
     const unsigned char* kl = lds + stage * Shape::kStageBytes;
     v4i frag[2][RB];
@@ -453,8 +463,7 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void attention_kernel(cons
 #pragma unroll
       for (int rb = 0; rb < RB; ++rb) {
         if (kk == 0) {
-          const v16i zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-          s[rb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(frag[kk & 1][rb], qreg[kk], zero, 0, 0, 0);
+          s[rb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(frag[kk & 1][rb], qreg[kk], score_seed, 0, 0, 0);
         } else {
           s[rb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(frag[kk & 1][rb], qreg[kk], s[rb], 0, 0, 0);
         }
@@ -494,8 +503,8 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void attention_kernel(cons
           else
             mx0 = max(mx0, s[rb][i]);
         }
-      tile_m = __builtin_fmaxf(__builtin_fmaf(static_cast<float>(mx0), sc0, -kU8Offset),
-                               __builtin_fmaf(static_cast<float>(mx1), sc1, -kU8Offset));
+      tile_m = __builtin_fmaxf(__builtin_fmaf(score_value(mx0), sc0, -kU8Offset),
+                               __builtin_fmaf(score_value(mx1), sc1, -kU8Offset));
       tile_m = max_across_halves(tile_m);
       const float neg_m = -tile_m;
 #pragma unroll
@@ -505,7 +514,7 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void attention_kernel(cons
           uint32_t packed = 0;
 #pragma unroll
           for (int r = 0; r < 4; ++r) {
-            const float x = __builtin_fmaf(static_cast<float>(s[rb][b4 * 4 + r]), (r & 2) ? sc1 : sc0, neg_m);
+            const float x = __builtin_fmaf(score_value(s[rb][b4 * 4 + r]), (r & 2) ? sc1 : sc0, neg_m);
             packed = __builtin_amdgcn_cvt_pk_u8_f32(__builtin_amdgcn_exp2f(x), r, packed);
           }
           row_sum = __builtin_amdgcn_udot4(packed, 0x01010101u, row_sum, false);
@@ -520,7 +529,7 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void attention_kernel(cons
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
           const int key = key0 + rb * 32 + (i >> 2) * 8 + (i & 3);
-          const float raw = key < p.k_len ? static_cast<float>(s[rb][i]) : -1.0e30f;
+          const float raw = key < p.k_len ? score_value(s[rb][i]) : -1.0e30f;
           s[rb][i] = __float_as_int(raw);
           if (i & 2)
             mx1 = __builtin_fmaxf(mx1, raw);
@@ -558,7 +567,7 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void attention_kernel(cons
         for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
           for (int i = 0; i < 16; ++i) {
-            const float value = static_cast<float>(s[rb][i]) * ((i & 2) ? sc1 : sc0);
+            const float value = score_value(s[rb][i]) * ((i & 2) ? sc1 : sc0);
             s[rb][i] = __float_as_int(value);
             mx = __builtin_fmaxf(mx, value);
           }
@@ -583,7 +592,7 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void attention_kernel(cons
               const float terms[4] = {bias[0], bias[1], bias[2], bias[3]};
 #pragma unroll
               for (int r = 0; r < 4; ++r) {
-                float value = static_cast<float>(s[rb][b4 * 4 + r]) * ((r & 2) ? sc1 : sc0) + terms[r];
+                float value = score_value(s[rb][b4 * 4 + r]) * ((r & 2) ? sc1 : sc0) + terms[r];
                 if constexpr (DIAGONAL) {
                   if (tile * CTA_K + local + r > query) value = neg_inf;
                 }
@@ -704,7 +713,7 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void attention_kernel(cons
               }
 #pragma unroll
               for (int r = 0; r < 4; ++r) {
-                float value = static_cast<float>(s[rb][b4 * 4 + r]) * ((r & 2) ? sc1 : sc0);
+                float value = score_value(s[rb][b4 * 4 + r]) * ((r & 2) ? sc1 : sc0);
                 if constexpr (DT >= 0) value = keep[r] ? value + bias[r] * kLog2e : neg_inf;
                 if constexpr (DIAGONAL) {
                   if (key + r > query) value = neg_inf;

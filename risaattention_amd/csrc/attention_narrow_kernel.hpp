@@ -198,8 +198,9 @@ __global__ __launch_bounds__(64 * WAVES * KSPLIT) void attention_narrow_kernel(c
 #pragma unroll
       for (int kb = 0; kb < KB; ++kb) {
         if (kk == 0) {
-          const v4i zero = {0, 0, 0, 0};
-          s[kb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(frag[kk & 1][kb], qreg[kk], zero, 0, 0, 0);
+          // seeded like the wide kernel's scores (kScoreSeedBits)
+          const v4i seed = {kScoreSeedBits, kScoreSeedBits, kScoreSeedBits, kScoreSeedBits};
+          s[kb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(frag[kk & 1][kb], qreg[kk], seed, 0, 0, 0);
         } else {
           s[kb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(frag[kk & 1][kb], qreg[kk], s[kb], 0, 0, 0);
         }
@@ -228,8 +229,8 @@ __global__ __launch_bounds__(64 * WAVES * KSPLIT) void attention_narrow_kernel(c
           else
             mx0 = max(mx0, s[kb][i]);
         }
-      tile_m = __builtin_fmaxf(__builtin_fmaf(static_cast<float>(mx0), sc0, -kU8Offset),
-                               __builtin_fmaf(static_cast<float>(mx1), sc1, -kU8Offset));
+      tile_m = __builtin_fmaxf(__builtin_fmaf(score_value(mx0), sc0, -kU8Offset),
+                               __builtin_fmaf(score_value(mx1), sc1, -kU8Offset));
     } else {
       // Last tile: out-of-range keys become -1e30 and every scale group's maximum
       // starts from -50000 before scaling.
@@ -240,7 +241,7 @@ __global__ __launch_bounds__(64 * WAVES * KSPLIT) void attention_narrow_kernel(c
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           const int key = key0 + (kb >> 2) * 64 + (kb & 3) * 8 + i;
-          const float raw = key < p.k_len ? static_cast<float>(s[kb][i]) : -1.0e30f;
+          const float raw = key < p.k_len ? score_value(s[kb][i]) : -1.0e30f;
           s[kb][i] = __float_as_int(raw);
           if (i & 2)
             mx1 = __builtin_fmaxf(mx1, raw);
@@ -256,7 +257,7 @@ __global__ __launch_bounds__(64 * WAVES * KSPLIT) void attention_narrow_kernel(c
       uint32_t packed = 0;
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const float raw = LAST ? __int_as_float(s[kb][i]) : static_cast<float>(s[kb][i]);
+        const float raw = LAST ? __int_as_float(s[kb][i]) : score_value(s[kb][i]);
         const float x = __builtin_fmaf(raw, (i & 2) ? sc1 : sc0, neg_m);
         packed = __builtin_amdgcn_cvt_pk_u8_f32(__builtin_amdgcn_exp2f(x), i, packed);
       }
