@@ -102,13 +102,13 @@ void launch_stages(const FusedArgs& a, hipStream_t stream) {
           a.v.stride_h, a.v.stride_n, a.v.permutation);
     } else {
       const int threads = summation_threads(a.v.length);
-      const int per_block = 256 / (a.v.head_dim / 8);
+      const int per_block = 256 / (a.v.head_dim / 4);
       const int rows = a.kv * a.v.head_dim;
       dim3 residual_grid(threads / per_block, a.kv);
       value_residual_kernel<DT><<<residual_grid, 256, 0, stream>>>(
           a.v.v, a.partial, a.inverse, a.midpoint, a.v.length, a.v.head_dim, a.v.heads, threads,
           a.v.stride_b, a.v.stride_h, a.v.stride_n, a.v.permutation);
-      value_center_from_partials_kernel<<<(rows + 63) / 64, 64, 0, stream>>>(
+      value_center_from_partials_kernel<<<rows, threads, 0, stream>>>(
           a.partial, a.inverse, a.midpoint, a.v.center, rows, threads, a.v.length);
     }
   } else {

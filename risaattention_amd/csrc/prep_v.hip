@@ -60,12 +60,12 @@ template <int DT> int run(const ValueArgs& a, hipStream_t stream) {
           a.stride_n, a.permutation);
     } else {
       const int threads = summation_threads(a.length);
-      const int per_block = 256 / (a.head_dim / 8);
+      const int per_block = 256 / (a.head_dim / 4);
       dim3 residual_grid(threads / per_block, bh);
       value_residual_kernel<DT><<<residual_grid, 256, 0, stream>>>(
           a.v, w.partial, w.inverse, w.midpoint, a.length, a.head_dim, a.heads, threads, a.stride_b,
           a.stride_h, a.stride_n, a.permutation);
-      value_center_from_partials_kernel<<<(rows + 63) / 64, 64, 0, stream>>>(
+      value_center_from_partials_kernel<<<rows, threads, 0, stream>>>(
           w.partial, w.inverse, w.midpoint, a.center, rows, threads, a.length);
     }
   }

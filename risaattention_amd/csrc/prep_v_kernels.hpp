@@ -21,6 +21,8 @@
 
 #pragma once
 
+#include <type_traits>
+
 #include "common.hpp"
 #include "launchers.hpp"
 
@@ -310,7 +312,8 @@ __global__ __launch_bounds__(256) void value_codes_kernel(const void* __restrict
                                        blockIdx.x, blockIdx.y, blockIdx.z);
 }
 
-// grid (T / (256/octets), B*H), 256 threads: thread = (summation thread t, octet).
+// grid (T / (256/quads), B*H), 256 threads: thread = (summation thread t, four channels);
+// four rather than eight channels per thread so that a long sequence fills every SIMD.
 template <int DT>
 __global__ __launch_bounds__(256) void value_residual_kernel(const void* __restrict__ v,
                                                              float* __restrict__ partial,
@@ -322,56 +325,86 @@ __global__ __launch_bounds__(256) void value_residual_kernel(const void* __restr
                                                              const int32_t* __restrict__ permutation) {
   const int bh = blockIdx.y;
   const int b = bh / heads, h = bh - b * heads;
-  const int octets = dim / 8;
-  const int octet = threadIdx.x % octets;
-  const int t = blockIdx.x * (256 / octets) + threadIdx.x / octets;
+  const int quads = dim / 4;
+  const int quad = threadIdx.x % quads;
+  const int t = blockIdx.x * (256 / quads) + threadIdx.x / quads;
   const int64_t base = static_cast<int64_t>(b) * stride_b + static_cast<int64_t>(h) * stride_h;
-  const int64_t row0 = static_cast<int64_t>(bh) * dim + octet * 8;
-  float inv[8], mid[8], residual[8];
+  const int64_t row0 = static_cast<int64_t>(bh) * dim + quad * 4;
+  float inv[4], mid[4], residual[4];
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {
+  for (int i = 0; i < 4; ++i) {
     inv[i] = inverse[row0 + i];
     mid[i] = midpoint[row0 + i];
     residual[i] = 0.0f;
   }
-  for (int src = length - 1 - t; src >= 0; src -= threads) {
-    const int from = permutation != nullptr ? permutation[static_cast<int64_t>(bh) * length + src] : src;
-    float x[8];
-    load8<DT>(v, base + static_cast<int64_t>(from) * stride_n + octet * 8, x);
+  // The additions of one thread are sequential by contract; the loads are not: eight tokens
+  // are requested before the first is consumed, which is what hides the memory latency with
+  // only 512 summation threads per (batch, head).
+  // Loads past the front of the sequence are clamped to token 0 and not accumulated, so
+  // that no load sits inside a branch (the compiler would wait for each of those in turn).
+  constexpr int kInFlight = 8;
+  auto accumulate = [&](auto permuted_tag) {
+    constexpr bool PERMUTED = decltype(permuted_tag)::value;
+    const int32_t* order = PERMUTED ? permutation + static_cast<int64_t>(bh) * length : nullptr;
+    for (int src0 = length - 1 - t; src0 >= 0; src0 -= threads * kInFlight) {
+      int from[kInFlight];
+      float x[kInFlight][4];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const float normalized = (x[i] - mid[i]) * inv[i];
-      const float code = static_cast<float>(quantize_s8(normalized));
-      residual[i] += normalized - code;
+      for (int j = 0; j < kInFlight; ++j) {
+        const int src = max(src0 - j * threads, 0);
+        if constexpr (PERMUTED) {
+          from[j] = order[src];
+        } else {
+          from[j] = src;
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < kInFlight; ++j)
+        load4<DT>(v, base + static_cast<int64_t>(from[j]) * stride_n + quad * 4, x[j]);
+#pragma unroll
+      for (int j = 0; j < kInFlight; ++j) {
+        if (src0 - j * threads >= 0) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const float normalized = (x[j][i] - mid[i]) * inv[i];
+            const float code = static_cast<float>(quantize_s8(normalized));
+            residual[i] += normalized - code;
+          }
+        }
+      }
     }
+  };
+  if (permutation != nullptr) {
+    accumulate(std::true_type{});
+  } else {
+    accumulate(std::false_type{});
   }
 #pragma unroll
-  for (int i = 0; i < 8; ++i) partial[(row0 + i) * threads + t] = residual[i];
+  for (int i = 0; i < 4; ++i) partial[(row0 + i) * threads + t] = residual[i];
 }
 
-__global__ void value_center_from_partials_kernel(const float* __restrict__ partial,
-                                    const float* __restrict__ inverse,
-                                    const float* __restrict__ midpoint, float* __restrict__ center,
-                                    int rows, int threads, int length) {
-  const int row = blockIdx.x * blockDim.x + threadIdx.x;
-  if (row >= rows) return;
-  const float* p = partial + static_cast<int64_t>(row) * threads;
-  float total = 0.0f;
-  for (int w = 0; w < threads / 32; ++w) {
-    float t[32];
+// One workgroup of `threads` threads per row: every 32 partials combine with the reference's
+// tree (t[i] += t[i+16], +8, +4, +2, +1: a shuffle-down) and the totals of the 32-thread
+// groups are added in group order.
+__global__ __launch_bounds__(512) void value_center_from_partials_kernel(
+    const float* __restrict__ partial, const float* __restrict__ inverse,
+    const float* __restrict__ midpoint, float* __restrict__ center, int rows, int threads, int length) {
+  __shared__ float group_total[16];
+  const int row = blockIdx.x;
+  const int t = threadIdx.x;
+  float value = partial[static_cast<int64_t>(row) * threads + t];
 #pragma unroll
-    for (int i = 0; i < 32; ++i) t[i] = p[w * 32 + i];
-#pragma unroll
-    for (int offset = 16; offset > 0; offset >>= 1) {
-#pragma unroll
-      for (int i = 0; i < offset; ++i) t[i] = t[i] + t[i + offset];
-    }
-    total += t[0];
+  for (int offset = 16; offset > 0; offset >>= 1) value += __shfl_down(value, offset, 32);
+  if ((t & 31) == 0) group_total[t >> 5] = value;
+  __syncthreads();
+  if (t == 0) {
+    float total = 0.0f;
+    for (int w = 0; w < threads / 32; ++w) total += group_total[w];
+    const float scale = 1.0f / inverse[row];
+    const float mean = total / static_cast<float>(length);
+    const float correction = scale * mean;
+    center[row] = midpoint[row] + correction;
   }
-  const float scale = 1.0f / inverse[row];
-  const float mean = total / static_cast<float>(length);
-  const float correction = scale * mean;
-  center[row] = midpoint[row] + correction;
 }
 
 // One-launch form of the two kernels above for short sequences (a workgroup reads 16
@@ -403,16 +436,47 @@ __global__ __launch_bounds__(512) void value_center_fused_kernel(const void* __r
     mid[i] = midpoint[row0 + i];
     residual[i] = 0.0f;
   }
-  for (int src = length - 1 - t; src >= 0; src -= threads) {
-    const int from = permutation != nullptr ? permutation[static_cast<int64_t>(bh) * length + src] : src;
-    float x[8];
-    load8<DT>(v, base + static_cast<int64_t>(from) * stride_n + octet * 8, x);
+  // The additions of one thread are sequential by contract; the loads are not: eight tokens
+  // are requested before the first is consumed, which is what hides the memory latency with
+  // only 512 summation threads per (batch, head).
+  // Loads past the front of the sequence are clamped to token 0 and not accumulated, so
+  // that no load sits inside a branch (the compiler would wait for each of those in turn).
+  constexpr int kInFlight = 8;
+  auto accumulate = [&](auto permuted_tag) {
+    constexpr bool PERMUTED = decltype(permuted_tag)::value;
+    const int32_t* order = PERMUTED ? permutation + static_cast<int64_t>(bh) * length : nullptr;
+    for (int src0 = length - 1 - t; src0 >= 0; src0 -= threads * kInFlight) {
+      int from[kInFlight];
+      float x[kInFlight][8];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const float normalized = (x[i] - mid[i]) * inv[i];
-      const float code = static_cast<float>(quantize_s8(normalized));
-      residual[i] += normalized - code;
+      for (int j = 0; j < kInFlight; ++j) {
+        const int src = max(src0 - j * threads, 0);
+        if constexpr (PERMUTED) {
+          from[j] = order[src];
+        } else {
+          from[j] = src;
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < kInFlight; ++j)
+        load8<DT>(v, base + static_cast<int64_t>(from[j]) * stride_n + octet * 8, x[j]);
+#pragma unroll
+      for (int j = 0; j < kInFlight; ++j) {
+        if (src0 - j * threads >= 0) {
+#pragma unroll
+          for (int i = 0; i < 8; ++i) {
+            const float normalized = (x[j][i] - mid[i]) * inv[i];
+            const float code = static_cast<float>(quantize_s8(normalized));
+            residual[i] += normalized - code;
+          }
+        }
+      }
     }
+  };
+  if (permutation != nullptr) {
+    accumulate(std::true_type{});
+  } else {
+    accumulate(std::false_type{});
   }
 #pragma unroll
   for (int i = 0; i < 8; ++i) {

@@ -21,6 +21,10 @@ CASES = [
     (torch.bfloat16, 80, 100, 300, 2, 2, "absmax", 0.0),  # padded head dim
     (torch.float16, 128, 19, 257, 2, 1, "absmax", 4.0),  # anchor fires
     (torch.bfloat16, 128, 300, 2049, 4, 1, "midpoint_affine", 0.0),
+    # beyond 4096 keys the residual-corrected centre comes from the two-kernel path
+    (torch.bfloat16, 128, 40, 4611, 2, 2, "midpoint_affine", 0.0),
+    (torch.float16, 64, 40, 9000, 2, 1, "midpoint_affine", 0.0),
+    (torch.float32, 256, 40, 4200, 1, 1, "midpoint_affine", 0.0),
 ]
 
 
