@@ -159,49 +159,65 @@ __device__ __forceinline__ void quantize_group(const void* in, int64_t in_base, 
   const int j = sub & 15, row = sub >> 4;
   auto channel_of = [&](int block, int g) { return block * 128 + (GROUPS * j + g) * 4; };
 
-  auto load_row = [&](int64_t row_base, float (&dst)[BLOCKS][GROUPS][4]) {
-#pragma unroll
-    for (int block = 0; block < BLOCKS; ++block) {
-      if (GROUPS == 2 && DT != kF32 && wide) {
-        float eight[8];
-        load8<DT>(in, row_base + channel_of(block, 0), eight);
-#pragma unroll
-        for (int c = 0; c < 8; ++c) dst[block][c / 4][c % 4] = eight[c];
-      } else {
-#pragma unroll
-        for (int g = 0; g < GROUPS; ++g) load4<DT>(in, row_base + channel_of(block, g), dst[block][g]);
-      }
-    }
-  };
-
+  // Every load of the group is issued before any is consumed, and none sits inside a
+  // branch (the compiler waits for each load of a conditional block before leaving it):
+  // tokens past the end read the last row and are zeroed afterwards, the gather indices are
+  // fetched as one batch, the row that stands in for a missing anchor row is ignored, and the
+  // uniform choices (row width, permutation) are made once around the whole batch.
   float bias[BLOCKS][GROUPS][4];
-  if (bias_row != nullptr) load_row(in_base + *static_cast<const int64_t*>(bias_row), bias);
-
   float v[STEPS][BLOCKS][GROUPS][4];
+  int from[STEPS];
+  bool valid[STEPS];
 #pragma unroll
   for (int i = 0; i < STEPS; ++i) {
     const int n = token_of(PER_STEP * i + row);
-    if (n < length) {
-      // with a permutation, token n of the gathered sequence is source row source[n]
-      const int from = source != nullptr ? source[n] : n;
-      load_row(in_base + static_cast<int64_t>(from) * stride_n, v[i]);
-      if (bias_row != nullptr) {
-#pragma unroll
-        for (int block = 0; block < BLOCKS; ++block)
-#pragma unroll
-          for (int g = 0; g < GROUPS; ++g)
-#pragma unroll
-            for (int c = 0; c < 4; ++c) v[i][block][g][c] -= bias[block][g][c];
-      }
-    } else {
-#pragma unroll
-      for (int block = 0; block < BLOCKS; ++block)
-#pragma unroll
-        for (int g = 0; g < GROUPS; ++g)
-#pragma unroll
-          for (int c = 0; c < 4; ++c) v[i][block][g][c] = 0.0f;
-    }
+    valid[i] = n < length;
+    from[i] = min(n, length - 1);
   }
+  if (source != nullptr) {
+    // with a permutation, token n of the gathered sequence is source row source[n]
+#pragma unroll
+    for (int i = 0; i < STEPS; ++i) from[i] = source[from[i]];
+  }
+  const bool has_bias = bias_row != nullptr;
+  const int64_t bias_base =
+      in_base + (has_bias ? *static_cast<const int64_t*>(bias_row) : static_cast<int64_t>(from[0]) * stride_n);
+  auto load_all = [&](auto wide_tag) {
+    constexpr bool EIGHT = GROUPS == 2 && DT != kF32 && decltype(wide_tag)::value;
+    auto load_row = [&](int64_t row_base, float (&dst)[BLOCKS][GROUPS][4]) {
+#pragma unroll
+      for (int block = 0; block < BLOCKS; ++block) {
+        if constexpr (EIGHT) {
+          float eight[8];
+          load8<DT>(in, row_base + channel_of(block, 0), eight);
+#pragma unroll
+          for (int c = 0; c < 8; ++c) dst[block][c / 4][c % 4] = eight[c];
+        } else {
+#pragma unroll
+          for (int g = 0; g < GROUPS; ++g) load4<DT>(in, row_base + channel_of(block, g), dst[block][g]);
+        }
+      }
+    };
+    load_row(bias_base, bias);
+#pragma unroll
+    for (int i = 0; i < STEPS; ++i) load_row(in_base + static_cast<int64_t>(from[i]) * stride_n, v[i]);
+  };
+  if (wide) {
+    load_all(std::true_type{});
+  } else {
+    load_all(std::false_type{});
+  }
+#pragma unroll
+  for (int i = 0; i < STEPS; ++i)
+#pragma unroll
+    for (int block = 0; block < BLOCKS; ++block)
+#pragma unroll
+      for (int g = 0; g < GROUPS; ++g)
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+          const float shifted = has_bias ? v[i][block][g][c] - bias[block][g][c] : v[i][block][g][c];
+          v[i][block][g][c] = valid[i] ? shifted : 0.0f;
+        }
   float mx = 0.0f;
 #pragma unroll
   for (int i = 0; i < STEPS; ++i)
