@@ -81,18 +81,19 @@ __device__ __forceinline__ void value_range_block(const void* __restrict__ v, fl
   const int first = chunk * per_wave;
 #pragma unroll 8
   for (int t = row; t < per_wave; t += rows_per_load) {
-    const int n = first + t;
-    if (n < length) {
-      float x[8];
-      load8<DT>(v, base + static_cast<int64_t>(n) * stride_n + octet * 8, x);
+    // Past the end the last token is read again (a repeated element changes neither a
+    // minimum nor a maximum), which keeps the loads out of branches and lets the unrolled
+    // loop keep eight of them in flight.
+    const int n = min(first + t, length - 1);
+    float x[8];
+    load8<DT>(v, base + static_cast<int64_t>(n) * stride_n + octet * 8, x);
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        if constexpr (AFFINE) {
-          mx[i] = __builtin_fmaxf(mx[i], x[i]);
-          mn[i] = __builtin_fminf(mn[i], x[i]);
-        } else {
-          mx[i] = __builtin_fmaxf(mx[i], __builtin_fabsf(x[i]));
-        }
+    for (int i = 0; i < 8; ++i) {
+      if constexpr (AFFINE) {
+        mx[i] = __builtin_fmaxf(mx[i], x[i]);
+        mn[i] = __builtin_fminf(mn[i], x[i]);
+      } else {
+        mx[i] = __builtin_fmaxf(mx[i], __builtin_fabsf(x[i]));
       }
     }
   }
@@ -264,21 +265,23 @@ __device__ __forceinline__ void value_codes_block(const void* __restrict__ v, in
         }
       }
     }
+    // The four token loads are issued together, outside any branch; tokens past the end
+    // read the last row and their codes are zeroed.
     int q[8][4];
+    int from[4];
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      const int n = n0 + r;
-      if (n < length) {
-        const int from = permutation != nullptr ? permutation[static_cast<int64_t>(bh) * length + n] : n;
-        float x[8];
-        load8<DT>(v, base + static_cast<int64_t>(from) * stride_n + octet * 8, x);
+    for (int r = 0; r < 4; ++r) from[r] = min(n0 + r, length - 1);
+    if (permutation != nullptr) {
 #pragma unroll
-        for (int i = 0; i < 8; ++i) q[i][r] = quantize_s8((x[i] - mid[i]) * inv[i]);
-      } else {
-#pragma unroll
-        for (int i = 0; i < 8; ++i) q[i][r] = 0;
-      }
+      for (int r = 0; r < 4; ++r) from[r] = permutation[static_cast<int64_t>(bh) * length + from[r]];
     }
+    float x[4][8];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) load8<DT>(v, base + static_cast<int64_t>(from[r]) * stride_n + octet * 8, x[r]);
+#pragma unroll
+    for (int r = 0; r < 4; ++r)
+#pragma unroll
+      for (int i = 0; i < 8; ++i) q[i][r] = n0 + r < length ? quantize_s8((x[r][i] - mid[i]) * inv[i]) : 0;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       if (p0 < padded) {
