@@ -99,10 +99,21 @@ def draw_sparse_case(seed):
         "mask": ["none", "none", "causal", "key_bool", "key_float"][int(rng.integers(5))],
         "theta": float(rng.choice([0.5, 0.9, 0.99, 1.0])),
     }
+    # Key-only masks over more than 1024 keys and at least 256 queries also carry a list of
+    # unmasked key tiles; the pattern's lists take its place during reuse.
+    case.update(KEY_MASK_LIST_CASES.get(seed, {}))
     return case
 
 
-@pytest.mark.parametrize("seed", range(32))
+KEY_MASK_LIST_CASES = {
+    5032: {"q_len": 300, "k_len": 1300, "dim": 128, "mask": "key_bool", "theta": 0.9},
+    5033: {"q_len": 515, "k_len": 2050, "dim": 64, "mask": "key_float", "theta": 0.5},
+    5034: {"q_len": 256, "k_len": 1025, "dim": 256, "mask": "key_bool", "theta": 0.99},
+    5035: {"q_len": 300, "k_len": 2050, "dim": 80, "mask": "key_float", "theta": 1.0},
+}
+
+
+@pytest.mark.parametrize("seed", range(36))
 def test_random_sparse_shape_matches_oracle(risa, seed):
     """Construction on ragged shapes, then reuse of the constructed tile lists: the dense
     output, the CSR structure and the sparse output (both reuse entry points) against the
