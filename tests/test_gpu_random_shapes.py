@@ -82,6 +82,17 @@ def test_random_shape_matches_oracle(risa, seed):
     assert np.array_equal(np.isfinite(to_numpy(lse)), finite), case
     if finite.any():
         assert relative_l2(to_numpy(lse)[finite], expected_lse[finite]) < TOLERANCE, case
+    if case["mask"] == "none":
+        # Unmasked launches with more workgroups than compute units run the other kernel
+        # (32 queries per wavefront): repeat every query head until the launch is that large;
+        # copy r of head h still reads KV head h // group.
+        blocks = case["batch"] * case["q_heads"] * -(-case["q_len"] // 128)
+        repeat = torch.cuda.get_device_properties(0).multi_processor_count // blocks + 1
+        wide, wide_lse = risa.int8_attention(q.repeat_interleave(repeat, dim=1), k, v,
+                                             v_quantization=case["mode"], return_lse=True)
+        assert relative_l2(to_numpy(wide[:, ::repeat]), expected) < TOLERANCE, case
+        assert relative_l2(to_numpy(wide[:, repeat - 1::repeat]), expected) < TOLERANCE, case
+        assert relative_l2(to_numpy(wide_lse[:, ::repeat]), expected_lse) < TOLERANCE, case
 
 
 def draw_sparse_case(seed):
