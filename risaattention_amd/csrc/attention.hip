@@ -169,9 +169,12 @@ int launch_attention(const AttentionArgs& a, hipStream_t stream) {
   const bool fast = a.mask == nullptr && !a.is_causal && a.sm_scale > 0.0f;
 
   // A launch that cannot give every compute unit more than one workgroup runs the
-  // raw-score path with sixteen queries per wavefront (two wavefronts per SIMD).
+  // raw-score path with sixteen queries per wavefront (two wavefronts per SIMD).  So does
+  // every launch with head dim 256: thirty-two queries of 256 channels per wavefront need
+  // some 380 registers, which leaves one wavefront per SIMD (1200 against 1630
+  // dense-equivalent TOPS at N=16K).
   const int64_t workgroups = static_cast<int64_t>(p.n_qb) * a.q_heads * a.batch;
-  const bool narrow = fast && !indexed && !capture && workgroups <= narrow_attention_limit();
+  const bool narrow = fast && !indexed && !capture && (a.head_dim > 128 || workgroups <= narrow_attention_limit());
 
   int status;
   if (narrow)
