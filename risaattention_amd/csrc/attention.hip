@@ -174,7 +174,8 @@ int launch_attention(const AttentionArgs& a, hipStream_t stream) {
   // some 380 registers, which leaves one wavefront per SIMD (1200 against 1630
   // dense-equivalent TOPS at N=16K).
   const int64_t workgroups = static_cast<int64_t>(p.n_qb) * a.q_heads * a.batch;
-  const bool narrow = fast && !indexed && !capture && (a.head_dim > 128 || workgroups <= narrow_attention_limit());
+  const bool narrow = fast && p.index_mode != 2 && !capture &&
+                      (a.head_dim > 128 || workgroups <= narrow_attention_limit());
 
   int status;
   if (narrow)

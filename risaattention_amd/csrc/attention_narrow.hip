@@ -8,10 +8,11 @@ int narrow_attention_limit();
 
 namespace {
 
-template <int D, int CTA_K, int WAVES, int KSPLIT> int launch_block(const KernelParams& p, hipStream_t stream) {
+template <int D, int CTA_K, int WAVES, int KSPLIT, bool INDEXED = false>
+int launch_block(const KernelParams& p, hipStream_t stream) {
   using Shape = TileShape<D, CTA_K>;
   constexpr int kLdsBytes = Shape::kLdsBytes * KSPLIT;
-  auto kernel = attention_narrow_kernel<D, CTA_K, WAVES, KSPLIT>;
+  auto kernel = attention_narrow_kernel<D, CTA_K, WAVES, KSPLIT, INDEXED>;
   static thread_local int configured_device = -1;
   int device = -1;
   if (hipGetDevice(&device) != hipSuccess) return fail("risa_attention: hipGetDevice failed");
@@ -39,6 +40,12 @@ template <int D, int CTA_K> int launch_narrow(const KernelParams& p, hipStream_t
   // two sets of stages must fit the 160 KB of LDS of a compute unit
   constexpr bool kSplitFits = 2 * TileShape<D, CTA_K>::kLdsBytes <= 160 * 1024;
   const bool split = kSplitFits && p.n_kb >= 4 && p.n_kb % 2 == 0;
+  if (p.index_mode == 1) {
+    // sparse reuse: the tile lists stay whole
+    if (workgroups * 4 <= compute_units) return launch_block<D, CTA_K, 2, 1, true>(p, stream);
+    if (workgroups * 2 <= compute_units) return launch_block<D, CTA_K, 4, 1, true>(p, stream);
+    return launch_block<D, CTA_K, 8, 1, true>(p, stream);
+  }
   if (workgroups * 4 <= compute_units) {
     if constexpr (kSplitFits) {
       if (split) return launch_block<D, CTA_K, 2, 2>(p, stream);

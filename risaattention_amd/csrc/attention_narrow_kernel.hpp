@@ -45,10 +45,14 @@ template <int ROWBYTES> __device__ __forceinline__ int narrow_key_swizzle(int ro
 // the first part merges the two partial results through LDS at the end, which halves
 // the chain of dependent tiles of a short sequence.  The merge is the online-softmax
 // update applied once more, so only the FP32 rounding order differs.
-template <int D, int CTA_K, int WAVES, int KSPLIT = 1>
+// INDEXED walks the key tiles listed for the 128-query block of the workgroup's queries
+// (the CSR pattern of the sparse path) instead of all of them; the last listed tile takes
+// the last-tile formulas, as in the wide kernel.
+template <int D, int CTA_K, int WAVES, int KSPLIT = 1, bool INDEXED = false>
 __global__ __launch_bounds__(64 * WAVES * KSPLIT) void attention_narrow_kernel(const KernelParams p) {
   static_assert(WAVES == 8 || WAVES == 4 || WAVES == 2, "seeds and scales are copied by two different wavefronts");
   static_assert(KSPLIT == 1 || (KSPLIT == 2 && WAVES <= 4), "at most eight wavefronts per workgroup");
+  static_assert(!INDEXED || KSPLIT == 1, "tile lists are not split");
   constexpr int QUERIES = 16 * WAVES;
   using Shape = TileShape<D, CTA_K>;
   constexpr int KB = CTA_K / 16;  // 16-key blocks per tile
@@ -83,8 +87,19 @@ __global__ __launch_bounds__(64 * WAVES * KSPLIT) void attention_narrow_kernel(c
 
   const int query = bx * QUERIES + wave * 16 + ql;
   const bool query_ok = query < p.q_len;
-  const int n_it = p.n_kb / KSPLIT;  // the launcher splits even tile counts only
+  int n_it = p.n_kb / KSPLIT;  // the launcher splits even tile counts only
   const int first_tile = part * n_it;
+  [[maybe_unused]] const int32_t* indices = nullptr;
+  if constexpr (INDEXED) {
+    const int64_t row = bhq * p.n_qb + (bx * QUERIES) / kQueryBlock;
+    const int start = p.row_offsets[row];
+    n_it = __builtin_amdgcn_readfirstlane(p.row_offsets[row + 1] - start);
+    indices = p.tile_indices + start;
+  }
+  auto tile_at = [&](int step) -> int {
+    if constexpr (INDEXED) return __builtin_amdgcn_readfirstlane(indices[step]);
+    return first_tile + step;
+  };
 
   // --- copies HBM/L2 -> LDS ---------------------------------------------------------
   // Copy instruction (wave*NC + i) fills LDS bytes [(wave*NC + i)*1024, +1024) of a
@@ -342,15 +357,16 @@ __global__ __launch_bounds__(64 * WAVES * KSPLIT) void attention_narrow_kernel(c
     v4i acc_first[GROUP];
     v4i v_first[GROUP][SB];
     float ks0, ks1;
-    issue_tile(first_tile, 0);
+    int tile = tile_at(0);
+    issue_tile(tile, 0);
     for (int step = 0; step < n_it - 1; ++step) {
       const int stage = step & 1;
-      const int tile = first_tile + step;
+      const int next_tile = tile_at(step + 1);
       __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
       __syncthreads();
       load_k_fragments(lds + stage * Shape::kStageBytes, 0, k_first);
       tile_scales(stage, ks0, ks1);
-      issue_tile(tile + 1, stage ^ 1);
+      issue_tile(next_tile, stage ^ 1);
       __builtin_amdgcn_s_setprio(0);  // vector phases before matrix phases, as in the wide kernel
       score_tile(stage, k_first, s);
       load_group(stage, 0, acc_first, v_first);
@@ -360,9 +376,9 @@ __global__ __launch_bounds__(64 * WAVES * KSPLIT) void attention_narrow_kernel(c
       __builtin_amdgcn_s_setprio(1);
       __builtin_amdgcn_sched_barrier(0);
       value_tile(stage, pk, acc_first, v_first, t_scale);
+      tile = next_tile;
     }
     const int stage = (n_it - 1) & 1;
-    const int tile = first_tile + n_it - 1;
     __builtin_amdgcn_s_waitcnt(0x0f70);
     __syncthreads();
     load_k_fragments(lds + stage * Shape::kStageBytes, 0, k_first);

@@ -320,3 +320,38 @@ def test_prequantized_mask_mutation_during_graph_replay(risa, mode):
         graph.replay()
         torch.cuda.synchronize()
         assert torch.equal(captured, eager)
+
+
+@pytest.mark.parametrize("dim,k_len", [(128, 1300), (64, 700), (256, 1300)])
+def test_reuse_matches_oracle_at_every_launch_size(risa, dim, k_len):
+    """Unmasked reuse runs sixteen queries per wavefront in workgroups of 32, 64 or 128
+    queries when the launch is small (and always for head dim 256), thirty-two per wavefront
+    otherwise: 16, 48, 96 and 160 query heads over two query blocks go through each of them.
+    The first eight heads are checked against the oracle walking the same lists, and every
+    launch against the largest one on the heads they share."""
+    q_len, oracle_heads = 200, 8
+    q_all = seeded((1, 160, q_len, dim), torch.bfloat16, 301, scale=2.0)
+    k = seeded((1, 1, k_len, dim), torch.bfloat16, 302, scale=2.0)
+    v = seeded((1, 1, k_len, dim), torch.bfloat16, 303, offset=0.25)
+    _, pattern_all = risa.construct_sparse_int8_attention(q_all, k, v, theta=0.9)
+    assert 0.0 < pattern_all.coverage < 1.0
+    query_blocks = -(-q_len // 128)
+    offsets_all = pattern_all.row_offsets.cpu().numpy()
+    indices_all = pattern_all.block_indices.cpu().numpy()
+
+    def pattern_for(heads):
+        rows = heads * query_blocks
+        return replace(pattern_all, q_heads=heads,
+                       row_offsets=torch.from_numpy(offsets_all[:rows + 1].copy()).cuda(),
+                       block_indices=torch.from_numpy(indices_all[:offsets_all[rows]].copy()).cuda())
+
+    largest = risa.sparse_int8_attention(q_all, k, v, pattern_for(160))
+    prepared = oracle_prequantize(q_all[:, :oracle_heads], k, v)
+    rows = oracle_heads * query_blocks
+    expected, _, _ = oracle_pipeline.attend(
+        prepared, pattern=(offsets_all[:rows + 1], indices_all[:offsets_all[rows]]))
+    assert relative_l2(to_numpy(largest[:, :oracle_heads]), expected) < 1e-3
+    for heads in (16, 48, 96):
+        out = risa.sparse_int8_attention(q_all[:, :heads], k, v, pattern_for(heads))
+        assert relative_l2(to_numpy(out[:, :oracle_heads]), expected) < 1e-3, heads
+        assert relative_l2(to_numpy(out), to_numpy(largest[:, :heads])) < 1e-4, heads
