@@ -277,9 +277,9 @@ __device__ __forceinline__ void quantize_q_block(const void* __restrict__ q, int
                                   nullptr, wide != 0, [base](int i) { return base + i * 8; });
 }
 
-// grid (slices, Hq, B), 256 threads.  One slice (8 KB of input) per workgroup is
-// fastest: looping over four slices serialises their loads (59.8 us against 52.6 us
-// at 16 x 32768 tokens), and workgroup launch is not what limits the kernel.
+// grid (slices, Hq, B), 256 threads.  One slice (8 KB of input) per workgroup: two or
+// four slices per workgroup measure the same (52-54 us at 16 x 32768 tokens), workgroup
+// launch is not what limits the kernel.
 template <int DT, int DK, int ROT>
 __global__ __launch_bounds__(256) void quantize_q_kernel(const void* __restrict__ q,
                                                          int8_t* __restrict__ codes,
