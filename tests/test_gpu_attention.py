@@ -339,3 +339,43 @@ def test_small_launches_match_oracle(risa, heads, dim, k_len):
     expected, expected_lse, _ = oracle_pipeline.attend(prepared, return_lse=True)
     assert relative_l2(to_numpy(out[:, keep]), expected) < TOLERANCE
     assert relative_l2(to_numpy(lse[:, keep]), expected_lse) < TOLERANCE
+
+
+def test_concurrent_host_threads_on_their_own_streams(risa):
+    """The C ABI keeps no shared mutable state (per-thread error text and device caches):
+    two host threads, each on its own stream and with its own shapes, get the bits a
+    single thread gets.  ctypes releases the interpreter lock during the native calls."""
+    import threading
+
+    problems = []
+    for index, (heads, q_len, k_len, dim) in enumerate([(4, 300, 1300, 128), (6, 129, 700, 64)]):
+        q = seeded((1, heads, q_len, dim), torch.bfloat16, 400 + 3 * index)
+        k = seeded((1, 2, k_len, dim), torch.bfloat16, 401 + 3 * index)
+        v = seeded((1, 2, k_len, dim), torch.bfloat16, 402 + 3 * index, offset=0.5)
+        causal = bool(index)
+        expected = risa.int8_attention(q, k, v, is_causal=causal, v_quantization="midpoint_affine")
+        problems.append((q, k, v, causal, expected))
+    torch.cuda.synchronize()
+    failures = []
+
+    def worker(problem):
+        q, k, v, causal, expected = problem
+        try:
+            stream = torch.cuda.Stream()
+            with torch.cuda.stream(stream):
+                for _ in range(25):
+                    out = risa.int8_attention(q, k, v, is_causal=causal, v_quantization="midpoint_affine")
+                    if not torch.equal(out, expected):
+                        failures.append("outputs differ")
+                        break
+            stream.synchronize()
+        except Exception as error:  # noqa: BLE001 - reported by the main thread
+            failures.append(repr(error))
+
+    threads = [threading.Thread(target=worker, args=(problem,)) for problem in problems]
+    for thread in threads:
+        thread.start()
+    for thread in threads:
+        thread.join(timeout=100)
+    assert not any(thread.is_alive() for thread in threads)
+    assert not failures, failures
