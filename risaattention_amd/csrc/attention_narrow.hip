@@ -32,14 +32,14 @@ int launch_block(const KernelParams& p, hipStream_t stream) {
 
 // Queries per workgroup: 128, or 64 / 32 when that still leaves compute units without
 // a workgroup (every SIMD then runs one wavefront with a quarter of the usual work).
-// Those smaller workgroups also split the key tiles over two sets of wavefronts when
-// the tile count is even: the launch is short of work, not of hardware.
+// Those smaller workgroups also split four or more key tiles over two sets of wavefronts:
+// the launch is short of work, not of hardware.
 template <int D, int CTA_K> int launch_narrow(const KernelParams& p, hipStream_t stream) {
   const int64_t workgroups = static_cast<int64_t>(p.n_qb) * p.q_heads * p.batch;
   const int compute_units = narrow_attention_limit();
   // two sets of stages must fit the 160 KB of LDS of a compute unit
   constexpr bool kSplitFits = 2 * TileShape<D, CTA_K>::kLdsBytes <= 160 * 1024;
-  const bool split = kSplitFits && p.n_kb >= 4 && p.n_kb % 2 == 0;
+  const bool split = kSplitFits && p.n_kb >= 4;
   if (p.index_mode == 1) {
     // sparse reuse: the tile lists stay whole
     if (workgroups * 4 <= compute_units) return launch_block<D, CTA_K, 2, 1, true>(p, stream);

@@ -87,8 +87,10 @@ __global__ __launch_bounds__(64 * WAVES * KSPLIT) void attention_narrow_kernel(c
 
   const int query = bx * QUERIES + wave * 16 + ql;
   const bool query_ok = query < p.q_len;
-  int n_it = p.n_kb / KSPLIT;  // the launcher splits even tile counts only
-  const int first_tile = part * n_it;
+  // KSPLIT == 2: the second part takes the last floor(n/2) tiles, the first part the rest.
+  const int second_half = p.n_kb / 2;
+  int n_it = KSPLIT == 1 ? p.n_kb : part == 0 ? p.n_kb - second_half : second_half;
+  const int first_tile = part == 0 ? 0 : p.n_kb - second_half;
   [[maybe_unused]] const int32_t* indices = nullptr;
   if constexpr (INDEXED) {
     const int64_t row = bhq * p.n_qb + (bx * QUERIES) / kQueryBlock;
@@ -393,6 +395,12 @@ __global__ __launch_bounds__(64 * WAVES * KSPLIT) void attention_narrow_kernel(c
     }
     load_group(stage, 0, acc_first, v_first);
     value_tile(stage, pk, acc_first, v_first, t_scale);
+  }
+
+  if constexpr (KSPLIT == 2) {
+    // Both parts share the workgroup's barrier: with an odd tile count the second part has
+    // walked one tile less and takes the barrier of the tile it does not have.
+    if (part == 1 && (p.n_kb & 1)) __syncthreads();
   }
 
   // ---- merge of the two key halves ----------------------------------------------------------

@@ -319,12 +319,13 @@ def test_staged_mask_tiles_match_oracle(risa, mask_dtype, dim, causal):
 
 
 @pytest.mark.parametrize("heads", [4, 80, 200])
-@pytest.mark.parametrize("dim,k_len", [(64, 500), (128, 500), (128, 1400), (256, 444)])
+@pytest.mark.parametrize("dim,k_len", [(64, 500), (128, 500), (128, 1400), (256, 444), (128, 1100), (64, 180)])
 def test_small_launches_match_oracle(risa, heads, dim, k_len):
     """Unmasked launches below one workgroup per compute unit: 4 heads run 32 queries per
-    workgroup and 80 heads 64, both with the key tiles split over two sets of wavefronts
-    (8, 22 and 8 tiles: even counts, ragged last tile); 200 heads run 128 queries per
-    workgroup without the split.  444 keys are 7 tiles: an odd count is not split."""
+    workgroup and 80 heads 64, both with four or more key tiles split over two sets of
+    wavefronts (8, 22 and 8 tiles with a ragged last tile; 7 and 9 tiles: the second set
+    walks one tile less; 3 tiles are not split); 200 heads run 128 queries per workgroup
+    without the split."""
     assert 128 < torch.cuda.get_device_properties(0).multi_processor_count <= 256
     q = seeded((1, heads, 100, dim), torch.bfloat16, 91)
     k = seeded((1, 4, k_len, dim), torch.bfloat16, 92)
