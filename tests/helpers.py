@@ -55,3 +55,19 @@ def seeded(shape, dtype, seed, device="cuda", offset=0.0, scale=1.0):
     generator = torch.Generator(device="cpu").manual_seed(seed)
     values = torch.randn(shape, generator=generator, dtype=torch.float32) * scale + offset
     return values.to(dtype).to(device)
+
+
+def load_vectors():
+    """tests/golden/vectors.npz as {case: {field: array}}; 16-bit words become the float32
+    values of the bfloat16 numbers they hold."""
+    from pathlib import Path
+
+    archive = np.load(Path(__file__).with_name("golden") / "vectors.npz")
+    cases: dict[str, dict[str, np.ndarray]] = {}
+    for key in archive.files:
+        case, field = key.split(".", 1)
+        value = archive[key]
+        if value.dtype == np.uint16:
+            value = (value.astype(np.uint32) << 16).view(np.float32)
+        cases.setdefault(case, {})[field] = value
+    return cases
