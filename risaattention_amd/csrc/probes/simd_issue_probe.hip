@@ -104,6 +104,65 @@ __global__ __launch_bounds__(256) void overlap_kernel(int iterations, float* sin
   if (total == 12345.678f || integer == 0x7fffffff) sink[0] = total + integer;
 }
 
+// The instructions of one wavefront and one 128-key tile of the dense attention kernel at
+// head dim 128 (32 queries), register resident, in the kernel's order: 16 score MFMAs; per
+// score a subtraction, an FMA, an exp2 and a pack, plus the maxima, the row sum and the sign
+// flip; 16 value MFMAs with the 64 output updates (subtract + FMA) between them.  No memory,
+// no barrier, no dependency on the matrix results: the issue-rate floor of the tile loop.
+template <bool MATRIX, bool VECTOR>
+__global__ __launch_bounds__(256) void tile_mix_kernel(int iterations, float* sink) {
+  v4i a = {static_cast<int>(threadIdx.x), 1, 2, 3}, b = {4, 5, 6, static_cast<int>(threadIdx.x)};
+  v16i scores[4] = {}, values[4] = {};
+  float x[16], out[16];
+  int top[4];
+  uint32_t packed[4], sum = 0;
+  for (int i = 0; i < 16; ++i) x[i] = threadIdx.x * 0.001f + i, out[i] = i;
+  for (int i = 0; i < 4; ++i) top[i] = threadIdx.x + i, packed[i] = i;
+  float m = 1.0001f, c = 0.0001f, seed = 12582912.0f;
+  uint32_t flip = 0x80808080u, ones = 0x01010101u;
+  asm volatile("" : "+v"(m), "+v"(c), "+v"(seed), "+v"(flip), "+v"(ones));
+  for (int it = 0; it < iterations; ++it) {
+    if (MATRIX) {
+#pragma unroll
+      for (int j = 0; j < 16; ++j)
+        asm volatile("v_mfma_i32_32x32x32_i8 %0, %1, %2, %0" : "+v"(scores[j % 4]) : "v"(a), "v"(b));
+    }
+    if (VECTOR) {
+#pragma unroll
+      for (int j = 0; j < 32; ++j)
+        asm volatile("v_max3_i32 %0, %0, %1, %2" : "+v"(top[j % 4]) : "v"(packed[j % 4]), "v"(flip));
+#pragma unroll
+      for (int j = 0; j < 64; ++j) {
+        asm volatile("v_sub_f32 %0, %0, %1" : "+v"(x[j % 16]) : "v"(seed));
+        asm volatile("v_fma_f32 %0, %0, %1, %2" : "+v"(x[j % 16]) : "v"(m), "v"(c));
+        asm volatile("v_exp_f32 %0, %0" : "+v"(x[j % 16]));
+        asm volatile("v_cvt_pk_u8_f32 %0, %1, 1, %0" : "+v"(packed[j % 4]) : "v"(x[j % 16]));
+        if (j % 4 == 3) {
+          asm volatile("v_dot4_u32_u8 %0, %1, %2, %0" : "+v"(sum) : "v"(packed[(j / 4) % 4]), "v"(ones));
+          asm volatile("v_xor_b32 %0, %0, %1" : "+v"(packed[(j / 4) % 4]) : "v"(flip));
+        }
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+      if (MATRIX) asm volatile("v_mfma_i32_32x32x32_i8 %0, %1, %2, %0" : "+v"(values[j % 4]) : "v"(a), "v"(b));
+      if (VECTOR) {
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          float t = x[(j * 4 + k) % 16];
+          asm volatile("v_sub_f32 %0, %1, %2" : "=v"(t) : "v"(t), "v"(seed));
+          asm volatile("v_fmac_f32 %0, %1, %2" : "+v"(out[(j * 4 + k) % 16]) : "v"(t), "v"(m));
+        }
+      }
+    }
+  }
+  float total = sum;
+  for (int i = 0; i < 16; ++i) total += x[i] + out[i];
+  int integer = 0;
+  for (int i = 0; i < 4; ++i) integer += scores[i][0] + values[i][15] + top[i] + packed[i];
+  if (total == 12345.678f || integer == 0x7fffffff) sink[0] = total + integer;
+}
+
 // Milliseconds of `iterations` loop iterations with `waves` wavefronts resident per SIMD
 // on every compute unit: the dynamic LDS request limits the workgroups per compute unit.
 template <typename Kernel> float time_kernel(Kernel kernel, int compute_units, int waves, int iterations, float* sink) {
@@ -175,6 +234,17 @@ int main() {
   std::printf("\nmatrix and vector instructions on one SIMD (blocked: one after the other in a wavefront)\n");
   overlap_rows<8, 64, false>("v_mfma_i32_16x16x64_i8", compute_units, sink);
   overlap_rows<8, 128, true>("v_mfma_i32_32x32x32_i8", compute_units, sink);
+  std::printf("\none wavefront x one 128-key tile of the dense attention kernel (head dim 128), register resident\n");
+  for (int waves = 1; waves <= 2; ++waves) {
+    const int iterations = 5000;
+    const double scale = 1e6 / (double(iterations) * waves);
+    const float matrix = time_kernel(tile_mix_kernel<true, false>, compute_units, waves, iterations, sink);
+    const float vector = time_kernel(tile_mix_kernel<false, true>, compute_units, waves, iterations, sink);
+    const float both = time_kernel(tile_mix_kernel<true, true>, compute_units, waves, iterations, sink);
+    std::printf("%d w/SIMD: 32 MFMAs %.0f ns, vector instructions %.0f ns, both %.0f ns per wavefront and tile\n",
+                waves, matrix * scale, vector * scale, both * scale);
+    std::fflush(stdout);
+  }
   CHECK(hipFree(sink));
   return 0;
 }
