@@ -109,7 +109,7 @@ __global__ __launch_bounds__(256) void overlap_kernel(int iterations, float* sin
 // score a subtraction, an FMA, an exp2 and a pack, plus the maxima, the row sum and the sign
 // flip; 16 value MFMAs with the 64 output updates (subtract + FMA) between them.  No memory,
 // no barrier, no dependency on the matrix results: the issue-rate floor of the tile loop.
-template <bool MATRIX, bool VECTOR>
+template <bool MATRIX, bool VECTOR, bool SPREAD = false>
 __global__ __launch_bounds__(256) void tile_mix_kernel(int iterations, float* sink) {
   v4i a = {static_cast<int>(threadIdx.x), 1, 2, 3}, b = {4, 5, 6, static_cast<int>(threadIdx.x)};
   v16i scores[4] = {}, values[4] = {};
@@ -122,7 +122,7 @@ __global__ __launch_bounds__(256) void tile_mix_kernel(int iterations, float* si
   uint32_t flip = 0x80808080u, ones = 0x01010101u;
   asm volatile("" : "+v"(m), "+v"(c), "+v"(seed), "+v"(flip), "+v"(ones));
   for (int it = 0; it < iterations; ++it) {
-    if (MATRIX) {
+    if (MATRIX && !SPREAD) {
 #pragma unroll
       for (int j = 0; j < 16; ++j)
         asm volatile("v_mfma_i32_32x32x32_i8 %0, %1, %2, %0" : "+v"(scores[j % 4]) : "v"(a), "v"(b));
@@ -133,6 +133,8 @@ __global__ __launch_bounds__(256) void tile_mix_kernel(int iterations, float* si
         asm volatile("v_max3_i32 %0, %0, %1, %2" : "+v"(top[j % 4]) : "v"(packed[j % 4]), "v"(flip));
 #pragma unroll
       for (int j = 0; j < 64; ++j) {
+        if (MATRIX && SPREAD && j % 4 == 0)
+          asm volatile("v_mfma_i32_32x32x32_i8 %0, %1, %2, %0" : "+v"(scores[(j / 4) % 4]) : "v"(a), "v"(b));
         asm volatile("v_sub_f32 %0, %0, %1" : "+v"(x[j % 16]) : "v"(seed));
         asm volatile("v_fma_f32 %0, %0, %1, %2" : "+v"(x[j % 16]) : "v"(m), "v"(c));
         asm volatile("v_exp_f32 %0, %0" : "+v"(x[j % 16]));
@@ -153,6 +155,71 @@ __global__ __launch_bounds__(256) void tile_mix_kernel(int iterations, float* si
           asm volatile("v_sub_f32 %0, %1, %2" : "=v"(t) : "v"(t), "v"(seed));
           asm volatile("v_fmac_f32 %0, %1, %2" : "+v"(out[(j * 4 + k) % 16]) : "v"(t), "v"(m));
         }
+      }
+    }
+  }
+  float total = sum;
+  for (int i = 0; i < 16; ++i) total += x[i] + out[i];
+  int integer = 0;
+  for (int i = 0; i < 4; ++i) integer += scores[i][0] + values[i][15] + top[i] + packed[i];
+  if (total == 12345.678f || integer == 0x7fffffff) sink[0] = total + integer;
+}
+
+// The same instructions in a software-pipelined order: the score MFMAs of a tile run under
+// the output updates of the previous tile, and the value MFMAs of each 32-key block under
+// the exp2/pack chain of the next block; only the maxima have no matrix work beside them.
+template <bool UPDATES_UNDER_SCORES>
+__global__ __launch_bounds__(256) void tile_pipeline_kernel(int iterations, float* sink) {
+  v4i a = {static_cast<int>(threadIdx.x), 1, 2, 3}, b = {4, 5, 6, static_cast<int>(threadIdx.x)};
+  v16i scores[4] = {}, values[4] = {};
+  float x[16], out[16];
+  int top[4];
+  uint32_t packed[4], sum = 0;
+  for (int i = 0; i < 16; ++i) x[i] = threadIdx.x * 0.001f + i, out[i] = i;
+  for (int i = 0; i < 4; ++i) top[i] = threadIdx.x + i, packed[i] = i;
+  float m = 1.0001f, c = 0.0001f, seed = 12582912.0f;
+  uint32_t flip = 0x80808080u, ones = 0x01010101u;
+  asm volatile("" : "+v"(m), "+v"(c), "+v"(seed), "+v"(flip), "+v"(ones));
+  for (int it = 0; it < iterations; ++it) {
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+      asm volatile("v_mfma_i32_32x32x32_i8 %0, %1, %2, %0" : "+v"(scores[j % 4]) : "v"(a), "v"(b));
+      if (UPDATES_UNDER_SCORES) {
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          float t = x[(j * 4 + k) % 16];
+          asm volatile("v_sub_f32 %0, %1, %2" : "=v"(t) : "v"(t), "v"(seed));
+          asm volatile("v_fmac_f32 %0, %1, %2" : "+v"(out[(j * 4 + k) % 16]) : "v"(t), "v"(m));
+        }
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < 32; ++j)
+      asm volatile("v_max3_i32 %0, %0, %1, %2" : "+v"(top[j % 4]) : "v"(packed[j % 4]), "v"(flip));
+#pragma unroll
+    for (int block = 0; block < 5; ++block) {
+#pragma unroll
+      for (int j = 0; j < 16; ++j) {
+        if (block > 0 && j % 4 == 0)
+          asm volatile("v_mfma_i32_32x32x32_i8 %0, %1, %2, %0" : "+v"(values[j / 4]) : "v"(a), "v"(b));
+        if (block < 4) {
+          asm volatile("v_sub_f32 %0, %0, %1" : "+v"(x[j]) : "v"(seed));
+          asm volatile("v_fma_f32 %0, %0, %1, %2" : "+v"(x[j]) : "v"(m), "v"(c));
+          asm volatile("v_exp_f32 %0, %0" : "+v"(x[j]));
+          asm volatile("v_cvt_pk_u8_f32 %0, %1, 1, %0" : "+v"(packed[j % 4]) : "v"(x[j]));
+          if (j % 4 == 3) {
+            asm volatile("v_dot4_u32_u8 %0, %1, %2, %0" : "+v"(sum) : "v"(packed[j / 4]), "v"(ones));
+            asm volatile("v_xor_b32 %0, %0, %1" : "+v"(packed[j / 4]) : "v"(flip));
+          }
+        }
+      }
+    }
+    if (!UPDATES_UNDER_SCORES) {
+#pragma unroll
+      for (int j = 0; j < 64; ++j) {
+        float t = x[j % 16];
+        asm volatile("v_sub_f32 %0, %1, %2" : "=v"(t) : "v"(t), "v"(seed));
+        asm volatile("v_fmac_f32 %0, %1, %2" : "+v"(out[j % 16]) : "v"(t), "v"(m));
       }
     }
   }
@@ -241,8 +308,12 @@ int main() {
     const float matrix = time_kernel(tile_mix_kernel<true, false>, compute_units, waves, iterations, sink);
     const float vector = time_kernel(tile_mix_kernel<false, true>, compute_units, waves, iterations, sink);
     const float both = time_kernel(tile_mix_kernel<true, true>, compute_units, waves, iterations, sink);
-    std::printf("%d w/SIMD: 32 MFMAs %.0f ns, vector instructions %.0f ns, both %.0f ns per wavefront and tile\n",
-                waves, matrix * scale, vector * scale, both * scale);
+    const float spread = time_kernel(tile_mix_kernel<true, true, true>, compute_units, waves, iterations, sink);
+    const float pipelined = time_kernel(tile_pipeline_kernel<true>, compute_units, waves, iterations, sink);
+    const float half_pipelined = time_kernel(tile_pipeline_kernel<false>, compute_units, waves, iterations, sink);
+    std::printf("%d w/SIMD: 32 MFMAs %.0f ns, vector instructions %.0f ns, both %.0f ns per wavefront and tile "
+                "(%.0f ns with the score MFMAs spread through the softmax instructions, %.0f ns software pipelined, %.0f ns with only the value MFMAs pipelined)\n",
+                waves, matrix * scale, vector * scale, both * scale, spread * scale, pipelined * scale, half_pipelined * scale);
     std::fflush(stdout);
   }
   CHECK(hipFree(sink));
