@@ -30,6 +30,7 @@ struct FusedArgs {
   float* partial;
   int q_slices, q_blocks, anchor_blocks, range_groups, chunks;
   int key_tiles, key_blocks, code_blocks_x, kv;
+  int center_blocks;  // midpoint_affine centres computed inside the second launch (0: separate kernels)
   int q_wide, k_wide;
 };
 
@@ -73,6 +74,16 @@ __global__ __launch_bounds__(256) void prepare_stage2_kernel(const FusedArgs a) 
   }
   block -= a.key_blocks;
   const FusedParams fused{a.part_max, a.part_min, a.v.scale, a.v.center, a.inverse, a.midpoint, a.chunks};
+  if constexpr (PARAMS == kParamsAffine) {
+    // the centre blocks come first: each walks the whole sequence of its eight channels
+    if (block < a.center_blocks) {
+      const int octets = a.v.head_dim / 8;
+      value_center_block<DT>(a.v.v, fused, a.v.length, a.v.head_dim, a.v.heads, a.v.stride_b, a.v.stride_h,
+                             a.v.stride_n, a.v.permutation, block % octets, block / octets);
+      return;
+    }
+    block -= a.center_blocks;
+  }
   const int x = block % a.code_blocks_x;
   const int rest = block / a.code_blocks_x;
   value_codes_block<DT, CTA_K, PARAMS>(a.v.v, a.v.codes, a.v.tile_sum, a.inverse, a.midpoint, a.v.length,
@@ -83,8 +94,11 @@ __global__ __launch_bounds__(256) void prepare_stage2_kernel(const FusedArgs a) 
 template <int DT, int DK, int CTA_K, int ROT>
 void launch_stages(const FusedArgs& a, hipStream_t stream) {
   const int stage1_blocks = a.q_blocks + a.anchor_blocks + a.range_groups * a.kv;
-  const int stage2_blocks = a.key_blocks + a.code_blocks_x * a.kv * (a.v.head_dim / 32);
   const bool stored_params = a.chunks > 64;
+  const bool merged_center = a.v.midpoint_affine && !stored_params && a.v.length <= kFusedCenterMaxLength;
+  FusedArgs with_center = a;
+  with_center.center_blocks = merged_center ? a.kv * (a.v.head_dim / 8) : 0;
+  const int stage2_blocks = a.key_blocks + with_center.center_blocks + a.code_blocks_x * a.kv * (a.v.head_dim / 32);
   const int groups = a.kv * a.v.head_dim / 8;
   if (a.v.midpoint_affine) {
     prepare_stage1_kernel<DT, DK, ROT, true><<<stage1_blocks, 256, 0, stream>>>(a);
@@ -93,9 +107,11 @@ void launch_stages(const FusedArgs& a, hipStream_t stream) {
           a.part_max, a.part_min, a.v.scale, a.v.center, a.inverse, a.midpoint, a.v.head_dim, a.chunks, groups);
       prepare_stage2_kernel<DT, DK, CTA_K, ROT, kParamsStored><<<stage2_blocks, 256, 0, stream>>>(a);
     } else {
-      prepare_stage2_kernel<DT, DK, CTA_K, ROT, kParamsAffine><<<stage2_blocks, 256, 0, stream>>>(a);
+      prepare_stage2_kernel<DT, DK, CTA_K, ROT, kParamsAffine><<<stage2_blocks, 256, 0, stream>>>(with_center);
     }
-    if (a.v.length <= kFusedCenterMaxLength) {
+    if (merged_center) {
+      // done inside the second launch
+    } else if (a.v.length <= kFusedCenterMaxLength) {
       dim3 center_grid(a.v.head_dim / 8, a.kv);
       value_center_fused_kernel<DT><<<center_grid, summation_threads(a.v.length), 0, stream>>>(
           a.v.v, a.inverse, a.midpoint, a.v.center, a.v.length, a.v.head_dim, a.v.heads, a.v.stride_b,

@@ -410,6 +410,116 @@ __global__ __launch_bounds__(512) void value_center_from_partials_kernel(
   }
 }
 
+// The centre of value_center_fused_kernel as a block of a 256-thread launch that also
+// holds the code blocks: the parameters come from the partial ranges (the same reduction
+// and arithmetic as value_codes_block, so the same bits), and thread t plays the summation
+// threads t and t + 256 one after the other.  Warp totals land in the reference's order.
+template <int DT>
+__device__ __forceinline__ void value_center_block(const void* __restrict__ v, const FusedParams& fused,
+                                                   int length, int dim, int heads, int64_t stride_b,
+                                                   int64_t stride_h, int64_t stride_n,
+                                                   const int32_t* __restrict__ permutation, int octet,
+                                                   int bh) {
+  __shared__ float warp_total[8][16];
+  __shared__ float parameters[2][8];
+  const int b = bh / heads, h = bh - b * heads;
+  const int t = threadIdx.x, lane = t & 63;
+  const int threads = summation_threads(length);
+  const int64_t base = static_cast<int64_t>(b) * stride_b + static_cast<int64_t>(h) * stride_h;
+  const int64_t row0 = static_cast<int64_t>(bh) * dim + octet * 8;
+  float mx[8], mn[8], inv[8], mid[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    mx[i] = -FLT_MAX;
+    mn[i] = FLT_MAX;
+  }
+  if (lane < fused.chunks) {
+    const int64_t slot = (static_cast<int64_t>(bh) * fused.chunks + lane) * dim + octet * 8;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      mx[i] = fused.part_max[slot + i];
+      mn[i] = fused.part_min[slot + i];
+    }
+  }
+#pragma unroll
+  for (int offset = 32; offset > 0; offset >>= 1) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      mx[i] = __builtin_fmaxf(mx[i], __shfl_xor(mx[i], offset));
+      mn[i] = __builtin_fminf(mn[i], __shfl_xor(mn[i], offset));
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    mid[i] = 0.5f * (mn[i] + mx[i]);
+    const float radius = 0.5f * (mx[i] - mn[i]);
+    const float sc = __builtin_fmaxf(radius * (1.0f / 127.0f), 1e-12f);
+    inv[i] = 1.0f / sc;
+    if (t == i) {
+      parameters[0][i] = inv[i];
+      parameters[1][i] = mid[i];
+    }
+  }
+  constexpr int kInFlight = 8;
+  for (int pass = 0; pass * 256 < threads; ++pass) {
+    const int st = t + pass * 256;  // summation thread
+    float residual[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) residual[i] = 0.0f;
+    auto accumulate = [&](auto permuted_tag) {
+      constexpr bool PERMUTED = decltype(permuted_tag)::value;
+      const int32_t* order = PERMUTED ? permutation + static_cast<int64_t>(bh) * length : nullptr;
+      for (int src0 = st < threads ? length - 1 - st : -1; src0 >= 0; src0 -= threads * kInFlight) {
+        int from[kInFlight];
+        float x[kInFlight][8];
+#pragma unroll
+        for (int j = 0; j < kInFlight; ++j) {
+          const int src = max(src0 - j * threads, 0);
+          if constexpr (PERMUTED) {
+            from[j] = order[src];
+          } else {
+            from[j] = src;
+          }
+        }
+#pragma unroll
+        for (int j = 0; j < kInFlight; ++j)
+          load8<DT>(v, base + static_cast<int64_t>(from[j]) * stride_n + octet * 8, x[j]);
+#pragma unroll
+        for (int j = 0; j < kInFlight; ++j) {
+          if (src0 - j * threads >= 0) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+              const float normalized = (x[j][i] - mid[i]) * inv[i];
+              const float code = static_cast<float>(quantize_s8(normalized));
+              residual[i] += normalized - code;
+            }
+          }
+        }
+      }
+    };
+    if (permutation != nullptr) {
+      accumulate(std::true_type{});
+    } else {
+      accumulate(std::false_type{});
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+#pragma unroll
+      for (int offset = 16; offset > 0; offset >>= 1) residual[i] += __shfl_down(residual[i], offset, 32);
+      if ((t & 31) == 0 && st < threads) warp_total[i][st >> 5] = residual[i];
+    }
+  }
+  __syncthreads();
+  if (t < 8) {
+    float total = 0.0f;
+    for (int w = 0; w < threads / 32; ++w) total += warp_total[t][w];
+    const float scale = 1.0f / parameters[0][t];
+    const float mean = total / static_cast<float>(length);
+    const float correction = scale * mean;
+    fused.center[row0 + t] = parameters[1][t] + correction;
+  }
+}
+
 // One-launch form of the two kernels above for short sequences (a workgroup reads 16
 // bytes of every row, which wastes cache lines once the sequence is long).
 // Residual-corrected centre of the midpoint_affine mode (reference
