@@ -31,6 +31,7 @@ struct FusedArgs {
   int q_slices, q_blocks, anchor_blocks, range_groups, chunks;
   int key_tiles, key_blocks, code_blocks_x, kv;
   int center_blocks;  // midpoint_affine centres computed inside the second launch (0: separate kernels)
+  int residual_blocks_x;  // long midpoint_affine sequences: the residual pass rides in the second launch
   int q_wide, k_wide;
 };
 
@@ -84,6 +85,16 @@ __global__ __launch_bounds__(256) void prepare_stage2_kernel(const FusedArgs a) 
     }
     block -= a.center_blocks;
   }
+  if constexpr (PARAMS == kParamsStored) {
+    const int residual_blocks = a.residual_blocks_x * a.kv;
+    if (block < residual_blocks) {
+      value_residual_block<DT>(a.v.v, a.partial, a.inverse, a.midpoint, a.v.length, a.v.head_dim, a.v.heads,
+                               summation_threads(a.v.length), a.v.stride_b, a.v.stride_h, a.v.stride_n,
+                               a.v.permutation, block % a.residual_blocks_x, block / a.residual_blocks_x);
+      return;
+    }
+    block -= residual_blocks;
+  }
   const int x = block % a.code_blocks_x;
   const int rest = block / a.code_blocks_x;
   value_codes_block<DT, CTA_K, PARAMS>(a.v.v, a.v.codes, a.v.tile_sum, a.inverse, a.midpoint, a.v.length,
@@ -98,14 +109,18 @@ void launch_stages(const FusedArgs& a, hipStream_t stream) {
   const bool merged_center = a.v.midpoint_affine && !stored_params && a.v.length <= kFusedCenterMaxLength;
   FusedArgs with_center = a;
   with_center.center_blocks = merged_center ? a.kv * (a.v.head_dim / 8) : 0;
-  const int stage2_blocks = a.key_blocks + with_center.center_blocks + a.code_blocks_x * a.kv * (a.v.head_dim / 32);
+  const bool merged_residual = a.v.midpoint_affine && stored_params && a.v.length > kFusedCenterMaxLength;
+  with_center.residual_blocks_x =
+      merged_residual ? summation_threads(a.v.length) / (256 / (a.v.head_dim / 4)) : 0;
+  const int stage2_blocks = a.key_blocks + with_center.center_blocks + with_center.residual_blocks_x * a.kv +
+                            a.code_blocks_x * a.kv * (a.v.head_dim / 32);
   const int groups = a.kv * a.v.head_dim / 8;
   if (a.v.midpoint_affine) {
     prepare_stage1_kernel<DT, DK, ROT, true><<<stage1_blocks, 256, 0, stream>>>(a);
     if (stored_params) {
       value_params_kernel<true><<<(groups + 3) / 4, 256, 0, stream>>>(
           a.part_max, a.part_min, a.v.scale, a.v.center, a.inverse, a.midpoint, a.v.head_dim, a.chunks, groups);
-      prepare_stage2_kernel<DT, DK, CTA_K, ROT, kParamsStored><<<stage2_blocks, 256, 0, stream>>>(a);
+      prepare_stage2_kernel<DT, DK, CTA_K, ROT, kParamsStored><<<stage2_blocks, 256, 0, stream>>>(with_center);
     } else {
       prepare_stage2_kernel<DT, DK, CTA_K, ROT, kParamsAffine><<<stage2_blocks, 256, 0, stream>>>(with_center);
     }
@@ -120,10 +135,12 @@ void launch_stages(const FusedArgs& a, hipStream_t stream) {
       const int threads = summation_threads(a.v.length);
       const int per_block = 256 / (a.v.head_dim / 4);
       const int rows = a.kv * a.v.head_dim;
-      dim3 residual_grid(threads / per_block, a.kv);
-      value_residual_kernel<DT><<<residual_grid, 256, 0, stream>>>(
-          a.v.v, a.partial, a.inverse, a.midpoint, a.v.length, a.v.head_dim, a.v.heads, threads,
-          a.v.stride_b, a.v.stride_h, a.v.stride_n, a.v.permutation);
+      if (!merged_residual) {
+        dim3 residual_grid(threads / per_block, a.kv);
+        value_residual_kernel<DT><<<residual_grid, 256, 0, stream>>>(
+            a.v.v, a.partial, a.inverse, a.midpoint, a.v.length, a.v.head_dim, a.v.heads, threads,
+            a.v.stride_b, a.v.stride_h, a.v.stride_n, a.v.permutation);
+      }
       value_center_from_partials_kernel<<<rows, threads, 0, stream>>>(
           a.partial, a.inverse, a.midpoint, a.v.center, rows, threads, a.v.length);
     }
@@ -132,7 +149,7 @@ void launch_stages(const FusedArgs& a, hipStream_t stream) {
     if (stored_params) {
       value_params_kernel<false><<<(groups + 3) / 4, 256, 0, stream>>>(
           a.part_max, a.part_min, a.v.scale, a.v.center, a.inverse, a.midpoint, a.v.head_dim, a.chunks, groups);
-      prepare_stage2_kernel<DT, DK, CTA_K, ROT, kParamsStored><<<stage2_blocks, 256, 0, stream>>>(a);
+      prepare_stage2_kernel<DT, DK, CTA_K, ROT, kParamsStored><<<stage2_blocks, 256, 0, stream>>>(with_center);
     } else {
       prepare_stage2_kernel<DT, DK, CTA_K, ROT, kParamsAbsmax><<<stage2_blocks, 256, 0, stream>>>(a);
     }

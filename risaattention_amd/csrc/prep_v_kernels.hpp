@@ -318,19 +318,17 @@ __global__ __launch_bounds__(256) void value_codes_kernel(const void* __restrict
 // grid (T / (256/quads), B*H), 256 threads: thread = (summation thread t, four channels);
 // four rather than eight channels per thread so that a long sequence fills every SIMD.
 template <int DT>
-__global__ __launch_bounds__(256) void value_residual_kernel(const void* __restrict__ v,
-                                                             float* __restrict__ partial,
-                                                             const float* __restrict__ inverse,
-                                                             const float* __restrict__ midpoint,
-                                                             int length, int dim, int heads,
-                                                             int threads, int64_t stride_b,
-                                                             int64_t stride_h, int64_t stride_n,
-                                                             const int32_t* __restrict__ permutation) {
-  const int bh = blockIdx.y;
+__device__ __forceinline__ void value_residual_block(const void* __restrict__ v, float* __restrict__ partial,
+                                                     const float* __restrict__ inverse,
+                                                     const float* __restrict__ midpoint, int length,
+                                                     int dim, int heads, int threads, int64_t stride_b,
+                                                     int64_t stride_h, int64_t stride_n,
+                                                     const int32_t* __restrict__ permutation,
+                                                     int block, int bh) {
   const int b = bh / heads, h = bh - b * heads;
   const int quads = dim / 4;
   const int quad = threadIdx.x % quads;
-  const int t = blockIdx.x * (256 / quads) + threadIdx.x / quads;
+  const int t = block * (256 / quads) + threadIdx.x / quads;
   const int64_t base = static_cast<int64_t>(b) * stride_b + static_cast<int64_t>(h) * stride_h;
   const int64_t row0 = static_cast<int64_t>(bh) * dim + quad * 4;
   float inv[4], mid[4], residual[4];
@@ -384,6 +382,19 @@ __global__ __launch_bounds__(256) void value_residual_kernel(const void* __restr
   }
 #pragma unroll
   for (int i = 0; i < 4; ++i) partial[(row0 + i) * threads + t] = residual[i];
+}
+
+template <int DT>
+__global__ __launch_bounds__(256) void value_residual_kernel(const void* __restrict__ v,
+                                                             float* __restrict__ partial,
+                                                             const float* __restrict__ inverse,
+                                                             const float* __restrict__ midpoint,
+                                                             int length, int dim, int heads,
+                                                             int threads, int64_t stride_b,
+                                                             int64_t stride_h, int64_t stride_n,
+                                                             const int32_t* __restrict__ permutation) {
+  value_residual_block<DT>(v, partial, inverse, midpoint, length, dim, heads, threads, stride_b, stride_h,
+                           stride_n, permutation, blockIdx.x, blockIdx.y);
 }
 
 // One workgroup of `threads` threads per row: every 32 partials combine with the reference's
