@@ -46,18 +46,20 @@ __global__ __launch_bounds__(256) void prepare_stage1_kernel(const FusedArgs a) 
     return;
   }
   block -= a.anchor_blocks;
-  if (block < a.q_blocks) {
-    const int slice = block % a.q_slices;
-    const int rest = block / a.q_slices;
-    quantize_q_block<DT, DK, ROT>(a.qk.q, a.qk.q_codes, a.qk.q_scale, a.qk.q_len, a.qk.q_heads,
-                                  a.q_slices * 8, a.qk.q_stride_b, a.qk.q_stride_h, a.qk.q_stride_n,
-                                  a.q_wide, slice, rest % a.qk.q_heads, rest / a.qk.q_heads);
+  // then the V range walks (long chunks on long sequences), then the many short Q blocks
+  const int range_blocks = a.range_groups * a.kv;
+  if (block < range_blocks) {
+    value_range_block<DT, AFFINE>(a.v.v, a.part_max, a.part_min, a.v.length, a.v.head_dim, a.v.heads,
+                                  a.chunks, a.v.stride_b, a.v.stride_h, a.v.stride_n,
+                                  block % a.range_groups, block / a.range_groups);
     return;
   }
-  block -= a.q_blocks;
-  value_range_block<DT, AFFINE>(a.v.v, a.part_max, a.part_min, a.v.length, a.v.head_dim, a.v.heads,
-                                a.chunks, a.v.stride_b, a.v.stride_h, a.v.stride_n,
-                                block % a.range_groups, block / a.range_groups);
+  block -= range_blocks;
+  const int slice = block % a.q_slices;
+  const int rest = block / a.q_slices;
+  quantize_q_block<DT, DK, ROT>(a.qk.q, a.qk.q_codes, a.qk.q_scale, a.qk.q_len, a.qk.q_heads,
+                                a.q_slices * 8, a.qk.q_stride_b, a.qk.q_stride_h, a.qk.q_stride_n,
+                                a.q_wide, slice, rest % a.qk.q_heads, rest / a.qk.q_heads);
 }
 
 template <int DT, int DK, int CTA_K, int ROT, int PARAMS>
@@ -215,6 +217,11 @@ int launch_prepare_fused(const QkArgs& qk, const ValueArgs& v, hipStream_t strea
   a.kv = qk.batch * qk.kv_heads;
   a.anchor_blocks = a.kv;
   a.chunks = range_chunks(v.length);
+  // Long absmax sequences whose Q work covers the longer V range walks: fewer, longer chunks,
+  // so that the code blocks reduce the partial ranges themselves (no parameter launch).  The
+  // long midpoint_affine path keeps the stored parameters its residual blocks read.
+  if (!v.midpoint_affine && static_cast<int64_t>(qk.q_len) * qk.q_heads >= static_cast<int64_t>(v.length) * v.heads)
+    a.chunks = capped_range_chunks(v.length);
   a.range_groups = (a.chunks + 3) / 4;
   a.key_tiles = (qk.k_len + qk.cta_k - 1) / qk.cta_k;
   a.key_blocks = a.key_tiles * a.kv;

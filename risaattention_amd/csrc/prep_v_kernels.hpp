@@ -41,6 +41,17 @@ __host__ __device__ inline int range_chunks(int length) {
   return (length + per_wave - 1) / per_wave;
 }
 
+// Whole 64-token groups per chunk when `length` tokens are split into `chunks` chunks.
+__host__ __device__ inline int chunk_tokens(int length, int chunks) {
+  return ((length + chunks - 1) / chunks + 63) / 64 * 64;
+}
+// At most 64 partial ranges per (batch, head): one wavefront of a code block reduces them
+// itself and the parameter launch between the two stages is not needed.
+__host__ __device__ inline int capped_range_chunks(int length) {
+  const int per_wave = 64 * ((length + 4095) / 4096);
+  return (length + per_wave - 1) / per_wave;
+}
+
 __host__ __device__ inline int summation_threads(int length) { return length <= 256 ? 128 : 512; }
 // up to this many tokens the residual sums and the centre are one launch
 constexpr int kFusedCenterMaxLength = 4096;
@@ -70,7 +81,9 @@ __device__ __forceinline__ void value_range_block(const void* __restrict__ v, fl
   if (chunk >= chunks) return;
   const int octets = dim / 8;
   const int octet = lane % octets, row = lane / octets, rows_per_load = 64 / octets;
-  const int per_wave = tokens_per_wave(length);
+  // tokens per chunk follow from the chunk count: tokens_per_wave(length) for the standard
+  // count, more when the caller asked for fewer partial ranges
+  const int per_wave = chunk_tokens(length, chunks);
   const int64_t base = static_cast<int64_t>(b) * stride_b + static_cast<int64_t>(h) * stride_h;
   float mx[8], mn[8];
 #pragma unroll
