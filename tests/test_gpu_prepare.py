@@ -25,6 +25,9 @@ CASES = [
     (torch.bfloat16, 128, 40, 4611, 2, 2, "midpoint_affine", 0.0),
     (torch.float16, 64, 40, 9000, 2, 1, "midpoint_affine", 0.0),
     (torch.float32, 256, 40, 4200, 1, 1, "midpoint_affine", 0.0),
+    # long absmax self-attention shapes take at most 64 partial V ranges and no parameter launch
+    (torch.bfloat16, 128, 5000, 5000, 2, 1, "absmax", 0.0),
+    (torch.float16, 64, 9100, 9100, 1, 1, "absmax", 0.0),
 ]
 
 
