@@ -7,7 +7,17 @@ include quantisation (reference README.md:102-106).  The JSON line reports
 dense-equivalent TOPS (4*B*Hq*Lq*Lk*D operations per call, reference
 benchmarks/plot_scaling.py:66-75), the roofline fraction of the attention
 kernel against the dense INT8 MFMA peak, and the numpy oracle timed on the host
-cores on a bounded sample (N=2048) as the CPU baseline.
+cores on the reference's CPU-sized configuration (N=1024) as the CPU baseline.  The same
+line carries two short side measurements, timed by whoever runs this file: sparse reuse
+against dense at about half coverage (``config.sparse_reuse``) and the masked
+configuration (``config.masked``).
+
+The other workloads (``--workload``) follow the reference's measurement protocol
+(benchmarks/common.py:184-220): every method is warmed up, then timed in samples of
+several calls between two events, with the methods' positions rotated through every slot
+and each complete rotation reversed; seeds 0/1/2; medians of the per-seed medians.
+``--output FILE`` writes the records as JSON (schema of benchmarks/common.py:321-360) and
+``--report FILE`` prints such a file as Markdown tables.
 """
 
 from __future__ import annotations
@@ -30,6 +40,7 @@ INT8_MFMA_PEAK_TOPS = 5000.0  # MI355X dense INT8, published
 # profiles/attention_dense_32k_counters.md.
 ATTENTION_KERNEL_TRAFFIC_BYTES_32K = int((554751.9 * 2.0 + 131072.3) * 1024)
 SHAPE = dict(batch=1, q_heads=16, kv_heads=4, head_dim=128)
+SEEDS = (0, 1, 2)
 
 
 def dense_equivalent_ops(batch, q_heads, q_len, k_len, head_dim):
@@ -59,15 +70,63 @@ def fp32_reference(torch, q, k, v, chunk=2048):
 
 
 def accuracy(torch, actual, reference):
+    """The accuracy record of reference benchmarks/common.py:148-164."""
+    import math
+
     error = actual.float() - reference
     rmse = error.pow(2).mean().sqrt().item()
     rms = reference.pow(2).mean().sqrt().item()
     nrmse = rmse / max(rms, 1e-12)
-    return {"nrmse": nrmse, "sqnr_db": -20.0 * __import__("math").log10(max(nrmse, 1e-30))}
+    return {"rmse": rmse, "nrmse": nrmse, "sqnr_db": -20.0 * math.log10(max(nrmse, 1e-30)),
+            "mae": error.abs().mean().item(), "max_abs": error.abs().max().item(),
+            "max_channel_bias": error.mean(dim=2).abs().max().item(), "reference_rms": rms}
+
+
+def percentile(values, fraction):
+    ordered = sorted(values)
+    position = (len(ordered) - 1) * fraction
+    low = int(position)
+    high = min(low + 1, len(ordered) - 1)
+    return ordered[low] + (ordered[high] - ordered[low]) * (position - low)
+
+
+def measure_methods(torch, methods, samples=10, calls_per_sample=20, warmup=20):
+    """Paired timing of several callables on identical inputs (the protocol of reference
+    benchmarks/common.py:184-220): all are warmed up first; sample i then runs every method
+    once, ``calls_per_sample`` calls between two events on the current stream, in an order
+    that is the name list rotated by i and reversed on every other complete rotation, so
+    that each method takes every position (including first after the idle gap) equally often."""
+    names = list(methods)
+    stream = torch.cuda.current_stream()
+    for function in methods.values():
+        for _ in range(warmup):
+            function()
+    torch.cuda.synchronize()
+    recorded = {name: [] for name in names}
+    for sample in range(samples):
+        cycle, shift = divmod(sample, len(names))
+        base = names if cycle % 2 == 0 else names[::-1]
+        for name in base[shift:] + base[:shift]:
+            begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            begin.record(stream)
+            for _ in range(calls_per_sample):
+                methods[name]()
+            end.record(stream)
+            end.synchronize()
+            recorded[name].append(begin.elapsed_time(end) / calls_per_sample)
+    return {name: {"median_ms": statistics.median(values), "p10_ms": percentile(values, 0.1),
+                   "p90_ms": percentile(values, 0.9), "samples_ms": [round(v, 5) for v in values],
+                   "calls_per_sample": calls_per_sample, "warmup": warmup}
+            for name, values in recorded.items()}
+
+
+def calls_for(ops):
+    """Calls per sample: twenty for short problems, fewer as the call gets long."""
+    return max(2, min(20, int(4e13 / max(ops, 1.0))))
 
 
 def time_calls(torch, fn, calls, warmup=2):
-    """Median-free mean of ``calls`` back-to-back calls, HIP events on the current stream."""
+    """Mean of ``calls`` back-to-back calls, HIP events on the current stream."""
     stream = torch.cuda.current_stream()
     for _ in range(warmup):
         fn()
@@ -87,21 +146,30 @@ def sqnr_db(torch, actual, reference):
 
 
 def workload_sweep(torch, risa, args, device):
-    """Dense sweep over N, three seeds, both V modes; latency includes Q/K/V preparation."""
+    """Dense sweep over N, seeds 0/1/2, both V modes timed as a pair on the same inputs;
+    latency includes Q/K/V preparation; median of the per-seed medians, mean NRMSE."""
     rows = []
     for length in ([args.length] if args.length else (512, 1024, 2048, 4096, 8192, 16384, 32768)):
         ops = dense_equivalent_ops(SHAPE["batch"], SHAPE["q_heads"], length, length, SHAPE["head_dim"])
-        for mode in ("absmax", "midpoint_affine"):
-            samples, errors = [], []
-            for seed in (0, 1, 2):
-                q, k, v = make_inputs(torch, length, seed, device)
-                calls = max(3, min(50, int(2e10 / ops * 20)))
-                samples.append(time_calls(torch, lambda: risa.int8_attention(q, k, v, v_quantization=mode), calls))
-                out = risa.int8_attention(q, k, v, v_quantization=mode)
-                errors.append(accuracy(torch, out, fp32_reference(torch, q, k, v))["nrmse"])
-            ms = statistics.median(samples)
-            rows.append({"N": length, "v_quantization": mode, "ms": round(ms, 4),
-                         "tops": round(ops / (ms * 1e-3) / 1e12, 1), "nrmse": round(statistics.median(errors), 5)})
+        medians = {"absmax": [], "midpoint_affine": []}
+        records = {"absmax": [], "midpoint_affine": []}
+        for seed in SEEDS:
+            q, k, v = make_inputs(torch, length, seed, device)
+            methods = {mode: (lambda mode=mode: risa.int8_attention(q, k, v, v_quantization=mode)) for mode in medians}
+            timing = measure_methods(torch, methods, samples=args.samples, calls_per_sample=calls_for(ops),
+                                     warmup=args.method_warmup)
+            reference = fp32_reference(torch, q, k, v)
+            for mode in medians:
+                medians[mode].append(timing[mode]["median_ms"])
+                records[mode].append(accuracy(torch, methods[mode](), reference))
+            del reference
+        for mode in medians:
+            ms = statistics.median(medians[mode])
+            rows.append({"N": length, "v_quantization": mode, "ms": round(ms, 4), "per_seed_ms": [round(x, 4) for x in medians[mode]],
+                         "tops": round(ops / (ms * 1e-3) / 1e12, 1),
+                         "nrmse": round(statistics.mean(r["nrmse"] for r in records[mode]), 5),
+                         "sqnr_db": round(statistics.mean(r["sqnr_db"] for r in records[mode]), 2),
+                         "accuracy_per_seed": records[mode]})
     return rows
 
 
@@ -117,29 +185,37 @@ def outlier_inputs(torch, shape_q, shape_k, seed, device):
     return q.bfloat16(), k.bfloat16(), v.bfloat16()
 
 
-def workload_masked(torch, risa, args, device):
-    """Unequal lengths, outlier channels; causal, key-padding mask, additive bias, LSE."""
+def masked_variants(torch, batch, q_len, k_len, device):
+    key_padding = torch.ones(batch, 1, 1, k_len, dtype=torch.bool, device=device)
+    key_padding[1, ..., int(k_len * 0.9):] = False
+    generator = torch.Generator(device=device).manual_seed(1)
+    bias = torch.randn(batch, 1, q_len, k_len, generator=generator, device=device)  # float32
+    rowmask = torch.ones(batch, 1, q_len, k_len, dtype=torch.bool, device=device)
+    rowmask[0, :, :7] = False  # fully masked rows
+    return {"plain": dict(), "causal": dict(is_causal=True), "key_padding": dict(attn_mask=key_padding),
+            "additive_bias": dict(attn_mask=bias), "bool_mask_lse": dict(attn_mask=rowmask, return_lse=True)}
+
+
+def workload_masked(torch, risa, args, device, dims=(64, 128), seeds=None, samples=None):
+    """Unequal lengths, outlier channels; plain, causal, key-padding mask, additive bias, boolean
+    mask + LSE, timed as one rotating group per seed and head dim."""
     rows = []
     batch, heads, q_len, k_len = 2, 24, 4096, 4608
-    for dim in (64, 128):
-        q, k, v = outlier_inputs(torch, (batch, heads, q_len, dim), (batch, heads, k_len, dim), 0, device)
+    variants = masked_variants(torch, batch, q_len, k_len, device)
+    for dim in dims:
         ops = dense_equivalent_ops(batch, heads, q_len, k_len, dim)
-        key_padding = torch.ones(batch, 1, 1, k_len, dtype=torch.bool, device=device)
-        key_padding[1, ..., int(k_len * 0.9):] = False
-        generator = torch.Generator(device=device).manual_seed(1)
-        bias = torch.randn(batch, 1, q_len, k_len, generator=generator, device=device)  # float32
-        rowmask = torch.ones(batch, 1, q_len, k_len, dtype=torch.bool, device=device)
-        rowmask[0, :, :7] = False  # fully masked rows
-        variants = {
-            "plain": dict(),
-            "causal": dict(is_causal=True),
-            "key_padding": dict(attn_mask=key_padding),
-            "additive_bias": dict(attn_mask=bias),
-            "bool_mask_lse": dict(attn_mask=rowmask, return_lse=True),
-        }
-        for name, kwargs in variants.items():
-            ms = time_calls(torch, lambda: risa.int8_attention(q, k, v, **kwargs), 10)
-            rows.append({"D": dim, "variant": name, "ms": round(ms, 4),
+        medians = {name: [] for name in variants}
+        for seed in (seeds or SEEDS):
+            q, k, v = outlier_inputs(torch, (batch, heads, q_len, dim), (batch, heads, k_len, dim), seed, device)
+            methods = {name: (lambda kwargs=kwargs: risa.int8_attention(q, k, v, **kwargs)) for name, kwargs in variants.items()}
+            timing = measure_methods(torch, methods, samples=samples or args.samples, calls_per_sample=10,
+                                     warmup=args.method_warmup)
+            for name in variants:
+                medians[name].append(timing[name]["median_ms"])
+        for name in variants:
+            ms = statistics.median(medians[name])
+            rows.append({"D": dim, "variant": name, "ms": round(ms, 4), "per_seed_ms": [round(x, 4) for x in medians[name]],
+                         "vs_plain": round(ms / statistics.median(medians["plain"]), 3),
                          "tops": round(ops / (ms * 1e-3) / 1e12 * (0.5 if name == "causal" else 1.0), 1)})
     return rows
 
@@ -197,38 +273,66 @@ def workload_sparse(torch, risa, args, device):
     return rows
 
 
-def workload_sparse_blocks(torch, risa, args, device):
-    """The sparse table of the reference's README: Q/K = N(0,1) + one of two prototypes of
-    norm 8 per 128-token block (alternating), theta = 0.99, construction on the clean
-    tensors, reuse on tensors drifted by 0.05 (reference benchmarks/sparse.py:30-60,
-    README.md:127-142).  About half of the key tiles carry the mass of every query block."""
-    rows = []
+def block_prototype_inputs(torch, length, seed, device):
+    """Q/K = N(0,1) + one of two prototypes of norm 8 per 128-token block (alternating), V ~
+    N(0,1); clean tensors for the construction, tensors drifted by 0.05 for the reuse
+    (reference benchmarks/sparse.py:30-60)."""
     dim, kv_heads, q_heads = SHAPE["head_dim"], SHAPE["kv_heads"], SHAPE["q_heads"]
+    generator = torch.Generator(device=device).manual_seed(seed)
+    draw = lambda *shape: torch.randn(shape, generator=generator, device=device)
+    clean_q, clean_k, v32 = draw(1, q_heads, length, dim), draw(1, kv_heads, length, dim), draw(1, kv_heads, length, dim)
+    prototypes = draw(1, kv_heads, 2, dim)
+    prototypes = prototypes * (8.0 / prototypes.norm(dim=-1, keepdim=True))
+    block = (torch.arange(length, device=device) // 128) % 2
+    clean_k = clean_k + prototypes[:, :, block]
+    clean_q = clean_q + prototypes.repeat_interleave(q_heads // kv_heads, 1)[:, :, block]
+    drifted_q = (clean_q + 0.05 * draw(*clean_q.shape)).bfloat16()
+    drifted_k = (clean_k + 0.05 * draw(*clean_k.shape)).bfloat16()
+    return clean_q.bfloat16(), clean_k.bfloat16(), v32.bfloat16(), drifted_q, drifted_k
+
+
+def sparse_blocks_case(torch, risa, length, mode, seeds, samples, method_warmup, device, with_quality=True):
+    """One row of the reference's sparse table: construction / dense / reuse timed as a
+    rotating group on every seed; medians of the per-seed medians."""
+    ops = dense_equivalent_ops(SHAPE["batch"], SHAPE["q_heads"], length, length, SHAPE["head_dim"])
+    medians = {"construct": [], "dense": [], "reuse": []}
+    coverage, sparse_quality, dense_quality = [], [], []
+    for seed in seeds:
+        q0, k0, v, drifted_q, drifted_k = block_prototype_inputs(torch, length, seed, device)
+        build = lambda: risa.construct_sparse_int8_attention(q0, k0, v, theta=0.99, v_quantization=mode)
+        _, pattern = build()
+        dense = lambda: risa.int8_attention(drifted_q, drifted_k, v, v_quantization=mode)
+        reuse = lambda: risa.sparse_int8_attention(drifted_q, drifted_k, v, pattern, v_quantization=mode)
+        timing = measure_methods(torch, {"construct": build, "dense": dense, "reuse": reuse}, samples=samples,
+                                 calls_per_sample=calls_for(ops), warmup=method_warmup)
+        for name in medians:
+            medians[name].append(timing[name]["median_ms"])
+        coverage.append(pattern.coverage)
+        if with_quality:
+            reference = fp32_reference(torch, drifted_q, drifted_k, v)
+            sparse_quality.append(sqnr_db(torch, reuse(), reference))
+            dense_quality.append(sqnr_db(torch, dense(), reference))
+            del reference
+    row = {"N": length, "v_quantization": mode, "inputs": "two prototypes of norm 8 alternating per 128-token block, "
+           "theta 0.99, drift 0.05 (the reference README's sparse table)", "seeds": list(seeds),
+           "construct_ms": round(statistics.median(medians["construct"]), 4),
+           "dense_ms": round(statistics.median(medians["dense"]), 4),
+           "reuse_ms": round(statistics.median(medians["reuse"]), 4),
+           "coverage": round(statistics.mean(coverage), 4)}
+    row["speedup"] = round(row["dense_ms"] / row["reuse_ms"], 3)
+    if with_quality:
+        row["sparse_sqnr_db"] = round(statistics.mean(sparse_quality), 2)
+        row["dense_sqnr_db"] = round(statistics.mean(dense_quality), 2)
+    return row
+
+
+def workload_sparse_blocks(torch, risa, args, device):
+    """The sparse table of the reference's README (README.md:127-142): about half of the key
+    tiles carry the mass of every query block."""
+    rows = []
     for length in ([args.length] if args.length else (1024, 2048, 4096, 8192, 16384, 32768)):
-        generator = torch.Generator(device=device).manual_seed(0)
-        draw = lambda *shape: torch.randn(shape, generator=generator, device=device)
-        clean_q, clean_k, v32 = draw(1, q_heads, length, dim), draw(1, kv_heads, length, dim), draw(1, kv_heads, length, dim)
-        prototypes = draw(1, kv_heads, 2, dim)
-        prototypes = prototypes * (8.0 / prototypes.norm(dim=-1, keepdim=True))
-        block = (torch.arange(length, device=device) // 128) % 2
-        clean_k = clean_k + prototypes[:, :, block]
-        clean_q = clean_q + prototypes.repeat_interleave(q_heads // kv_heads, 1)[:, :, block]
-        drifted_q = (clean_q + 0.05 * draw(*clean_q.shape)).bfloat16()
-        drifted_k = (clean_k + 0.05 * draw(*clean_k.shape)).bfloat16()
-        q0, k0, v = clean_q.bfloat16(), clean_k.bfloat16(), v32.bfloat16()
-        reference = fp32_reference(torch, drifted_q, drifted_k, v)
         for mode in ("absmax", "midpoint_affine"):
-            build = lambda: risa.construct_sparse_int8_attention(q0, k0, v, theta=0.99, v_quantization=mode)
-            construct_ms = time_calls(torch, build, 5, 2)
-            _, pattern = build()
-            dense = lambda: risa.int8_attention(drifted_q, drifted_k, v, v_quantization=mode)
-            sparse = lambda: risa.sparse_int8_attention(drifted_q, drifted_k, v, pattern, v_quantization=mode)
-            dense_ms, sparse_ms = time_calls(torch, dense, 20, 3), time_calls(torch, sparse, 20, 3)
-            rows.append({"N": length, "v_quantization": mode, "construct_ms": round(construct_ms, 4),
-                         "dense_ms": round(dense_ms, 4), "sparse_ms": round(sparse_ms, 4),
-                         "speedup": round(dense_ms / sparse_ms, 3), "coverage": round(pattern.coverage, 4),
-                         "sparse_sqnr_db": round(sqnr_db(torch, sparse(), reference), 2),
-                         "dense_sqnr_db": round(sqnr_db(torch, dense(), reference), 2)})
+            rows.append(sparse_blocks_case(torch, risa, length, mode, SEEDS, args.samples, args.method_warmup, device))
     return rows
 
 
@@ -317,9 +421,10 @@ def workload_video(torch, risa, args, device):
             "loop_speedup_vs_dense": round(10 * dense_ms / (construct_ms + sum(reuse)), 3)}
 
 
-def cpu_baseline(length=2048, calls=5):
-    """Oracle (numpy port of the quantised pipeline) on the host cores: a bounded sample
-    of the headline workload (same heads and head dim, N=2048; about ten seconds)."""
+def cpu_baseline(length=1024, calls=15):
+    """Oracle (numpy port of the quantised pipeline) on the host cores: the reference's own
+    CPU-sized configuration (same heads and head dim as the headline, N=1024, seed 0,
+    tensors drawn in the order q, k, v; about ten seconds of CPU work)."""
     import numpy as np
     import torch
 
@@ -351,6 +456,73 @@ def cpu_baseline(length=2048, calls=5):
     }
 
 
+def dense_kernel_name(torch, length):
+    """Which kernel an unmasked dense launch of this length takes (the 16-query kernel serves
+    launches with no more 128-query workgroups than the GPU has compute units)."""
+    workgroups = SHAPE["batch"] * SHAPE["q_heads"] * ((length + 127) // 128)
+    units = torch.cuda.get_device_properties(0).multi_processor_count
+    return "attention_narrow_kernel<128,128>" if workgroups <= units else "attention_kernel<128,128,fast>"
+
+
+def write_records(torch, risa, args, rows):
+    """One JSON file per run in the layout of reference benchmarks/common.py:321-360."""
+    import hashlib
+    from datetime import datetime, timezone
+
+    from risaattention_amd import native
+
+    digest = hashlib.sha256()
+    for path in sorted((ROOT / "risaattention_amd").rglob("*")):
+        if path.suffix in (".py", ".hip", ".hpp", ".h") or path.name == "Makefile":
+            digest.update(path.relative_to(ROOT).as_posix().encode())
+            digest.update(path.read_bytes())
+    library = Path(native.library_path())
+    config = {key: (str(value) if isinstance(value, Path) else value) for key, value in vars(args).items()
+              if key not in ("output", "report")}
+    config["timing_order"] = "rotate-and-reverse"
+    config["seeds"] = list(SEEDS)
+    payload = {
+        "schema_version": 2,
+        "suite": args.workload,
+        "measured_at_utc": datetime.now(timezone.utc).isoformat(),
+        "environment": {
+            "gpu": torch.cuda.get_device_name(),
+            "arch": torch.cuda.get_device_properties(0).gcnArchName,
+            "hip": torch.version.hip,
+            "versions": {"torch": torch.__version__},
+            "package_path": risa.__file__,
+            "source_sha256": digest.hexdigest(),
+            "extension_sha256": hashlib.sha256(library.read_bytes()).hexdigest(),
+        },
+        "config": config,
+        "reference": "FP32 PyTorch attention in query chunks",
+        "results": rows if isinstance(rows, list) else [rows],
+    }
+    args.output.parent.mkdir(parents=True, exist_ok=True)
+    args.output.write_text(json.dumps(payload, indent=2, allow_nan=False) + "\n")
+
+
+def render_report(payload):
+    """Markdown tables from a file written with --output (the role of reference
+    benchmarks/report.py): one table per suite, columns in the order of the README tables."""
+    columns = {
+        "sweep": ["N", "v_quantization", "ms", "tops", "nrmse", "sqnr_db"],
+        "masked": ["D", "variant", "ms", "vs_plain", "tops"],
+        "sparse_blocks": ["N", "v_quantization", "construct_ms", "dense_ms", "reuse_ms", "speedup", "coverage",
+                          "sparse_sqnr_db", "dense_sqnr_db"],
+    }
+    results = payload["results"]
+    names = columns.get(payload["suite"]) or [key for key, value in results[0].items() if not isinstance(value, (list, dict))]
+    environment = payload["environment"]
+    lines = [f"## {payload['suite']} — {environment['gpu']} ({environment.get('arch', '')}), {payload['measured_at_utc']}",
+             f"timing: {payload['config'].get('timing_order')}, seeds {payload['config'].get('seeds')}, "
+             f"{payload['config'].get('samples')} samples per method; reference: {payload['reference']}", "",
+             "| " + " | ".join(names) + " |", "|" + "---|" * len(names)]
+    for row in results:
+        lines.append("| " + " | ".join(str(row.get(name, "")) for name in names) + " |")
+    return "\n".join(lines)
+
+
 def main():
     parser = argparse.ArgumentParser()
     parser.add_argument("--gpus", type=int, default=1)
@@ -364,9 +536,18 @@ def main():
     parser.add_argument("--workload", default="dense", choices=["dense", "sweep", "masked", "sparse", "sparse_blocks", "video", "prepare"],
                         help="dense = headline N=32K line (default); the others are the remaining benchmark "
                              "configurations of the reference, reported as one JSON line each")
+    parser.add_argument("--samples", type=int, default=10, help="event-timed samples per method and seed (--workload)")
+    parser.add_argument("--method-warmup", type=int, default=20, help="warm-up calls per method before its samples (--workload)")
+    parser.add_argument("--no-side-measurements", action="store_true",
+                        help="dense line only: skip config.sparse_reuse and config.masked")
+    parser.add_argument("--output", type=Path, default=None, help="also write the records of a --workload run to this JSON file")
+    parser.add_argument("--report", type=Path, default=None, help="print a file written with --output as Markdown tables and exit")
     parser.add_argument("--calibrate-copy", action="store_true",
                         help="only run a 1 GiB device copy (reference point for rocprofv3 FETCH_SIZE/WRITE_SIZE)")
     args = parser.parse_args()
+    if args.report is not None:
+        print(render_report(json.loads(args.report.read_text())))
+        return
     if args.gpus != 1:
         print("bench.py measures one MI355X; this path uses no second GPU",
               file=sys.stderr)
@@ -395,6 +576,8 @@ def main():
                   "sparse_blocks": workload_sparse_blocks}[args.workload]
         wall = time.perf_counter()
         rows = runner(torch, risa, args, device)
+        if args.output is not None:
+            write_records(torch, risa, args, rows)
         print(json.dumps({"metric": f"{args.workload} workload (see config.rows)", "value": None, "unit": "ms",
                           "n_gpus": 1, "steps": None, "warmup": None, "ms_per_step": None,
                           "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "int8",
@@ -456,16 +639,31 @@ def main():
             "prepare_ms": prepare_ms,
         },
         "roofline": {
+            # The contract of this line names the roof the fraction is taken against; the
+            # kernel's limiter on this hardware is the vector-instruction issue of the U8
+            # softmax next to the matrix instructions (profiles/attention_dense_32k_counters.md).
             "bound": "mfma",
+            "limited_by": "VALU issue of the softmax + MFMA (they share the SIMD issue capacity)",
             "achieved": achieved_tops,
             "peak": INT8_MFMA_PEAK_TOPS,
             "unit": "TOP/s",
             "frac": achieved_tops / INT8_MFMA_PEAK_TOPS,
+            # not measured in this run: the figure recorded from rocprofv3 for this shape
             "traffic": ATTENTION_KERNEL_TRAFFIC_BYTES_32K if (length == 32768 and args.mode == "absmax") else None,
-            "traffic_unit": "bytes per launch (rocprofv3 FETCH_SIZE + WRITE_SIZE, recorded)",
-            "kernel": "attention_kernel<128,128,fast>",
+            "traffic_source": "recorded from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs "
+                              "(profiles/attention_dense_32k_counters.md), bytes per launch",
+            "kernel": dense_kernel_name(torch, length),
         },
     }
+    if not args.no_side_measurements:
+        del out
+        result["config"]["sparse_reuse"] = sparse_blocks_case(
+            torch, risa, length, args.mode, seeds=(0,), samples=6, method_warmup=3, device=device, with_quality=False)
+        result["config"]["sparse_reuse"]["note"] = (
+            "BASELINE config 4's own recipe (64 groups, centroid x 3) keeps 1.6 % of the tiles and is not this row: "
+            "see --workload sparse")
+        result["config"]["masked"] = workload_masked(torch, risa, args, device, dims=(128, 64), seeds=(0,), samples=4)
+        out = step()
     if not args.no_accuracy:
         reference = fp32_reference(torch, q, k, v)
         result["config"]["accuracy_vs_fp32_sdpa"] = accuracy(torch, out, reference)

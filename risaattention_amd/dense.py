@@ -43,8 +43,15 @@ _masked_op.register_fake(_same_shape_as_query)
 
 
 def _plain_eager(*tensors) -> bool:
-    """Ordinary tensors outside tracing: nothing needs to see an operator boundary."""
+    """Ordinary tensors with nobody watching the dispatcher: no operator boundary is needed.
+
+    A compile in progress, an active ``TorchDispatchMode`` (``make_fx``, fake or
+    functional modes, user modes) and a ``torch.jit.trace`` all record what goes through
+    the dispatcher; the native call is invisible to them, so they must see the operator.
+    """
     if torch.compiler.is_compiling():
+        return False
+    if torch._C._len_torch_dispatch_stack() != 0 or torch._C._get_tracing_state() is not None:
         return False
     return all(t is None or type(t) is torch.Tensor for t in tensors)
 

@@ -50,6 +50,33 @@ def test_dense_matches_oracle(risa, mode, dim, causal, mask_name):
     torch.testing.assert_close(out.float(), reference, atol=0.10, rtol=0.03)
 
 
+@pytest.mark.parametrize("dim,heads,k_len", [(128, 4, 1300), (64, 4, 700), (256, 2, 1300), (128, 144, 1300)])
+@pytest.mark.parametrize("variant", ["plain", "causal", "row_mask", "key_bias"])
+def test_outlier_channels_match_oracle(risa, dim, heads, k_len, variant):
+    """One channel in a hundred scaled by 20: near one-hot attention rows, large score
+    scales.  144 heads x 3 query blocks take the 32-query kernel, the others the 16-query one."""
+    generator = torch.Generator().manual_seed(23)
+    q_len = 300
+    q = torch.randn(1, heads, q_len, dim, generator=generator)
+    k = torch.randn(1, 2, k_len, dim, generator=generator)
+    v = torch.randn(1, 2, k_len, dim, generator=generator)
+    hot = torch.randperm(dim, generator=generator)[: max(1, dim // 100)]
+    for tensor in (q, k, v):
+        tensor[..., hot] *= 20.0
+    q, k, v = (t.to(torch.bfloat16).cuda() for t in (q, k, v))
+    masks = mask_variants(q_len, k_len)
+    mask = masks.get(variant)
+    causal = variant == "causal"
+    out, lse = risa.int8_attention(q, k, v, attn_mask=mask, is_causal=causal, return_lse=True)
+    oracle_heads = slice(0, min(heads, 8))  # the oracle on a slice of whole KV groups
+    kv = slice(0, 1) if heads > 8 else slice(0, 2)
+    prepared = oracle_prequantize(q[:, oracle_heads], k[:, kv], v[:, kv], attn_mask=mask, is_causal=causal,
+                                  return_lse=True)
+    expected, expected_lse, _ = oracle_pipeline.attend(prepared, return_lse=True)
+    assert relative_l2(to_numpy(out[:, oracle_heads]), expected) < TOLERANCE
+    assert relative_l2(to_numpy(lse[:, oracle_heads]), expected_lse) < TOLERANCE
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("k_len", [1153, 2304])
 def test_large_tile_dense_and_scale_signs(risa, dtype, k_len):

@@ -59,6 +59,39 @@ def test_prepared_tensors_match_oracle_bit_for_bit(risa, dtype, dim, q_len, k_le
     assert kernel_dim in (64, 128, 256)
 
 
+@pytest.mark.parametrize("dim,k_len,mode", [(128, 1300, "absmax"), (64, 700, "midpoint_affine"),
+                                            (256, 1100, "midpoint_affine"), (128, 200, "absmax")])
+@pytest.mark.parametrize("shifted", [False, True])
+def test_outlier_channels_bit_for_bit(risa, dim, k_len, mode, shifted):
+    """One channel in a hundred scaled by 20 (the masked benchmark configuration's inputs): the
+    case the rotation spreads over the block and, with a common key offset on top, the anchor
+    removes.  Codes, scales, centres, anchors and the LSE shift equal the oracle's bit for bit."""
+    from risaattention_amd.layout import unpack_values
+
+    generator = torch.Generator().manual_seed(11)
+    q = torch.randn(2, 4, 150, dim, generator=generator)
+    k = torch.randn(2, 2, k_len, dim, generator=generator)
+    v = torch.randn(2, 2, k_len, dim, generator=generator)
+    hot = torch.randperm(dim, generator=generator)[: max(1, dim // 100)]
+    for tensor in (q, k, v):
+        tensor[..., hot] *= 20.0
+    if shifted:
+        k = k * 0.1 + 5.0 * torch.randn(1, 1, 1, dim, generator=generator)
+    q, k, v = (t.to(torch.bfloat16).cuda() for t in (q, k, v))
+    packed = risa.prequantize_int8_attention(q, k, v, v_quantization=mode, return_lse=True)
+    expected = oracle_prequantize(q, k, v, v_quantization=mode, return_lse=True)
+    if shifted:
+        assert (expected.anchor >= 0).all(), "a common key offset should trigger the anchor"
+    np.testing.assert_array_equal(packed.q.cpu().numpy(), expected.q)
+    np.testing.assert_array_equal(packed.q_scale.cpu().numpy(), expected.q_scale)
+    np.testing.assert_array_equal(packed.k.cpu().numpy(), expected.k)
+    np.testing.assert_array_equal(packed.k_scale.cpu().numpy(), expected.k_scale)
+    np.testing.assert_array_equal(unpack_values(packed.v).cpu().numpy(), expected.v)
+    np.testing.assert_array_equal(packed.v_scale.cpu().numpy(), expected.v_scale)
+    np.testing.assert_array_equal(packed.v_center.cpu().numpy(), expected.v_center)
+    np.testing.assert_array_equal(to_numpy(packed.lse_shift), expected.lse_shift)
+
+
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("layout", ["hnd", "nhd", "interleaved"])
 @pytest.mark.parametrize("length", [1025, 2048, 2049, 4097])
@@ -146,6 +179,19 @@ def test_fused_permutation_matches_materialized_gather(risa, dtype, layout, mode
     index = indices[..., None].expand_as(k)
     plain = risa.prequantize_int8_attention(q, k.gather(2, index), v.gather(2, index), v_quantization=mode)
     assert torch.equal(plain.k, fused.k) and torch.equal(plain.v, fused.v)
+    # the oracle on the materialised gather pins the fused path outside the library
+    from risaattention_amd.layout import unpack_values
+
+    expected = oracle_prequantize(q, k.gather(2, index), v.gather(2, index), v_quantization=mode)
+    assert (expected.anchor >= 0).all()
+    np.testing.assert_array_equal(fused.k.cpu().numpy(), expected.k)
+    np.testing.assert_array_equal(fused.k_scale.cpu().numpy(), expected.k_scale)
+    np.testing.assert_array_equal(unpack_values(fused.v).cpu().numpy(), expected.v)
+    np.testing.assert_array_equal(fused.v_scale.cpu().numpy(), expected.v_scale)
+    np.testing.assert_array_equal(fused.v_center.cpu().numpy(), expected.v_center)
+    sums = oracle_prepare.value_tile_sums(expected.v, expected.cta_k)
+    got = fused.v_tile_sum.cpu().numpy().transpose(0, 2, 1).reshape(expected.v.shape[0], -1)
+    np.testing.assert_array_equal(got, sums * 128 + 0x4B400000)
     out = risa.int8_attention(q, k, v, kv_permutation=permutation, v_quantization=mode)
     expected = risa.int8_attention_from_prequantized(plain)
     assert torch.equal(out, expected)

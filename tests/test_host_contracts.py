@@ -157,6 +157,44 @@ def test_fake_tensor_shapes():
             assert masked.shape == q.shape
 
 
+def test_operator_is_recorded_whenever_the_dispatcher_is_watched():
+    """Plain eager tensors skip the operator dispatch; under make_fx(real), a
+    TorchDispatchMode or torch.jit.trace the call must go through
+    risa_attention::int8_attention[_masked] (reference src/risa_attention/dense.py:123-146
+    always dispatches through them), or the recorded graph would miss the kernel."""
+    from torch.fx.experimental.proxy_tensor import make_fx
+    from torch.utils._python_dispatch import TorchDispatchMode
+
+    q = torch.randn(1, 2, 3, 64)
+    mask = torch.ones(3, 3, dtype=torch.bool)
+    with patch.object(dense, "execute_dense_attention", side_effect=lambda q, *a, **k: q.clone()):
+        # eager: no operator involved
+        seen = []
+
+        class Recorder(TorchDispatchMode):
+            def __torch_dispatch__(self, func, types, args=(), kwargs=None):
+                seen.append(str(func))
+                return func(*args, **(kwargs or {}))
+
+        assert dense._plain_eager(q, q, q, None)
+        with Recorder():
+            assert not dense._plain_eager(q, q, q, None)
+            risa.int8_attention(q, q, q)
+            risa.int8_attention(q, q, q, attn_mask=mask)
+        assert any("risa_attention.int8_attention.default" in name for name in seen)
+        assert any("risa_attention.int8_attention_masked.default" in name for name in seen)
+
+        graph = make_fx(lambda a: risa.int8_attention(a, a, a) + 1, tracing_mode="real")(q)
+        targets = [str(node.target) for node in graph.graph.nodes if node.op == "call_function"]
+        assert any("risa_attention.int8_attention" in name for name in targets), targets
+        masked = make_fx(lambda a, m: risa.int8_attention(a, a, a, attn_mask=m), tracing_mode="real")(q, mask)
+        targets = [str(node.target) for node in masked.graph.nodes if node.op == "call_function"]
+        assert any("risa_attention.int8_attention_masked" in name for name in targets), targets
+
+        traced = torch.jit.trace(lambda a: risa.int8_attention(a, a, a), (q,), check_trace=False)
+        assert "risa_attention::int8_attention" in str(traced.graph)
+
+
 def test_mask_signature_and_score_mask():
     mask = torch.ones(1, 1, 3, 5, dtype=torch.bool)
     before = policy.mask_signature(mask)
@@ -250,3 +288,48 @@ def test_bench_rejects_more_than_one_gpu():
 
     done = subprocess.run([sys.executable, str(ROOT / "bench.py"), "--gpus", "2"], capture_output=True, text=True)
     assert done.returncode != 0 and "one MI355X" in done.stderr
+
+
+def test_bench_paired_timing_rotates_and_reverses_positions():
+    """bench.py's timing protocol (reference benchmarks/common.py:184-220): after the warm-ups
+    every sample runs all methods, in the name order rotated by the sample index and reversed
+    on every other complete rotation."""
+    import importlib.util
+    import types as pytypes
+
+    spec = importlib.util.spec_from_file_location("bench_module", ROOT / "bench.py")
+    bench = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(bench)
+
+    class Event:
+        clock = 0.0
+
+        def __init__(self, enable_timing=True):
+            self.at = None
+
+        def record(self, stream=None):
+            Event.clock += 1.0
+            self.at = Event.clock
+
+        def synchronize(self):
+            pass
+
+        def elapsed_time(self, other):
+            return other.at - self.at
+
+    fake = pytypes.SimpleNamespace(cuda=pytypes.SimpleNamespace(
+        current_stream=lambda: None, synchronize=lambda: None, Event=Event))
+    calls = []
+    methods = {name: (lambda name=name: calls.append(name)) for name in "abc"}
+    stats = bench.measure_methods(fake, methods, samples=6, calls_per_sample=2, warmup=1)
+    assert calls[:3] == ["a", "b", "c"]  # warm-ups
+    order = calls[3::2]
+    assert order == list("abc" "bca" "cab" "cba" "bac" "acb")
+    assert all(len(stats[name]["samples_ms"]) == 6 and stats[name]["median_ms"] == 0.5 for name in "abc")
+    assert bench.percentile([1.0, 2.0, 3.0, 4.0], 0.5) == 2.5
+    report = bench.render_report({
+        "suite": "sweep", "measured_at_utc": "now", "reference": "fp32",
+        "environment": {"gpu": "MI355X", "arch": "gfx950"},
+        "config": {"timing_order": "rotate-and-reverse", "seeds": [0, 1, 2], "samples": 10},
+        "results": [{"N": 512, "v_quantization": "absmax", "ms": 0.025, "tops": 85.0, "nrmse": 0.0145, "sqnr_db": 36.8}]})
+    assert "| 512 | absmax | 0.025 | 85.0 | 0.0145 | 36.8 |" in report
