@@ -78,6 +78,25 @@ int risa_quantize_v(const void* v, void* out, float* scale, float* center, int32
                     const int32_t* kv_permutation, void* stream);
 
 /*
+ * V preparation for callers that cannot allocate: same arguments, kernels and results as
+ * risa_quantize_v without the workspace, which is an array of
+ * RISA_QUANTIZE_V_NOALLOC_MAX_BYTES (16 MiB) built into the library.  No counterpart in the reference: it is for code
+ * under HIP graph capture, tight serving loops and harnesses that forbid hipMalloc.  The
+ * call allocates nothing; the first call on each device resolves the array's address
+ * (hipGetSymbolAddress), so make that call outside a capture.  Problems whose workspace
+ * (risa_quantize_v_workspace_bytes) exceeds the array are rejected with an error.  All calls
+ * on one GPU share the array: calls that overlap in time on the same GPU race (serialise
+ * them on one stream); nothing in it has to be cleared between calls, every kernel writes
+ * what it later reads.
+ */
+#define RISA_QUANTIZE_V_NOALLOC_MAX_BYTES (16u << 20)
+int risa_quantize_v_noalloc(const void* v, void* out, float* scale, float* center, int32_t* tile_sum,
+                            int batch, int heads, int length, int head_dim, int padded_length,
+                            int cta_k, int64_t stride_b, int64_t stride_h, int64_t stride_n,
+                            int input_dtype, int midpoint_affine, const int32_t* kv_permutation,
+                            void* stream);
+
+/*
  * Q, K and V preparation in one call.  Replaces risa_sdpa_quantize (reference
  * csrc/bindings.cpp:195-272), which also prepares all three operands at once.
  * Arguments as for risa_quantize_qk and risa_quantize_v (padded length =

@@ -6,7 +6,38 @@
 #include "common.hpp"
 #include "launchers.hpp"
 
+#include <mutex>
+
+// Scratch memory of risa_quantize_v_noalloc: the V preparation's partial ranges, channel
+// parameters and residual partial sums, for callers that cannot hand over a workspace.
+// Every GPU the library runs on holds its own copy of this array until the process ends.
+// In host code the name is only a handle for hipGetSymbolAddress; kernels get the address.
+#define RISA_STATIC_SCRATCH_BYTES RISA_QUANTIZE_V_NOALLOC_MAX_BYTES
+static __device__ __align__(256) unsigned char risa_static_scratch[RISA_STATIC_SCRATCH_BYTES];
+
 namespace {
+
+constexpr int kMaxDevices = 64;
+
+// Device address of risa_static_scratch on the current device, resolved once per device.
+int static_scratch_address(void** address) {
+  static std::mutex guard;
+  static void* resolved[kMaxDevices] = {};
+  int device = -1;
+  if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= kMaxDevices)
+    return risa::fail("risa_quantize_v_noalloc: cannot identify the current device");
+  std::lock_guard<std::mutex> lock(guard);
+  if (resolved[device] == nullptr) {
+    void* pointer = nullptr;
+    const hipError_t status = hipGetSymbolAddress(&pointer, HIP_SYMBOL(risa_static_scratch));
+    if (status != hipSuccess || pointer == nullptr)
+      return risa::fail(std::string("risa_quantize_v_noalloc: hipGetSymbolAddress failed: ") +
+                        hipGetErrorString(status));
+    resolved[device] = pointer;
+  }
+  *address = resolved[device];
+  return 0;
+}
 
 bool aligned(const void* pointer, size_t bytes) {
   return reinterpret_cast<uintptr_t>(pointer) % bytes == 0;
@@ -147,6 +178,30 @@ int risa_quantize_v(const void* v, void* out, float* scale, float* center, int32
   const int status = checked_v_args(a, v, out, scale, center, tile_sum, workspace, workspace_bytes,
                                     batch, heads, length, head_dim, padded_length, cta_k, stride_b,
                                     stride_h, stride_n, input_dtype, midpoint_affine, kv_permutation);
+  if (status != 0) return status;
+  return risa::launch_quantize_v(a, static_cast<hipStream_t>(stream));
+}
+
+int risa_quantize_v_noalloc(const void* v, void* out, float* scale, float* center, int32_t* tile_sum,
+                            int batch, int heads, int length, int head_dim, int padded_length,
+                            int cta_k, int64_t stride_b, int64_t stride_h, int64_t stride_n,
+                            int input_dtype, int midpoint_affine, const int32_t* kv_permutation,
+                            void* stream) {
+  if (batch <= 0 || heads <= 0 || length <= 0 || (head_dim != 64 && head_dim != 128 && head_dim != 256))
+    return risa::fail("risa_quantize_v_noalloc: extents must be positive and head_dim 64, 128, or 256");
+  const size_t needed = risa::value_workspace_bytes(batch, heads, length, head_dim, midpoint_affine != 0);
+  if (needed > RISA_STATIC_SCRATCH_BYTES)
+    return risa::fail("risa_quantize_v_noalloc: this problem needs " + std::to_string(needed) +
+                      " bytes of scratch memory, the built-in buffer holds " +
+                      std::to_string(static_cast<size_t>(RISA_STATIC_SCRATCH_BYTES)) +
+                      "; use risa_quantize_v with a caller-provided workspace");
+  void* scratch = nullptr;
+  int status = static_scratch_address(&scratch);
+  if (status != 0) return status;
+  risa::ValueArgs a{};
+  status = checked_v_args(a, v, out, scale, center, tile_sum, scratch, RISA_STATIC_SCRATCH_BYTES, batch,
+                          heads, length, head_dim, padded_length, cta_k, stride_b, stride_h, stride_n,
+                          input_dtype, midpoint_affine, kv_permutation);
   if (status != 0) return status;
   return risa::launch_quantize_v(a, static_cast<hipStream_t>(stream));
 }

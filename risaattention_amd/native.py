@@ -38,6 +38,10 @@ SIGNATURES = {
         _c_int,
         [_c_ptr] * 6 + [_c_size] + [_c_int] * 6 + [_c_i64] * 3 + [_c_int, _c_int, _c_ptr, _c_ptr],
     ),
+    "risa_quantize_v_noalloc": (
+        _c_int,
+        [_c_ptr] * 5 + [_c_int] * 6 + [_c_i64] * 3 + [_c_int, _c_int, _c_ptr, _c_ptr],
+    ),
     "risa_sdpa_quantize": (
         _c_int,
         [_c_ptr] * 12 + [_c_size] + [_c_int] * 7 + [_c_i64] * 9 + [_c_int, _c_int, _c_ptr, _c_ptr, _c_ptr],
