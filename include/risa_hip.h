@@ -45,10 +45,13 @@ int risa_abi_version(void);
  *   q_int8 [B,Hq,Lq,D], k_int8 [B,Hkv,Lk,D] contiguous.
  *   q_scale [B,Hq,ceil(Lq/128)*(D==256?64:32)], k_scale [B,Hkv,ceil(Lk/cta_k)*4].
  *   anchor_indices int32 [B,Hkv]: receives the anchor row or -1.
-  *   kv_permutation (nullable) int32 [B,Hkv,Lk]: key n is read from source token
+ *   kv_permutation (nullable) int32 [B,Hkv,Lk]: key n is read from source token
  *   kv_permutation[b,h,n] (the reference's fused gather, csrc/kernels/
  *   quantize_gather.cu, bindings.cpp:195-272 permutation_ptr); anchors, codes
- *   and scales are those of the gathered K.
+ *   and scales are those of the gathered K.  Every [b,h] row must be a bijection of
+ *   0..Lk-1: the library does not check it, and the V range pass reads the rows in
+ *   storage order (exact for a permutation only; a subset or a list with duplicates
+ *   would give other V scales than a materialised gather).
  */
 int risa_quantize_qk(const void* q, void* q_int8, float* q_scale, const void* k, void* k_int8,
                      float* k_scale, int batch, int q_heads, int q_len, int kv_heads, int k_len,
@@ -67,7 +70,7 @@ int risa_quantize_qk(const void* q, void* q_int8, float* q_scale, const void* k,
  *   of the signed product) + 0x4B400000 (the bits of 1.5 * 2^23, which make the
  *   finished integer accumulator readable as a float); no reference counterpart,
  *   workspace of risa_quantize_v_workspace_bytes(...) bytes.
-  *   kv_permutation (nullable) int32 [B,Hkv,L] as for risa_quantize_qk.
+ *   kv_permutation (nullable) int32 [B,Hkv,L] as for risa_quantize_qk (a bijection per row).
  */
 size_t risa_quantize_v_workspace_bytes(int batch, int heads, int length, int head_dim,
                                        int midpoint_affine);
