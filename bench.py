@@ -479,8 +479,9 @@ def write_records(torch, risa, args, rows):
     library = Path(native.library_path())
     config = {key: (str(value) if isinstance(value, Path) else value) for key, value in vars(args).items()
               if key not in ("output", "report")}
-    config["timing_order"] = "rotate-and-reverse"
-    config["seeds"] = list(SEEDS)
+    paired = args.workload in ("sweep", "masked", "sparse_blocks")
+    config["timing_order"] = "rotate-and-reverse" if paired else "back-to-back calls between two events"
+    config["seeds"] = list(SEEDS) if paired else [0]
     payload = {
         "schema_version": 2,
         "suite": args.workload,

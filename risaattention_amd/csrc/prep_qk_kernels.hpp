@@ -50,9 +50,9 @@ __device__ __forceinline__ void apply_sign_diagonal(float* v, int sub) {
 }
 
 // Value of lane (l xor BIT) for BIT in {1, 2, 4, 8}, with DPP moves (no LDS
-// traffic): quad permutations inside groups of four lanes, row shifts inside
-// rows of sixteen lanes written under a bank mask (lanes whose partner is above
-// take the left shift, the others the right shift).
+// traffic): quad permutations inside groups of four lanes, for BIT 4 two row shifts
+// written under a bank mask (lanes whose partner is above take the left shift, the
+// others the right shift), for BIT 8 one rotation of the row by eight lanes.
 template <int BIT> __device__ __forceinline__ float dpp_partner(float value) {
   const int bits = __float_as_int(value);
   if constexpr (BIT == 1) {
@@ -64,8 +64,8 @@ template <int BIT> __device__ __forceinline__ float dpp_partner(float value) {
     return __int_as_float(__builtin_amdgcn_update_dpp(up, bits, 0x114, 0xf, 0xA, false));  // row_shr:4 -> banks 1, 3
   } else {
     static_assert(BIT == 8, "DPP reaches partners inside a row of sixteen lanes");
-    const int up = __builtin_amdgcn_update_dpp(0, bits, 0x108, 0xf, 0x3, true);      // row_shl:8 -> banks 0, 1
-    return __int_as_float(__builtin_amdgcn_update_dpp(up, bits, 0x118, 0xf, 0xC, false));  // row_shr:8 -> banks 2, 3
+    // rotating a row of sixteen lanes by eight swaps its halves: lane l reads lane l xor 8
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, bits, 0x128, 0xf, 0xf, true));  // row_ror:8
   }
 }
 
