@@ -129,16 +129,24 @@ __device__ __forceinline__ float load1(const void* base, int64_t offset) {
 }
 
 // Round to nearest even, saturate to the signed 8-bit range, NaN -> 0.
-__device__ __forceinline__ int quantize_s8(float value) {
-  float rounded = __builtin_rintf(value);
-  rounded = rounded != rounded ? 0.0f : rounded;
-  rounded = __builtin_fminf(__builtin_fmaxf(rounded, -128.0f), 127.0f);
-  return static_cast<int>(rounded);
+// Round-to-nearest-even conversion of a code in [-127.5, 127.5] by adding 1.5 * 2^23: the sum's
+// integer part is rint(value) (the sum has an ulp of 1 and 1.5 * 2^23 is even, so ties go to the
+// even code), and the low byte of its bit pattern is the two's-complement INT8 code.  One add
+// replaces round, NaN test, clamp and convert; the scales of this library keep |value| below
+// 127.5 for finite inputs (scale > max / 127), so the reference's clamp never binds, and a NaN
+// (0 * inf from a non-finite row) has a zero low byte like the reference's saturating convert.
+constexpr float kRoundMagic = 12582912.0f;
+__device__ __forceinline__ float round_to_code(float value) { return value + kRoundMagic; }
+__device__ __forceinline__ float code_value(float magic_sum) { return magic_sum - kRoundMagic; }
+// Byte k of the result is the code of the k-th argument.
+__device__ __forceinline__ uint32_t pack_codes(float a, float b, float c, float d) {
+  const uint32_t low = __builtin_amdgcn_perm(__float_as_uint(b), __float_as_uint(a), 0x0c0c0400u);
+  const uint32_t high = __builtin_amdgcn_perm(__float_as_uint(d), __float_as_uint(c), 0x0c0c0400u);
+  return low | (high << 16);
 }
-
-__device__ __forceinline__ uint32_t pack_s8x4(int a, int b, int c, int d) {
-  return (static_cast<uint32_t>(a) & 0xffu) | ((static_cast<uint32_t>(b) & 0xffu) << 8) |
-         ((static_cast<uint32_t>(c) & 0xffu) << 16) | ((static_cast<uint32_t>(d) & 0xffu) << 24);
+// Sum of the four signed bytes of a word.
+__device__ __forceinline__ int sum_of_codes(uint32_t packed) {
+  return __builtin_amdgcn_sdot4(static_cast<int>(packed), 0x01010101, 0, false);
 }
 
 // Maximum over lanes l and l ^ 32 (max_across_halves) or l and l ^ 16

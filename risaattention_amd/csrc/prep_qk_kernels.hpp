@@ -243,8 +243,8 @@ __device__ __forceinline__ void quantize_group(const void* in, int64_t in_base, 
         uint32_t packed[GROUPS];
 #pragma unroll
         for (int g = 0; g < GROUPS; ++g) {
-          packed[g] = pack_s8x4(quantize_s8(v[i][block][g][0] * inverse), quantize_s8(v[i][block][g][1] * inverse),
-                                quantize_s8(v[i][block][g][2] * inverse), quantize_s8(v[i][block][g][3] * inverse));
+          packed[g] = pack_codes(round_to_code(v[i][block][g][0] * inverse), round_to_code(v[i][block][g][1] * inverse),
+                                 round_to_code(v[i][block][g][2] * inverse), round_to_code(v[i][block][g][3] * inverse));
         }
         int8_t* at = out + static_cast<int64_t>(n) * DK + channel_of(block, 0);
         if constexpr (GROUPS == 2) {

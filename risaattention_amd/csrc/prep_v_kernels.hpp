@@ -280,7 +280,7 @@ __device__ __forceinline__ void value_codes_block(const void* __restrict__ v, in
     }
     // The four token loads are issued together, outside any branch; tokens past the end
     // read the last row and their codes are zeroed.
-    int q[8][4];
+    float q[8][4];  // codes as magic sums (round_to_code)
     int from[4];
 #pragma unroll
     for (int r = 0; r < 4; ++r) from[r] = min(n0 + r, length - 1);
@@ -294,14 +294,13 @@ __device__ __forceinline__ void value_codes_block(const void* __restrict__ v, in
 #pragma unroll
     for (int r = 0; r < 4; ++r)
 #pragma unroll
-      for (int i = 0; i < 8; ++i) q[i][r] = n0 + r < length ? quantize_s8((x[r][i] - mid[i]) * inv[i]) : 0;
+      for (int i = 0; i < 8; ++i)
+        q[i][r] = n0 + r < length ? round_to_code((x[r][i] - mid[i]) * inv[i]) : kRoundMagic;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-      if (p0 < padded) {
-        *reinterpret_cast<uint32_t*>(codes + (row0 + i) * padded + p0) =
-            pack_s8x4(q[i][0], q[i][1], q[i][2], q[i][3]);
-      }
-      int sum = q[i][0] + q[i][1] + q[i][2] + q[i][3];
+      const uint32_t word = pack_codes(q[i][0], q[i][1], q[i][2], q[i][3]);
+      if (p0 < padded) *reinterpret_cast<uint32_t*>(codes + (row0 + i) * padded + p0) = word;
+      int sum = sum_of_codes(word);
 #pragma unroll
       for (int offset = CTA_K / 8; offset > 0; offset >>= 1) sum += __shfl_xor(sum, offset);
       if ((lane & (CTA_K / 4 - 1)) == 0 && p0 < padded) {
@@ -381,7 +380,7 @@ __device__ __forceinline__ void value_residual_block(const void* __restrict__ v,
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
             const float normalized = (x[j][i] - mid[i]) * inv[i];
-            const float code = static_cast<float>(quantize_s8(normalized));
+            const float code = code_value(round_to_code(normalized));
             residual[i] += normalized - code;
           }
         }
@@ -514,7 +513,7 @@ __device__ __forceinline__ void value_center_block(const void* __restrict__ v, c
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
               const float normalized = (x[j][i] - mid[i]) * inv[i];
-              const float code = static_cast<float>(quantize_s8(normalized));
+              const float code = code_value(round_to_code(normalized));
               residual[i] += normalized - code;
             }
           }
@@ -603,7 +602,7 @@ __global__ __launch_bounds__(512) void value_center_fused_kernel(const void* __r
 #pragma unroll
           for (int i = 0; i < 8; ++i) {
             const float normalized = (x[j][i] - mid[i]) * inv[i];
-            const float code = static_cast<float>(quantize_s8(normalized));
+            const float code = code_value(round_to_code(normalized));
             residual[i] += normalized - code;
           }
         }
