@@ -66,13 +66,14 @@ template <int DT, int DK, int CTA_K, int ROT, int PARAMS>
 __global__ __launch_bounds__(256) void prepare_stage2_kernel(const FusedArgs a) {
   int block = blockIdx.x;
   if (block < a.key_blocks) {
-    // one key tile per workgroup: four wavefronts = its four scale groups
-    const int tile = block % a.key_tiles;
-    const int rest = block / a.key_tiles;
+    // half a key tile per workgroup: two wavefronts for each of its two scale groups
+    const int part = block & 1;
+    const int tile = (block >> 1) % a.key_tiles;
+    const int rest = (block >> 1) / a.key_tiles;
     quantize_k_block<DT, DK, CTA_K, ROT>(a.qk.k, a.qk.k_codes, a.qk.k_scale, a.qk.anchors, a.qk.k_len,
                                          a.qk.kv_heads, a.key_tiles * 4, a.qk.k_stride_b, a.qk.k_stride_h,
-                                         a.qk.k_stride_n, a.k_wide, a.qk.permutation, tile,
-                                         threadIdx.x >> 6, rest % a.qk.kv_heads, rest / a.qk.kv_heads);
+                                         a.qk.k_stride_n, a.k_wide, a.qk.permutation, tile, part,
+                                         rest % a.qk.kv_heads, rest / a.qk.kv_heads);
     return;
   }
   block -= a.key_blocks;
@@ -224,7 +225,7 @@ int launch_prepare_fused(const QkArgs& qk, const ValueArgs& v, hipStream_t strea
     a.chunks = capped_range_chunks(v.length);
   a.range_groups = (a.chunks + 3) / 4;
   a.key_tiles = (qk.k_len + qk.cta_k - 1) / qk.cta_k;
-  a.key_blocks = a.key_tiles * a.kv;
+  a.key_blocks = 2 * a.key_tiles * a.kv;  // half a tile per workgroup
   a.code_blocks_x = (v.padded + 255) / 256;
   a.q_wide = rows_are_16_byte_aligned(qk.q, qk.q_stride_b, qk.q_stride_h, qk.q_stride_n, qk.dtype);
   a.k_wide = rows_are_16_byte_aligned(qk.k, qk.k_stride_b, qk.k_stride_h, qk.k_stride_n, qk.dtype);

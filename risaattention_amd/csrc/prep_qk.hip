@@ -19,7 +19,7 @@ void launch_q(const QkArgs& a, hipStream_t stream) {
 template <int DT, int DK, int CTA_K, int ROT>
 void launch_k(const QkArgs& a, hipStream_t stream) {
   const int tiles = (a.k_len + CTA_K - 1) / CTA_K;
-  dim3 grid(tiles, a.kv_heads, a.batch);
+  dim3 grid(2 * tiles, a.kv_heads, a.batch);  // half a tile (two scale groups) per workgroup
   quantize_k_kernel<DT, DK, CTA_K, ROT><<<grid, 256, 0, stream>>>(
       a.k, a.k_codes, a.k_scale, a.anchors, a.k_len, a.kv_heads, tiles * 4, a.k_stride_b,
       a.k_stride_h, a.k_stride_n,

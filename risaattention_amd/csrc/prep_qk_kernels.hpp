@@ -145,11 +145,15 @@ __device__ __forceinline__ float half_wave_max(float value) {
 // `token_of(i)` gives the i-th token of the group, `sub` the lane's index inside the
 // LANES.  `wide` says rows are 16-byte aligned, so 16-bit inputs are read eight
 // channels per load.
+// `partner_max` (optional): LDS slots through which two wavefronts that share one scale group
+// (each with NTOK of its tokens) exchange their maxima; `partner_max[0]` is written, a
+// workgroup barrier follows, `partner_max[1]` is read.  The maximum is order independent.
 template <int DT, int DK, int ROT, int NTOK, int LANES = 32, typename TokenOf>
 __device__ __forceinline__ void quantize_group(const void* in, int64_t in_base, int64_t stride_n,
                                                int8_t* out, float* scale_slot, int length, int sub,
                                                const void* bias_row, bool wide, TokenOf token_of,
-                                               const int32_t* source = nullptr) {
+                                               const int32_t* source = nullptr,
+                                               float* const* partner_max = nullptr) {
   constexpr int BLOCKS = DK == 256 ? 2 : 1;   // 128-channel rotation blocks
   constexpr int GROUPS = DK == 64 ? 1 : 2;    // runs of four channels per lane and block
   constexpr int PER_STEP = LANES / 16;
@@ -231,6 +235,11 @@ __device__ __forceinline__ void quantize_group(const void* in, int64_t in_base, 
     }
   mx = half_wave_max(mx);
   if constexpr (LANES == 64) mx = max_across_halves(mx);
+  if (partner_max != nullptr) {
+    if (sub == 0) *partner_max[0] = mx;
+    __syncthreads();
+    mx = __builtin_fmaxf(mx, *partner_max[1]);
+  }
   const float scale = mx / 127.0f + 1e-7f;
   const float inverse = 1.0f / scale;
   if (sub == 0) *scale_slot = scale;
@@ -291,9 +300,11 @@ __global__ __launch_bounds__(256) void quantize_q_kernel(const void* __restrict_
                                 stride_n, wide, blockIdx.x, blockIdx.y, blockIdx.z);
 }
 
-// One scale group ((token mod 8) / 2 = `group`) of key tile `tile`, handled by the
-// calling wavefront: four tokens per step keep the per-lane working set at half the
-// registers of a 32-lane group and put twice the wavefronts behind every tile.
+// Half of key tile `tile` (`part` 0 or 1: its scale groups 2*part and 2*part + 1, scale group of
+// a token = (token mod 8) / 2) by one workgroup of four wavefronts: two wavefronts per scale
+// group, each with half of the group's tokens, four tokens per step; the two exchange their
+// maxima through LDS.  A wavefront then keeps CTA_K / 8 rotated tokens in registers instead of
+// CTA_K / 4, and twice as many wavefronts stand behind every tile.
 template <int DT, int DK, int CTA_K, int ROT>
 __device__ __forceinline__ void quantize_k_block(const void* __restrict__ k, int8_t* __restrict__ codes,
                                                  float* __restrict__ scales,
@@ -301,9 +312,13 @@ __device__ __forceinline__ void quantize_k_block(const void* __restrict__ k, int
                                                  int scales_per_head, int64_t stride_b,
                                                  int64_t stride_h, int64_t stride_n, int wide,
                                                  const int32_t* __restrict__ permutation, int tile,
-                                                 int group, int h, int b) {
-  constexpr int NTOK = CTA_K / 4;
+                                                 int part, int h, int b) {
+  constexpr int NTOK = CTA_K / 8;  // tokens of the group held by one wavefront
+  __shared__ float wave_max[4];
   const int sub = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int group = part * 2 + (wave >> 1);
+  const int first_index = (wave & 1) * NTOK;  // this wavefront's share of the group's CTA_K / 4 tokens
   const int64_t in_base = static_cast<int64_t>(b) * stride_b + static_cast<int64_t>(h) * stride_h;
   const int64_t bh = static_cast<int64_t>(b) * heads + h;
   const int anchor = anchors[b * heads + h];
@@ -312,14 +327,15 @@ __device__ __forceinline__ void quantize_k_block(const void* __restrict__ k, int
   const int anchor_row = anchor >= 0 && source != nullptr ? source[anchor] : anchor;
   const int64_t anchor_offset = static_cast<int64_t>(anchor_row) * stride_n;
   const int first = tile * CTA_K + group * 2;
-  quantize_group<DT, DK, ROT, NTOK, 64>(k, in_base, stride_n, codes + bh * length * DK,
-                                    scales + bh * scales_per_head + tile * 4 + group, length, sub,
-                                    anchor >= 0 ? &anchor_offset : nullptr, wide != 0,
-                                    [first](int i) { return first + (i >> 1) * 8 + (i & 1); }, source);
+  float* const exchange[2] = {wave_max + wave, wave_max + (wave ^ 1)};
+  quantize_group<DT, DK, ROT, NTOK, 64>(
+      k, in_base, stride_n, codes + bh * length * DK, scales + bh * scales_per_head + tile * 4 + group,
+      length, sub, anchor >= 0 ? &anchor_offset : nullptr, wide != 0,
+      [first, first_index](int i) { return first + ((i + first_index) >> 1) * 8 + ((i + first_index) & 1); },
+      source, exchange);
 }
 
-// grid (key tiles, Hkv, B), 256 threads: four wavefronts = the four scale groups of
-// one key tile of CTA_K tokens.
+// grid (2 * key tiles, Hkv, B), 256 threads: half a key tile of CTA_K tokens per workgroup.
 template <int DT, int DK, int CTA_K, int ROT>
 __global__ __launch_bounds__(256) void quantize_k_kernel(const void* __restrict__ k,
                                                          int8_t* __restrict__ codes,
@@ -330,8 +346,8 @@ __global__ __launch_bounds__(256) void quantize_k_kernel(const void* __restrict_
                                                          int64_t stride_n, int wide,
                                                          const int32_t* __restrict__ permutation) {
   quantize_k_block<DT, DK, CTA_K, ROT>(k, codes, scales, anchors, length, heads, scales_per_head,
-                                       stride_b, stride_h, stride_n, wide, permutation, blockIdx.x,
-                                       threadIdx.x >> 6, blockIdx.y, blockIdx.z);
+                                       stride_b, stride_h, stride_n, wide, permutation, blockIdx.x >> 1,
+                                       blockIdx.x & 1, blockIdx.y, blockIdx.z);
 }
 
 // ---------------------------------------------------------------------------
