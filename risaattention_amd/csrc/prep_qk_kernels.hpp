@@ -69,64 +69,89 @@ template <int BIT> __device__ __forceinline__ float dpp_partner(float value) {
   }
 }
 
-// Hadamard butterflies over the lane bits below LANES, in the reference's order
-// (bit 1 first): the lane with the bit clear keeps a + b, the other b - a.
-template <int LANES> __device__ __forceinline__ void lane_butterflies(float* v, int sub) {
-  auto level = [&](auto bit_tag) {
-    constexpr int BIT = decltype(bit_tag)::value;
-    if constexpr (BIT < LANES) {
+// One Hadamard butterfly level between lanes l and l xor BIT for COUNT values of a lane: the
+// lane with the bit clear keeps a + b, the other b - a (other - v on the lanes with the bit
+// set, other + v on the rest: one exact sign flip and one addition instead of both results and
+// a select).  All values of the lane pass a level together, so that the exchanges of one value
+// (which must wait two cycles for the instruction that produced their operand) issue between
+// those of the others.
+template <int BIT, int COUNT> __device__ __forceinline__ void butterfly_level(float* (&values)[COUNT], int sub) {
+  const uint32_t flip = (sub & BIT) ? 0x80000000u : 0u;
+  // The sign flips first, all of them: an instruction with a DPP operand must not follow the
+  // instruction that wrote any of its registers by less than two cycles.
+  float flipped[COUNT];
 #pragma unroll
-      for (int c = 0; c < 4; ++c) {
-        float other;
-        if constexpr (BIT < 16) {
-          other = dpp_partner<BIT>(v[c]);
-        } else {
-          other = __shfl_xor(v[c], BIT);
-        }
-        // other - v on the lanes with the bit set, other + v on the rest: one sign
-        // flip (exact) and one addition instead of both results and a select
-        const uint32_t flip = (sub & BIT) ? 0x80000000u : 0u;
-        v[c] = other + __uint_as_float(__float_as_uint(v[c]) ^ flip);
+  for (int n = 0; n < COUNT; ++n) flipped[n] = __uint_as_float(__float_as_uint(*values[n]) ^ flip);
+  asm volatile("" ::: "memory");
+  if constexpr (BIT == 4) {
+    // l xor 4 = (l xor 3) xor 7: the reversal of every quad, then the reversal of every eight
+    // lanes; the second move joins the addition.  (A row shift reaches l xor 4 only for half
+    // of the lanes, which takes two moves that cannot join it.)
+    int reversed[COUNT];
+#pragma unroll
+    for (int n = 0; n < COUNT; ++n)
+      reversed[n] = __builtin_amdgcn_update_dpp(0, __float_as_int(*values[n]), 0x1B, 0xf, 0xf, true);  // quad_perm [3,2,1,0]
+    asm volatile("" ::: "memory");
+#pragma unroll
+    for (int n = 0; n < COUNT; ++n)
+      *values[n] = __int_as_float(__builtin_amdgcn_update_dpp(0, reversed[n], 0x141, 0xf, 0xf, true)) +  // row_half_mirror
+                   flipped[n];
+  } else {
+#pragma unroll
+    for (int n = 0; n < COUNT; ++n) {
+      float other;
+      if constexpr (BIT < 16) {
+        other = dpp_partner<BIT>(*values[n]);
+      } else {
+        other = __shfl_xor(*values[n], BIT);
       }
+      *values[n] = other + flipped[n];
     }
-  };
-  level(std::integral_constant<int, 1>{});
-  level(std::integral_constant<int, 2>{});
-  level(std::integral_constant<int, 4>{});
-  level(std::integral_constant<int, 8>{});
-  level(std::integral_constant<int, 16>{});
+  }
 }
 
-// Rotation of the channels one lane holds of one 128-channel block (64 for head
-// dim 64).  Sixteen lanes share a token; lane j owns GROUPS runs of four
-// consecutive channels, 4*GROUPS*j + 4g .. +3, i.e. the channels of lanes 2j and
-// 2j+1 (GROUPS 2) or of lane j (GROUPS 1) of the reference's 32-lane layout
-// (csrc/kernels/quantize_qk.cuh).  The additions are the reference's, in its
-// order: 4-point transform per run, then one butterfly level per channel bit from
-// bit 2 up -- the first inside the lane when it holds two runs, the others
-// between lanes with DPP moves.
-template <int ROT, int GROUPS> __device__ __forceinline__ void rotate(float (&v)[GROUPS][4], int j) {
+// Rotation of the channels one lane holds of SETS 128-channel blocks (64 channels for head
+// dim 64), SETS = tokens x blocks the lane works on.  Sixteen lanes share a token; lane j
+// owns GROUPS runs of four consecutive channels per block, 4*GROUPS*j + 4g .. +3, i.e. the
+// channels of lanes 2j and 2j+1 (GROUPS 2) or of lane j (GROUPS 1) of the reference's 32-lane
+// layout (csrc/kernels/quantize_qk.cuh).  The additions are the reference's, in its order for
+// every value: 4-point transform per run, then one butterfly level per channel bit from bit 2
+// up -- the first inside the lane when it holds two runs, the others between lanes with DPP
+// moves, bits 1, 2, 4, 8 of the lane index in turn.
+template <int ROT, int GROUPS, int SETS> __device__ __forceinline__ void rotate(float (*v[SETS])[4], int j) {
 #pragma unroll
-  for (int g = 0; g < GROUPS; ++g) {
-    if constexpr (ROT == kRot128Signed) apply_sign_diagonal(v[g], GROUPS * j + g);
-    rotate4(v[g]);
-  }
+  for (int set = 0; set < SETS; ++set)
+#pragma unroll
+    for (int g = 0; g < GROUPS; ++g) {
+      if constexpr (ROT == kRot128Signed) apply_sign_diagonal(v[set][g], GROUPS * j + g);
+      rotate4(v[set][g]);
+    }
   if constexpr (ROT == kRot4) return;
   if constexpr (GROUPS == 2) {
 #pragma unroll
-    for (int c = 0; c < 4; ++c) {
-      const float low = v[0][c], high = v[1][c];
-      v[0][c] = low + high;
-      v[1][c] = low - high;
-    }
-  }
+    for (int set = 0; set < SETS; ++set)
 #pragma unroll
-  for (int g = 0; g < GROUPS; ++g) lane_butterflies<16>(v[g], j);
+      for (int c = 0; c < 4; ++c) {
+        const float low = v[set][0][c], high = v[set][1][c];
+        v[set][0][c] = low + high;
+        v[set][1][c] = low - high;
+      }
+  }
+  constexpr int COUNT = SETS * GROUPS * 4;
+  float* values[COUNT];
+#pragma unroll
+  for (int set = 0; set < SETS; ++set)
+#pragma unroll
+    for (int g = 0; g < GROUPS; ++g)
+#pragma unroll
+      for (int c = 0; c < 4; ++c) values[(set * GROUPS + g) * 4 + c] = &v[set][g][c];
+  butterfly_level<1, COUNT>(values, j);
+  butterfly_level<2, COUNT>(values, j);
+  butterfly_level<4, COUNT>(values, j);
+  butterfly_level<8, COUNT>(values, j);
   constexpr float factor = ROT == kRot64 ? 0.25f : 0.1767766952966369f;
 #pragma unroll
-  for (int g = 0; g < GROUPS; ++g)
-#pragma unroll
-    for (int c = 0; c < 4; ++c) v[g][c] *= factor;
+  for (int n = 0; n < COUNT; ++n) *values[n] *= factor;
 }
 
 // Maximum over the 32 lanes of a half wavefront, in every lane: one lane swap for the
@@ -223,16 +248,28 @@ __device__ __forceinline__ void quantize_group(const void* in, int64_t in_base, 
           v[i][block][g][c] = valid[i] ? shifted : 0.0f;
         }
   float mx = 0.0f;
+  {
+    // Eight token-blocks (32 values of a lane) at a time through the butterfly levels: enough
+    // independent exchanges to hide their operand latency, few enough to stay in registers.
+    constexpr int SETS = STEPS * BLOCKS;
+    constexpr int BATCH = SETS < 8 ? SETS : 8;
+    static_assert(SETS % BATCH == 0, "whole batches");
+#pragma unroll
+    for (int first = 0; first < SETS; first += BATCH) {
+      float (*sets[BATCH])[4];
+#pragma unroll
+      for (int n = 0; n < BATCH; ++n) sets[n] = v[(first + n) / BLOCKS][(first + n) % BLOCKS];
+      rotate<ROT, GROUPS, BATCH>(sets, j);
+    }
+  }
 #pragma unroll
   for (int i = 0; i < STEPS; ++i)
 #pragma unroll
-    for (int block = 0; block < BLOCKS; ++block) {
-      rotate<ROT, GROUPS>(v[i][block], j);
+    for (int block = 0; block < BLOCKS; ++block)
 #pragma unroll
       for (int g = 0; g < GROUPS; ++g)
 #pragma unroll
         for (int c = 0; c < 4; ++c) mx = __builtin_fmaxf(mx, __builtin_fabsf(v[i][block][g][c]));
-    }
   mx = half_wave_max(mx);
   if constexpr (LANES == 64) mx = max_across_halves(mx);
   if (partner_max != nullptr) {
