@@ -170,15 +170,15 @@ __device__ __forceinline__ float half_wave_max(float value) {
 // `token_of(i)` gives the i-th token of the group, `sub` the lane's index inside the
 // LANES.  `wide` says rows are 16-byte aligned, so 16-bit inputs are read eight
 // channels per load.
-// `partner_max` (optional): LDS slots through which two wavefronts that share one scale group
-// (each with NTOK of its tokens) exchange their maxima; `partner_max[0]` is written, a
-// workgroup barrier follows, `partner_max[1]` is read.  The maximum is order independent.
+// `own_max` / `partner_max` (optional): LDS slots through which two wavefronts that share one
+// scale group (each with NTOK of its tokens) exchange their maxima; `own_max` is written, a
+// workgroup barrier follows, `partner_max` is read.  The maximum is order independent.
 template <int DT, int DK, int ROT, int NTOK, int LANES = 32, typename TokenOf>
 __device__ __forceinline__ void quantize_group(const void* in, int64_t in_base, int64_t stride_n,
                                                int8_t* out, float* scale_slot, int length, int sub,
-                                               const void* bias_row, bool wide, TokenOf token_of,
-                                               const int32_t* source = nullptr,
-                                               float* const* partner_max = nullptr) {
+                                               bool has_bias, int64_t bias_offset, bool wide, TokenOf token_of,
+                                               const int32_t* source = nullptr, float* own_max = nullptr,
+                                               const float* partner_max = nullptr) {
   constexpr int BLOCKS = DK == 256 ? 2 : 1;   // 128-channel rotation blocks
   constexpr int GROUPS = DK == 64 ? 1 : 2;    // runs of four channels per lane and block
   constexpr int PER_STEP = LANES / 16;
@@ -208,9 +208,8 @@ __device__ __forceinline__ void quantize_group(const void* in, int64_t in_base, 
 #pragma unroll
     for (int i = 0; i < STEPS; ++i) from[i] = source[from[i]];
   }
-  const bool has_bias = bias_row != nullptr;
   const int64_t bias_base =
-      in_base + (has_bias ? *static_cast<const int64_t*>(bias_row) : static_cast<int64_t>(from[0]) * stride_n);
+      in_base + (has_bias ? bias_offset : static_cast<int64_t>(from[0]) * stride_n);
   auto load_all = [&](auto wide_tag) {
     constexpr bool EIGHT = GROUPS == 2 && DT != kF32 && decltype(wide_tag)::value;
     auto load_row = [&](int64_t row_base, float (&dst)[BLOCKS][GROUPS][4]) {
@@ -272,10 +271,10 @@ __device__ __forceinline__ void quantize_group(const void* in, int64_t in_base, 
         for (int c = 0; c < 4; ++c) mx = __builtin_fmaxf(mx, __builtin_fabsf(v[i][block][g][c]));
   mx = half_wave_max(mx);
   if constexpr (LANES == 64) mx = max_across_halves(mx);
-  if (partner_max != nullptr) {
-    if (sub == 0) *partner_max[0] = mx;
+  if (own_max != nullptr) {
+    if (sub == 0) *own_max = mx;
     __syncthreads();
-    mx = __builtin_fmaxf(mx, *partner_max[1]);
+    mx = __builtin_fmaxf(mx, *partner_max);
   }
   const float scale = mx / 127.0f + 1e-7f;
   const float inverse = 1.0f / scale;
@@ -320,7 +319,7 @@ __device__ __forceinline__ void quantize_q_block(const void* __restrict__ q, int
   const int base = slice * W + group;
   quantize_group<DT, DK, ROT, NR>(q, in_base, stride_n, codes + bh * length * DK,
                                   scales + bh * scales_per_head + slice * 8 + group, length, sub,
-                                  nullptr, wide != 0, [base](int i) { return base + i * 8; });
+                                  false, 0, wide != 0, [base](int i) { return base + i * 8; });
 }
 
 // grid (slices, Hq, B), 256 threads.  One slice (8 KB of input) per workgroup: two or
@@ -364,12 +363,11 @@ __device__ __forceinline__ void quantize_k_block(const void* __restrict__ k, int
   const int anchor_row = anchor >= 0 && source != nullptr ? source[anchor] : anchor;
   const int64_t anchor_offset = static_cast<int64_t>(anchor_row) * stride_n;
   const int first = tile * CTA_K + group * 2;
-  float* const exchange[2] = {wave_max + wave, wave_max + (wave ^ 1)};
   quantize_group<DT, DK, ROT, NTOK, 64>(
       k, in_base, stride_n, codes + bh * length * DK, scales + bh * scales_per_head + tile * 4 + group,
-      length, sub, anchor >= 0 ? &anchor_offset : nullptr, wide != 0,
+      length, sub, anchor >= 0, anchor_offset, wide != 0,
       [first, first_index](int i) { return first + ((i + first_index) >> 1) * 8 + ((i + first_index) & 1); },
-      source, exchange);
+      source, wave_max + wave, wave_max + (wave ^ 1));
 }
 
 // grid (2 * key tiles, Hkv, B), 256 threads: half a key tile of CTA_K tokens per workgroup.
