@@ -125,6 +125,63 @@ def calls_for(ops):
     return max(2, min(20, int(4e13 / max(ops, 1.0))))
 
 
+RECORDS = []  # per-seed records of a --workload run, in the reference's result schema
+
+
+def case_label(batch, q_heads, kv_heads, q_len, k_len, dim):
+    return f"B{batch}_Hq{q_heads}_Hkv{kv_heads}_Lq{q_len}_Lk{k_len}_D{dim}"
+
+
+def add_record(case, shape, seed, qk_distribution, value_distribution, mode, stage, timing, error=None,
+               memory=None, sparse=None):
+    """One measurement of one method on one seed, with the field names of reference
+    benchmarks/common.py:250-268 (so that its report tool reads the files written here)."""
+    RECORDS.append({"case": case, "shape": shape, "seed": seed, "layout": "hnd",
+                    "qk_distribution": qk_distribution, "value_distribution": value_distribution,
+                    "implementation": "risaattention_amd", "v_quantization": mode, "stage": stage,
+                    "timing": timing, "accuracy": error, "memory": memory, "sparse": sparse})
+
+
+def peak_memory(torch, function):
+    """Device memory a call allocates beyond what is resident (reference benchmarks/common.py:222-233)."""
+    torch.cuda.synchronize()
+    resident = torch.cuda.memory_allocated()
+    torch.cuda.reset_peak_memory_stats()
+    output = function()
+    torch.cuda.synchronize()
+    peak = max(0, torch.cuda.max_memory_allocated() - resident) / 1024**2
+    del output
+    return {"peak_incremental_mib": peak}
+
+
+GROUP_FIELDS = ("case", "layout", "qk_distribution", "value_distribution", "implementation", "v_quantization", "stage")
+
+
+def summarize_records(records):
+    """Per (case, method): median over the seeds of the per-seed medians, mean accuracy, mean
+    sparse figures (the aggregation of reference benchmarks/report.py:23-63)."""
+    groups = {}
+    for record in records:
+        groups.setdefault(tuple(record[field] for field in GROUP_FIELDS), []).append(record)
+    rows = []
+    for key, members in groups.items():
+        row = dict(zip(GROUP_FIELDS, key))
+        row["seed_count"] = len(members)
+        for metric in ("median_ms", "p10_ms", "p90_ms"):
+            row[metric] = statistics.median(member["timing"][metric] for member in members)
+        errors = [member["accuracy"] for member in members if member["accuracy"] is not None]
+        for metric in ("nrmse", "rmse", "sqnr_db", "mae", "max_abs", "max_channel_bias"):
+            row[metric] = statistics.mean(error[metric] for error in errors) if errors else None
+        row["nrmse_std"] = statistics.stdev(error["nrmse"] for error in errors) if len(errors) > 1 else (0 if errors else None)
+        memory = [member["memory"]["peak_incremental_mib"] for member in members if member["memory"]]
+        row["peak_incremental_mib"] = statistics.median(memory) if memory else None
+        sparse = [member["sparse"] for member in members if member["sparse"]]
+        for metric in ("coverage", "pattern_index_mib", "exact_construction_recall", "current_recall"):
+            row[metric] = statistics.mean(entry[metric] for entry in sparse) if sparse else None
+        rows.append(row)
+    return rows
+
+
 def time_calls(torch, fn, calls, warmup=2):
     """Mean of ``calls`` back-to-back calls, HIP events on the current stream."""
     stream = torch.cuda.current_stream()
@@ -149,27 +206,30 @@ def workload_sweep(torch, risa, args, device):
     """Dense sweep over N, seeds 0/1/2, both V modes timed as a pair on the same inputs;
     latency includes Q/K/V preparation; median of the per-seed medians, mean NRMSE."""
     rows = []
+    batch, q_heads, kv_heads, dim = SHAPE["batch"], SHAPE["q_heads"], SHAPE["kv_heads"], SHAPE["head_dim"]
     for length in ([args.length] if args.length else (512, 1024, 2048, 4096, 8192, 16384, 32768)):
-        ops = dense_equivalent_ops(SHAPE["batch"], SHAPE["q_heads"], length, length, SHAPE["head_dim"])
-        medians = {"absmax": [], "midpoint_affine": []}
-        records = {"absmax": [], "midpoint_affine": []}
+        ops = dense_equivalent_ops(batch, q_heads, length, length, dim)
+        case = case_label(batch, q_heads, kv_heads, length, length, dim)
+        shape = dict(batch=batch, q_heads=q_heads, kv_heads=kv_heads, q_len=length, k_len=length, head_dim=dim)
+        first = len(RECORDS)
         for seed in SEEDS:
             q, k, v = make_inputs(torch, length, seed, device)
-            methods = {mode: (lambda mode=mode: risa.int8_attention(q, k, v, v_quantization=mode)) for mode in medians}
+            methods = {mode: (lambda mode=mode: risa.int8_attention(q, k, v, v_quantization=mode))
+                       for mode in ("absmax", "midpoint_affine")}
             timing = measure_methods(torch, methods, samples=args.samples, calls_per_sample=calls_for(ops),
                                      warmup=args.method_warmup)
             reference = fp32_reference(torch, q, k, v)
-            for mode in medians:
-                medians[mode].append(timing[mode]["median_ms"])
-                records[mode].append(accuracy(torch, methods[mode](), reference))
+            for mode, method in methods.items():
+                add_record(case, shape, seed, "normal", "normal", mode, "dense", timing[mode],
+                           accuracy(torch, method(), reference), peak_memory(torch, method))
             del reference
-        for mode in medians:
-            ms = statistics.median(medians[mode])
-            rows.append({"N": length, "v_quantization": mode, "ms": round(ms, 4), "per_seed_ms": [round(x, 4) for x in medians[mode]],
-                         "tops": round(ops / (ms * 1e-3) / 1e12, 1),
-                         "nrmse": round(statistics.mean(r["nrmse"] for r in records[mode]), 5),
-                         "sqnr_db": round(statistics.mean(r["sqnr_db"] for r in records[mode]), 2),
-                         "accuracy_per_seed": records[mode]})
+        for summary in summarize_records(RECORDS[first:]):
+            ms = summary["median_ms"]
+            rows.append({"N": length, "v_quantization": summary["v_quantization"], "ms": round(ms, 4),
+                         "p10_ms": round(summary["p10_ms"], 4), "p90_ms": round(summary["p90_ms"], 4),
+                         "tops": round(ops / (ms * 1e-3) / 1e12, 1), "nrmse": round(summary["nrmse"], 5),
+                         "nrmse_std": round(summary["nrmse_std"], 6), "sqnr_db": round(summary["sqnr_db"], 2),
+                         "peak_incremental_mib": round(summary["peak_incremental_mib"], 1)})
     return rows
 
 
@@ -204,18 +264,21 @@ def workload_masked(torch, risa, args, device, dims=(64, 128), seeds=None, sampl
     variants = masked_variants(torch, batch, q_len, k_len, device)
     for dim in dims:
         ops = dense_equivalent_ops(batch, heads, q_len, k_len, dim)
-        medians = {name: [] for name in variants}
+        case = case_label(batch, heads, heads, q_len, k_len, dim)
+        shape = dict(batch=batch, q_heads=heads, kv_heads=heads, q_len=q_len, k_len=k_len, head_dim=dim)
+        first = len(RECORDS)
         for seed in (seeds or SEEDS):
             q, k, v = outlier_inputs(torch, (batch, heads, q_len, dim), (batch, heads, k_len, dim), seed, device)
             methods = {name: (lambda kwargs=kwargs: risa.int8_attention(q, k, v, **kwargs)) for name, kwargs in variants.items()}
             timing = measure_methods(torch, methods, samples=samples or args.samples, calls_per_sample=10,
                                      warmup=args.method_warmup)
             for name in variants:
-                medians[name].append(timing[name]["median_ms"])
+                add_record(case, shape, seed, "outlier_channels", "outlier_channels", "absmax", name, timing[name])
+        summaries = {summary["stage"]: summary for summary in summarize_records(RECORDS[first:])}
         for name in variants:
-            ms = statistics.median(medians[name])
-            rows.append({"D": dim, "variant": name, "ms": round(ms, 4), "per_seed_ms": [round(x, 4) for x in medians[name]],
-                         "vs_plain": round(ms / statistics.median(medians["plain"]), 3),
+            ms = summaries[name]["median_ms"]
+            rows.append({"D": dim, "variant": name, "ms": round(ms, 4),
+                         "vs_plain": round(ms / summaries["plain"]["median_ms"], 3),
                          "tops": round(ops / (ms * 1e-3) / 1e12 * (0.5 if name == "causal" else 1.0), 1)})
     return rows
 
@@ -294,35 +357,53 @@ def block_prototype_inputs(torch, length, seed, device):
 def sparse_blocks_case(torch, risa, length, mode, seeds, samples, method_warmup, device, with_quality=True):
     """One row of the reference's sparse table: construction / dense / reuse timed as a
     rotating group on every seed; medians of the per-seed medians."""
-    ops = dense_equivalent_ops(SHAPE["batch"], SHAPE["q_heads"], length, length, SHAPE["head_dim"])
-    medians = {"construct": [], "dense": [], "reuse": []}
-    coverage, sparse_quality, dense_quality = [], [], []
+    from risaattention_amd.fp32_patterns import measure_pattern_recall
+
+    batch, q_heads, kv_heads, dim = SHAPE["batch"], SHAPE["q_heads"], SHAPE["kv_heads"], SHAPE["head_dim"]
+    ops = dense_equivalent_ops(batch, q_heads, length, length, dim)
+    case = case_label(batch, q_heads, kv_heads, length, length, dim)
+    shape = dict(batch=batch, q_heads=q_heads, kv_heads=kv_heads, q_len=length, k_len=length, head_dim=dim)
+    first = len(RECORDS)
     for seed in seeds:
         q0, k0, v, drifted_q, drifted_k = block_prototype_inputs(torch, length, seed, device)
         build = lambda: risa.construct_sparse_int8_attention(q0, k0, v, theta=0.99, v_quantization=mode)
         _, pattern = build()
         dense = lambda: risa.int8_attention(drifted_q, drifted_k, v, v_quantization=mode)
         reuse = lambda: risa.sparse_int8_attention(drifted_q, drifted_k, v, pattern, v_quantization=mode)
-        timing = measure_methods(torch, {"construct": build, "dense": dense, "reuse": reuse}, samples=samples,
-                                 calls_per_sample=calls_for(ops), warmup=method_warmup)
-        for name in medians:
-            medians[name].append(timing[name]["median_ms"])
-        coverage.append(pattern.coverage)
+        methods = {"construct": build, "dense": dense, "reuse": reuse}
+        timing = measure_methods(torch, methods, samples=samples, calls_per_sample=calls_for(ops), warmup=method_warmup)
+        errors = {name: None for name in methods}
+        sparse = None
         if with_quality:
             reference = fp32_reference(torch, drifted_q, drifted_k, v)
-            sparse_quality.append(sqnr_db(torch, reuse(), reference))
-            dense_quality.append(sqnr_db(torch, dense(), reference))
+            errors["dense"] = accuracy(torch, dense(), reference)
+            errors["reuse"] = accuracy(torch, reuse(), reference)
             del reference
+            sparse = {"coverage": pattern.coverage, "pattern_index_mib": pattern.index_bytes / 1024**2,
+                      "retained_mass_target": 0.99, "measured_retained_mass": pattern.measured_retained_mass,
+                      "exact_construction_recall": measure_pattern_recall(q0, k0, pattern),
+                      "current_recall": measure_pattern_recall(drifted_q, drifted_k, pattern)}
+        else:
+            sparse = {"coverage": pattern.coverage, "pattern_index_mib": pattern.index_bytes / 1024**2,
+                      "retained_mass_target": 0.99, "measured_retained_mass": pattern.measured_retained_mass,
+                      "exact_construction_recall": float("nan"), "current_recall": float("nan")}
+        for name, method in methods.items():
+            add_record(case, shape, seed, "video_blocks", "normal", mode, name, timing[name], errors[name],
+                       peak_memory(torch, method) if with_quality else None, None if name == "dense" else sparse)
+    summaries = {summary["stage"]: summary for summary in summarize_records(RECORDS[first:])}
     row = {"N": length, "v_quantization": mode, "inputs": "two prototypes of norm 8 alternating per 128-token block, "
            "theta 0.99, drift 0.05 (the reference README's sparse table)", "seeds": list(seeds),
-           "construct_ms": round(statistics.median(medians["construct"]), 4),
-           "dense_ms": round(statistics.median(medians["dense"]), 4),
-           "reuse_ms": round(statistics.median(medians["reuse"]), 4),
-           "coverage": round(statistics.mean(coverage), 4)}
+           "construct_ms": round(summaries["construct"]["median_ms"], 4),
+           "dense_ms": round(summaries["dense"]["median_ms"], 4),
+           "reuse_ms": round(summaries["reuse"]["median_ms"], 4),
+           "coverage": round(summaries["reuse"]["coverage"], 4)}
     row["speedup"] = round(row["dense_ms"] / row["reuse_ms"], 3)
     if with_quality:
-        row["sparse_sqnr_db"] = round(statistics.mean(sparse_quality), 2)
-        row["dense_sqnr_db"] = round(statistics.mean(dense_quality), 2)
+        row["sparse_sqnr_db"] = round(summaries["reuse"]["sqnr_db"], 2)
+        row["dense_sqnr_db"] = round(summaries["dense"]["sqnr_db"], 2)
+        row["exact_construction_recall"] = round(summaries["reuse"]["exact_construction_recall"], 5)
+        row["current_recall"] = round(summaries["reuse"]["current_recall"], 5)
+        row["construct_peak_mib"] = round(summaries["construct"]["peak_incremental_mib"], 1)
     return row
 
 
@@ -465,7 +546,9 @@ def dense_kernel_name(torch, length):
 
 
 def write_records(torch, risa, args, rows):
-    """One JSON file per run in the layout of reference benchmarks/common.py:321-360."""
+    """One JSON file per run in the layout of reference benchmarks/common.py:321-360: per-seed
+    records under `results` (read by the reference's report tool as they are), the summary rows
+    of this run's JSON line under `summary`."""
     import hashlib
     from datetime import datetime, timezone
 
@@ -478,7 +561,7 @@ def write_records(torch, risa, args, rows):
             digest.update(path.read_bytes())
     library = Path(native.library_path())
     config = {key: (str(value) if isinstance(value, Path) else value) for key, value in vars(args).items()
-              if key not in ("output", "report")}
+              if key not in ("output", "report", "csv", "markdown")}
     paired = args.workload in ("sweep", "masked", "sparse_blocks")
     config["timing_order"] = "rotate-and-reverse" if paired else "back-to-back calls between two events"
     config["seeds"] = list(SEEDS) if paired else [0]
@@ -497,30 +580,43 @@ def write_records(torch, risa, args, rows):
         },
         "config": config,
         "reference": "FP32 PyTorch attention in query chunks",
-        "results": rows if isinstance(rows, list) else [rows],
+        "results": RECORDS,
+        "summary": rows if isinstance(rows, list) else [rows],
     }
     args.output.parent.mkdir(parents=True, exist_ok=True)
-    args.output.write_text(json.dumps(payload, indent=2, allow_nan=False) + "\n")
+    args.output.write_text(json.dumps(payload, indent=2, allow_nan=True) + "\n")
 
 
-def render_report(payload):
-    """Markdown tables from a file written with --output (the role of reference
-    benchmarks/report.py): one table per suite, columns in the order of the README tables."""
-    columns = {
-        "sweep": ["N", "v_quantization", "ms", "tops", "nrmse", "sqnr_db"],
-        "masked": ["D", "variant", "ms", "vs_plain", "tops"],
-        "sparse_blocks": ["N", "v_quantization", "construct_ms", "dense_ms", "reuse_ms", "speedup", "coverage",
-                          "sparse_sqnr_db", "dense_sqnr_db"],
-    }
-    results = payload["results"]
-    names = columns.get(payload["suite"]) or [key for key, value in results[0].items() if not isinstance(value, (list, dict))]
+def render_report(payload, csv_path=None):
+    """Summary of a file written with --output (the role of reference benchmarks/report.py): one
+    row per (case, method) with the median of the per-seed medians and the mean accuracy, as a
+    Markdown table and optionally as CSV; suites without per-seed records print their summary rows."""
+    import csv
+
     environment = payload["environment"]
     lines = [f"## {payload['suite']} — {environment['gpu']} ({environment.get('arch', '')}), {payload['measured_at_utc']}",
-             f"timing: {payload['config'].get('timing_order')}, seeds {payload['config'].get('seeds')}, "
-             f"{payload['config'].get('samples')} samples per method; reference: {payload['reference']}", "",
-             "| " + " | ".join(names) + " |", "|" + "---|" * len(names)]
-    for row in results:
-        lines.append("| " + " | ".join(str(row.get(name, "")) for name in names) + " |")
+             f"timing: {payload['config'].get('timing_order')}, seeds {payload['config'].get('seeds')}"
+             + (f", {payload['config'].get('samples')} samples per method and seed"
+                if payload['config'].get('timing_order') == 'rotate-and-reverse' else "")
+             + f"; reference: {payload['reference']}", ""]
+    records = payload.get("results") or []
+    if records and "timing" in records[0]:
+        rows = summarize_records(records)
+        names = ["case", "v_quantization", "stage", "seed_count", "median_ms", "p10_ms", "p90_ms", "nrmse", "sqnr_db",
+                 "peak_incremental_mib", "coverage", "current_recall"]
+        if csv_path is not None:
+            csv_path.parent.mkdir(parents=True, exist_ok=True)
+            with csv_path.open("w", newline="") as file:
+                writer = csv.DictWriter(file, fieldnames=list(rows[0]))
+                writer.writeheader()
+                writer.writerows(rows)
+    else:
+        rows = payload.get("summary") or records
+        names = [key for key, value in rows[0].items() if not isinstance(value, (list, dict))]
+    def shown(value):
+        return "" if value is None else f"{value:.5g}" if isinstance(value, float) else str(value)
+    lines += ["| " + " | ".join(names) + " |", "|" + "---|" * len(names)]
+    lines += ["| " + " | ".join(shown(row.get(name)) for name in names) + " |" for row in rows]
     return "\n".join(lines)
 
 
@@ -542,12 +638,18 @@ def main():
     parser.add_argument("--no-side-measurements", action="store_true",
                         help="dense line only: skip config.sparse_reuse and config.masked")
     parser.add_argument("--output", type=Path, default=None, help="also write the records of a --workload run to this JSON file")
-    parser.add_argument("--report", type=Path, default=None, help="print a file written with --output as Markdown tables and exit")
+    parser.add_argument("--report", type=Path, default=None, help="print a file written with --output as a Markdown table and exit")
+    parser.add_argument("--csv", type=Path, default=None, help="with --report: also write the summary rows as CSV")
+    parser.add_argument("--markdown", type=Path, default=None, help="with --report: also write the table to this file")
     parser.add_argument("--calibrate-copy", action="store_true",
                         help="only run a 1 GiB device copy (reference point for rocprofv3 FETCH_SIZE/WRITE_SIZE)")
     args = parser.parse_args()
     if args.report is not None:
-        print(render_report(json.loads(args.report.read_text())))
+        table = render_report(json.loads(args.report.read_text()), args.csv)
+        if args.markdown is not None:
+            args.markdown.parent.mkdir(parents=True, exist_ok=True)
+            args.markdown.write_text(table + "\n")
+        print(table)
         return
     if args.gpus != 1:
         print("bench.py measures one MI355X; this path uses no second GPU",

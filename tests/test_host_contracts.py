@@ -327,9 +327,36 @@ def test_bench_paired_timing_rotates_and_reverses_positions():
     assert order == list("abc" "bca" "cab" "cba" "bac" "acb")
     assert all(len(stats[name]["samples_ms"]) == 6 and stats[name]["median_ms"] == 0.5 for name in "abc")
     assert bench.percentile([1.0, 2.0, 3.0, 4.0], 0.5) == 2.5
-    report = bench.render_report({
-        "suite": "sweep", "measured_at_utc": "now", "reference": "fp32",
-        "environment": {"gpu": "MI355X", "arch": "gfx950"},
-        "config": {"timing_order": "rotate-and-reverse", "seeds": [0, 1, 2], "samples": 10},
-        "results": [{"N": 512, "v_quantization": "absmax", "ms": 0.025, "tops": 85.0, "nrmse": 0.0145, "sqnr_db": 36.8}]})
-    assert "| 512 | absmax | 0.025 | 85.0 | 0.0145 | 36.8 |" in report
+    # per-seed records in the reference's result schema -> median of the per-seed medians, mean accuracy
+    def record(seed, median, nrmse, stage="dense", sparse=None):
+        return {"case": "B1_Hq16_Hkv4_Lq512_Lk512_D128", "shape": {}, "seed": seed, "layout": "hnd",
+                "qk_distribution": "normal", "value_distribution": "normal", "implementation": "risaattention_amd",
+                "v_quantization": "absmax", "stage": stage,
+                "timing": {"median_ms": median, "p10_ms": median - 0.001, "p90_ms": median + 0.001},
+                "accuracy": {"nrmse": nrmse, "rmse": 1e-4, "sqnr_db": 36.0, "mae": 1e-4, "max_abs": 1e-3,
+                             "max_channel_bias": 1e-4},
+                "memory": {"peak_incremental_mib": 10.0 + seed}, "sparse": sparse}
+
+    records = [record(0, 0.030, 0.0150), record(1, 0.025, 0.0140), record(2, 0.026, 0.0145)]
+    records += [record(seed, 0.020, 0.02, "reuse", {"coverage": 0.5, "pattern_index_mib": 1.0,
+                                                    "exact_construction_recall": 0.99, "current_recall": 0.98})
+                for seed in (0, 1)]
+    rows = bench.summarize_records(records)
+    dense_row = next(row for row in rows if row["stage"] == "dense")
+    assert dense_row["seed_count"] == 3 and dense_row["median_ms"] == 0.026
+    assert dense_row["nrmse"] == pytest.approx(0.0145) and dense_row["peak_incremental_mib"] == 11.0
+    assert dense_row["coverage"] is None
+    reuse_row = next(row for row in rows if row["stage"] == "reuse")
+    assert reuse_row["coverage"] == 0.5 and reuse_row["current_recall"] == 0.98
+    import tempfile
+
+    with tempfile.TemporaryDirectory() as folder:
+        csv_path = Path(folder) / "summary.csv"
+        report = bench.render_report({
+            "suite": "sweep", "measured_at_utc": "now", "reference": "fp32",
+            "environment": {"gpu": "MI355X", "arch": "gfx950"},
+            "config": {"timing_order": "rotate-and-reverse", "seeds": [0, 1, 2], "samples": 10},
+            "results": records}, csv_path)
+        assert "| B1_Hq16_Hkv4_Lq512_Lk512_D128 | absmax | dense | 3 | 0.026 |" in report
+        header, first, *_ = csv_path.read_text().splitlines()
+        assert header.startswith("case,layout,qk_distribution") and "0.026" in first
