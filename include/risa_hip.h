@@ -153,7 +153,11 @@ void risa_unpack_order(int32_t* order);
  *   risa_prepare_key_mask_tiles; key_bias (nullable) float32 [Bm,Hm,padded keys]
  *   from risa_prepare_key_bias with its batch and head strides in elements (0
  *   for a broadcast extent): given together with a key-only mask (mask_stride_q
- *   0), the kernel stages this row per key tile instead of reading mask elements.
+ *   0), the kernel stages this row per key tile instead of reading mask elements;
+ *   mask_lanes (nullable) the lane words of a query-dependent boolean mask from
+ *   risa_prepare_mask_lanes with their batch and head strides in 64-bit words (0
+ *   for a broadcast extent): given together with that mask and 64-key tiles, the
+ *   kernel applies the words instead of reading mask elements.
  */
 int risa_attention(const void* q_int8, const void* k_int8, const void* v_int8, void* out,
                    const float* q_scale, const float* k_scale, const float* v_scale,
@@ -165,7 +169,8 @@ int risa_attention(const void* q_int8, const void* k_int8, const void* v_int8, v
                    const int32_t* sparse_row_offsets, const int32_t* sparse_block_indices,
                    float* block_mass, int is_causal, float* lse, const int32_t* key_mask_tiles,
                    const float* key_bias, int64_t key_bias_stride_b, int64_t key_bias_stride_h,
-                   void* stream);
+                   const uint64_t* mask_lanes, int64_t mask_lanes_stride_b,
+                   int64_t mask_lanes_stride_h, void* stream);
 
 /*
  * Quantise and attend in one call.  Replaces risa_sdpa (reference
@@ -175,14 +180,18 @@ int risa_attention(const void* q_int8, const void* k_int8, const void* v_int8, v
  * one caller-provided workspace of risa_sdpa_workspace_bytes(...) bytes (256-byte
  * aligned).  q/k/v are [B,H,L,D] with element strides, head_dim 64, 128 or 256;
  * out and the mask as for risa_attention; mask_batch / mask_heads are the mask's
- * own extents (1 where it broadcasts).  key_only_mask in the size query says
- * whether a mask with query stride 0 will be passed.  sparse_row_offsets /
+ * own extents (1 where it broadcasts).  The size query takes the description of the
+ * mask that will be passed (mask_dtype -1 for none): a key-only mask needs room for its
+ * bias row and tile list, a boolean mask shared by several heads for its lane words.
+ * sparse_row_offsets /
  * sparse_block_indices (both or neither, as for risa_attention) restrict the
  * attention to a retained-mass pattern: the reuse call of the sparse path
  * (reference src/risa_attention/sparse.py:150-191) in one call as well.
  */
 size_t risa_sdpa_workspace_bytes(int batch, int q_heads, int q_len, int kv_heads, int k_len,
-                                 int head_dim, int cta_k, int midpoint_affine, int key_only_mask);
+                                 int head_dim, int cta_k, int midpoint_affine, int mask_dtype,
+                                 int64_t mask_stride_q, int64_t mask_stride_k, int mask_batch,
+                                 int mask_heads);
 int risa_sdpa(const void* q, const void* k, const void* v, void* out, void* workspace,
               size_t workspace_bytes, int batch, int q_heads, int q_len, int kv_heads, int k_len,
               int head_dim, int cta_k, int64_t q_stride_b, int64_t q_stride_h, int64_t q_stride_n,
@@ -227,6 +236,27 @@ int risa_prepare_key_mask_tiles(const void* mask, int32_t* tiles, int batch, int
 int risa_prepare_key_bias(const void* mask, float* bias, int batch, int heads, int key_length,
                           int padded_length, int64_t stride_b, int64_t stride_h, int64_t stride_k,
                           int mask_dtype, void* stream);
+
+/*
+ * Lane words of a query-dependent boolean mask with unit key stride, for 64-key tiles:
+ * lanes[b,h,w,t,16*rb+i] (64-bit words; b, h over the mask's own extents, w over
+ * 4*ceil(q_len/128) blocks of 32 queries, t over ceil(k_len/64) key tiles) has bit l set
+ * when query 32*w + l%32 may attend to key 64*t + 32*rb + 8*(i/4) + 4*(l/32) + i%4; no bit
+ * is set past the last query or key.  The attention kernel applies one word per score
+ * from scalar registers.  risa_mask_lanes_bytes returns the size of the buffer, or 0
+ * when the form does not apply or does not pay: the mask is not boolean, the tiles are
+ * not 64 keys, the key stride is not 1, the query stride is 0, or fewer than four
+ * (batch, head) pairs share each mask plane (the conversion reads the mask once, the
+ * attention kernel would read it once per pair).  No counterpart in the reference, whose
+ * kernel reads the mask per score (csrc/kernels/attention_masks.cuh:27-164); the
+ * decisions are the ones it takes.
+ */
+size_t risa_mask_lanes_bytes(int mask_dtype, int cta_k, int64_t mask_stride_q, int64_t mask_stride_k,
+                             int batch, int q_heads, int mask_batch, int mask_heads, int q_len,
+                             int k_len);
+int risa_prepare_mask_lanes(const void* mask, uint64_t* lanes, int mask_batch, int mask_heads,
+                            int q_len, int k_len, int64_t stride_b, int64_t stride_h,
+                            int64_t stride_q, void* stream);
 
 /*
  * LSE anchor correction out[b,h,i] = scale * <q[b,h,i], k[b,h/G,anchor[b,h/G]]>.

@@ -10,7 +10,7 @@ import math
 import torch
 
 from . import native
-from .key_mask import prepare_key_bias, prepare_key_mask_tiles
+from .key_mask import prepare_key_bias, prepare_key_mask_tiles, prepare_mask_lanes
 from .policy import (
     DTYPE_CODES,
     MASK_DTYPE_CODES,
@@ -145,6 +145,8 @@ def launch_attention(*, q_codes, k_codes, v_codes, output, q_scale, k_scale, v_s
     sums = ensure_tile_sums(v_codes, v_tile_sum, batch * kv_heads, dim, cta_k)
     key_bias = prepare_key_bias(attn_mask, cta_k)
     bias_args = (None, 0, 0) if key_bias is None else (key_bias[0].data_ptr(), key_bias[1], key_bias[2])
+    mask_lanes = prepare_mask_lanes(attn_mask, cta_k)
+    lane_args = (None, 0, 0) if mask_lanes is None else (mask_lanes[0].data_ptr(), mask_lanes[1], mask_lanes[2])
     out_b = output.stride(0) if batch > 1 else q_heads * q_len * dim
     out_n = output.stride(2) if q_len > 1 else dim
     out_h = output.stride(1) if q_heads > 1 else q_len * dim
@@ -156,7 +158,7 @@ def launch_attention(*, q_codes, k_codes, v_codes, output, q_scale, k_scale, v_s
             out_b, out_n, out_h, float(sm_scale), DTYPE_CODES[output.dtype],
             native.pointer(row_offsets), native.pointer(block_indices), native.pointer(block_mass),
             int(bool(is_causal)), native.pointer(lse), native.pointer(key_mask_tiles),
-            *bias_args, native.current_stream(q_codes.device),
+            *bias_args, *lane_args, native.current_stream(q_codes.device),
         )
     )
 
@@ -186,7 +188,6 @@ def execute_dense_attention(
     batch, q_heads, q_len, _ = q.shape
     kv_heads, k_len = k.shape[1], k.shape[2]
     query_mask = attn_mask is not None and attn_mask.stride(-2) != 0
-    key_only = attn_mask is not None and not query_mask
     cta_k = select_key_block_size(dim, k_len, has_mask=query_mask)
     lib = native.library()
     csr = (None, None)
@@ -201,15 +202,17 @@ def execute_dense_attention(
         output = torch.empty(batch, q_len, q_heads, dim, dtype=out_dtype, device=q.device).permute(0, 2, 1, 3)
     else:
         output = torch.empty(batch, q_heads, q_len, dim, dtype=out_dtype, device=q.device)
-    workspace = torch.empty(
-        lib.risa_sdpa_workspace_bytes(batch, q_heads, q_len, kv_heads, k_len, dim, cta_k,
-                                      int(use_midpoint_affine), int(key_only)),
-        dtype=torch.uint8, device=q.device)
     if attn_mask is None:
         mask_args = (None, 0, 0, 0, 0, -1, 1, 1)
     else:
         mask_args = (attn_mask.data_ptr(), *attn_mask.stride(), MASK_DTYPE_CODES[attn_mask.dtype],
                      batch if attn_mask.stride(0) != 0 else 1, q_heads if attn_mask.stride(1) != 0 else 1)
+    # the size query takes the mask's dtype, query and key strides and own extents
+    workspace = torch.empty(
+        lib.risa_sdpa_workspace_bytes(batch, q_heads, q_len, kv_heads, k_len, dim, cta_k,
+                                      int(use_midpoint_affine), mask_args[5], mask_args[3], mask_args[4],
+                                      mask_args[6], mask_args[7]),
+        dtype=torch.uint8, device=q.device)
     native.check(
         lib.risa_sdpa(
             q.data_ptr(), k.data_ptr(), v.data_ptr(), output.data_ptr(), workspace.data_ptr(),

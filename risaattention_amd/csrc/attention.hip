@@ -128,6 +128,16 @@ int launch_attention(const AttentionArgs& a, hipStream_t stream) {
         mask_mode = kMaskStaged;
       }
     }
+    if (a.mask_lanes != nullptr) {
+      if (a.mask_dtype != kBool || a.cta_k != 64 || a.mask_stride_q == 0)
+        return fail("risa_attention: lane words go with a query-dependent boolean mask and 64-key tiles");
+      if (reinterpret_cast<uintptr_t>(a.mask_lanes) % 8 != 0)
+        return fail("risa_attention: lane words must be 8-byte aligned");
+      mask_mode = kMaskLanes;
+      p.mask_lanes = a.mask_lanes;
+      p.mask_lanes_stride_b = a.mask_lanes_stride_b;
+      p.mask_lanes_stride_h = a.mask_lanes_stride_h;
+    }
     if (a.key_bias != nullptr) {
       if (a.mask_stride_q != 0) return fail("risa_attention: a key bias row needs a key-only mask");
       if (reinterpret_cast<uintptr_t>(a.key_bias) % 16 != 0 || (a.key_bias_stride_b | a.key_bias_stride_h) % 4 != 0)

@@ -46,6 +46,9 @@ int launch_general(const KernelParams& p, bool indexed, bool capture, hipStream_
 template <int D, int CTA_K, int MASK_DT>
 int launch_masked(const KernelParams& p, int mask_mode, bool indexed, bool capture, hipStream_t stream) {
   if constexpr (CTA_K == 64) {
+    if constexpr (MASK_DT == kBool) {
+      if (mask_mode == kMaskLanes) return launch_general<D, CTA_K, MASK_DT, kMaskLanes>(p, indexed, capture, stream);
+    }
     if (mask_mode == kMaskStaged) return launch_general<D, CTA_K, MASK_DT, kMaskStaged>(p, indexed, capture, stream);
     if (mask_mode != kMaskScalar) return launch_general<D, CTA_K, MASK_DT, kMaskVector>(p, indexed, capture, stream);
   }

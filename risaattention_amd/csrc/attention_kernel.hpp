@@ -68,6 +68,8 @@ struct KernelParams {
   int mask_dtype;  // -1: no mask
   const float* key_bias;  // key-only mask as an additive row [Bm,Hm,padded] (mask_dtype kKeyBias)
   int64_t key_bias_stride_b, key_bias_stride_h;
+  const uint64_t* mask_lanes;  // boolean mask as one 64-lane word per score slot (kMaskLanes)
+  int64_t mask_lanes_stride_b, mask_lanes_stride_h;  // in words; 0 where the mask broadcasts
   int q_len, k_len, q_heads, kv_heads, padded, n_kb, n_qb, batch;
   int64_t out_stride_b, out_stride_n, out_stride_h;
   float sm2;  // sm_scale * log2(e)
@@ -141,6 +143,18 @@ template <int D, int CTA_K, int MASK_BYTES = 0, int SHARED_MASK_BYTES = 0> struc
 constexpr int kMaskScalar = 0;  // element by element: any strides
 constexpr int kMaskVector = 1;  // one load per four keys: unit key stride, aligned rows
 constexpr int kMaskStaged = 2;  // mask tile copied to LDS with K and V: 16-byte aligned rows, 64-key tiles
+// Boolean mask shared by several heads, turned beforehand into lane words: for every block
+// of 32 queries, 64-key tile and score slot of the kernel's register layout, the 64 bits
+// that say which lanes keep that score.  The words are wave-uniform, so they arrive through
+// the scalar cache in scalar registers (no vector load, no LDS, no unpacking) and one
+// v_cndmask per score applies them.
+constexpr int kMaskLanes = 3;
+constexpr int kLaneWordsPerTile = 32;  // 64-key tile: two 32-key blocks x 16 scores per lane
+
+// Word index of (block of 32 queries, key tile) within one (batch, head) plane of lane words.
+__host__ __device__ constexpr int64_t lane_word_offset(int64_t query_wave, int64_t key_tiles, int64_t tile) {
+  return (query_wave * key_tiles + tile) * kLaneWordsPerTile;
+}
 
 constexpr int mask_element_bytes(int mask_dtype) { return mask_dtype == kF32 ? 4 : mask_dtype == kBool ? 1 : 2; }
 // LDS bytes of a staged mask tile (128 queries x CTA_K keys).
@@ -168,8 +182,10 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void attention_kernel(cons
   static_assert(!FAST || MASK_DT < 0, "the raw-score path takes no mask");
   static_assert(MASK_MODE == kMaskScalar || (MASK_DT >= 0 && MASK_DT != kKeyBias), "vector loads need a mask tensor");
   static_assert(MASK_MODE != kMaskStaged || CTA_K == 64, "staged masks: 64-key tiles");
+  static_assert(MASK_MODE != kMaskLanes || (CTA_K == 64 && MASK_DT == kBool), "lane words: boolean masks, 64-key tiles");
   constexpr bool MASK_VEC = MASK_MODE != kMaskScalar;
   constexpr bool STAGED = MASK_MODE == kMaskStaged;
+  constexpr bool LANES = MASK_MODE == kMaskLanes;
   constexpr bool SHARED_MASK = STAGED && staged_mask_is_shared(MASK_DT);
   using Shape = AttentionTileShape<D, CTA_K, MASK_DT, MASK_MODE>;
   constexpr int RB = CTA_K / 32;  // 32-key blocks per tile
@@ -281,7 +297,8 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void attention_kernel(cons
   constexpr int MASK_ROW_BYTES = CTA_K * MASK_ES;
   constexpr int MASK_CH = MASK_ROW_BYTES / 16;                       // chunks per row
   constexpr int NM = STAGED ? kQueryBlock * MASK_CH / 256 : 1;       // copy instructions per wave
-  auto mask_swizzle = [](int row) { return (row / (256 / MASK_ROW_BYTES)) & (MASK_CH - 1); };
+  constexpr int MASK_ROWS_PER_256 = MASK_ROW_BYTES >= 256 ? 1 : 256 / MASK_ROW_BYTES;
+  auto mask_swizzle = [](int row) { return (row / MASK_ROWS_PER_256) & (MASK_CH - 1); };
   [[maybe_unused]] const int8_t* mask_block = nullptr;
   if constexpr (STAGED) {
     mask_block = static_cast<const int8_t*>(p.mask) +
@@ -403,6 +420,25 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void attention_kernel(cons
                 static_cast<int64_t>(query) * p.mask_stride_q
           : 0;
 
+  // Lane words of one tile: 16 scalar register pairs per 32-key block, loaded through the
+  // scalar cache from a wave-uniform address.  The words of a tile's first key block are
+  // requested a tile ahead, as soon as their predecessors have been applied; those of the
+  // second block at the start of the softmax, where the first block's scores hide most of
+  // the load (requested before the score product instead, the kernel is 1-4 % slower: more
+  // scalar registers spilled).  All 32 requested a tile ahead do not fit the scalar registers.
+  constexpr int kLaneWordsPerBlock = kLaneWordsPerTile / 2;
+  [[maybe_unused]] uint64_t lane_words[2][LANES ? kLaneWordsPerBlock : 1];
+  auto load_lane_words = [&](int tile, int key_block) {
+    if constexpr (LANES) {
+      typedef const __attribute__((address_space(4))) uint64_t* UniformWords;
+      const uint64_t* at = p.mask_lanes + batch * p.mask_lanes_stride_b + head * p.mask_lanes_stride_h +
+                           lane_word_offset(bx * 4 + wave, p.n_kb, tile) + key_block * kLaneWordsPerBlock;
+      const UniformWords words = (UniformWords)(reinterpret_cast<uintptr_t>(at));
+#pragma unroll
+      for (int slot = 0; slot < kLaneWordsPerBlock; ++slot) lane_words[key_block][slot] = words[slot];
+    }
+  };
+
   // Mask elements of a full tile, requested before the next tile's copies.  Vector
   // memory operations complete in order: a mask load issued after the copies can only
   // be consumed once they have landed, which stalls the softmax of this tile on the
@@ -482,7 +518,7 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void attention_kernel(cons
   // changes FP32 rounding only, while the output accumulators are rescaled on
   // a handful of tiles instead of on every new maximum.
   constexpr float kRescaleSlack = 8.0f;
-  auto softmax_tile = [&](auto last_tag, int it, int tile, float ks0, float ks1, v16i (&s)[RB],
+  auto softmax_tile = [&](auto last_tag, int it, int tile, int next_tile, float ks0, float ks1, v16i (&s)[RB],
                           v4i (&pk)[RB]) -> float {
     constexpr bool LAST = decltype(last_tag)::value;
     // K scale groups of this lane: keys 8b+4*half+r, group (key % 8) / 2 = 2*half + r/2.
@@ -605,6 +641,35 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void attention_kernel(cons
           biased_scores(std::true_type{});
         } else {
           biased_scores(std::false_type{});
+        }
+      } else if constexpr (LANES) {
+        // Lane words: bit l of word (rb, i) says whether lane l keeps score (rb, i); keys past
+        // the end and rows past the last query have no bit set, so the last tile needs nothing else.
+        auto lane_masked_scores = [&](auto diagonal_tag, auto block_tag) {
+          constexpr bool DIAGONAL = decltype(diagonal_tag)::value;
+          constexpr int rb = decltype(block_tag)::value;
+#pragma unroll
+          for (int i = 0; i < 16; ++i) {
+            bool keep = __builtin_amdgcn_inverse_ballot_w64(lane_words[rb][i]);
+            if constexpr (DIAGONAL) keep = keep && key0 + rb * 32 + (i >> 2) * 8 + (i & 3) <= query;
+            const float scaled = score_value(s[rb][i]) * ((i & 2) ? sc1 : sc0);
+            const float value = keep ? scaled : neg_inf;
+            s[rb][i] = __float_as_int(value);
+            mx = __builtin_fmaxf(mx, value);
+          }
+        };
+        auto lane_pass = [&](auto diagonal_tag) {
+          load_lane_words(tile, 1);
+          __builtin_amdgcn_sched_barrier(0);
+          lane_masked_scores(diagonal_tag, std::integral_constant<int, 0>{});
+          lane_masked_scores(diagonal_tag, std::integral_constant<int, 1>{});
+          __builtin_amdgcn_sched_barrier(0);
+          if (!LAST) load_lane_words(next_tile, 0);
+        };
+        if (on_diagonal) {
+          lane_pass(std::true_type{});
+        } else {
+          lane_pass(std::false_type{});
         }
       } else {
         // DT: mask element type (-1: none, only the causal / key-range tests);
@@ -880,6 +945,7 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void attention_kernel(cons
     issue_tile(tile, 0);
     // The last listed tile reads its mask elements directly (it may be partial).
     if (n_it > 1) issue_mask_tile(tile, 0);
+    load_lane_words(tile, 0);
     float ks0 = ks_base[tile * 4 + 2 * half];
     float ks1 = ks_base[tile * 4 + 2 * half + 1];
     for (int it = 0; it < n_it - 1; ++it) {
@@ -912,7 +978,7 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void attention_kernel(cons
         __builtin_amdgcn_sched_barrier(0);
       }
       __builtin_amdgcn_s_setprio(2);
-      const float t_scale = softmax_tile(std::false_type{}, it, tile, ks0, ks1, s, pk);
+      const float t_scale = softmax_tile(std::false_type{}, it, tile, next_tile, ks0, ks1, s, pk);
       __builtin_amdgcn_s_setprio(1);
       if constexpr (LATE_COPIES) {
         __builtin_amdgcn_sched_barrier(0);
@@ -939,7 +1005,7 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void attention_kernel(cons
     __syncthreads();
     load_k_fragments(lds + stage * Shape::kStageBytes, 0, k_first);
     score_tile(stage, k_first, s);
-    const float t_scale = softmax_tile(std::true_type{}, n_it - 1, tile, ks0, ks1, s, pk);
+    const float t_scale = softmax_tile(std::true_type{}, n_it - 1, tile, tile, ks0, ks1, s, pk);
     load_seed_pair(stage, 0, seed);
     load_v_pair(stage, 0, 0, v_first);
     value_tile(stage, pk, seed, v_first, t_scale);

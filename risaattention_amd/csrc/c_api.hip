@@ -147,7 +147,7 @@ extern "C" {
 
 const char* risa_last_error(void) { return risa::last_error_storage().c_str(); }
 
-int risa_abi_version(void) { return 1; }
+int risa_abi_version(void) { return 2; }
 
 int risa_quantize_qk(const void* q, void* q_int8, float* q_scale, const void* k, void* k_int8,
                      float* k_scale, int batch, int q_heads, int q_len, int kv_heads, int k_len,
@@ -256,7 +256,8 @@ int risa_attention(const void* q_int8, const void* k_int8, const void* v_int8, v
                    const int32_t* sparse_row_offsets, const int32_t* sparse_block_indices,
                    float* block_mass, int is_causal, float* lse, const int32_t* key_mask_tiles,
                    const float* key_bias, int64_t key_bias_stride_b, int64_t key_bias_stride_h,
-                   void* stream) {
+                   const uint64_t* mask_lanes, int64_t mask_lanes_stride_b,
+                   int64_t mask_lanes_stride_h, void* stream) {
   using risa::fail;
   if (out_dtype != 1 && out_dtype != 2)
     return fail("risa_attention: output dtype code must be 1 (fp16) or 2 (bf16)");
@@ -305,6 +306,11 @@ int risa_attention(const void* q_int8, const void* k_int8, const void* v_int8, v
   a.key_bias = key_bias;
   a.key_bias_stride_b = key_bias_stride_b;
   a.key_bias_stride_h = key_bias_stride_h;
+  if (mask_lanes != nullptr && mask == nullptr)
+    return fail("risa_attention: lane words go with the boolean mask they were made from");
+  a.mask_lanes = mask_lanes;
+  a.mask_lanes_stride_b = mask_lanes_stride_b;
+  a.mask_lanes_stride_h = mask_lanes_stride_h;
   return risa::launch_attention(a, static_cast<hipStream_t>(stream));
 }
 
@@ -347,6 +353,27 @@ int risa_prepare_key_bias(const void* mask, float* bias, int batch, int heads, i
                                stride_h, stride_k, mask_dtype, static_cast<hipStream_t>(stream));
 }
 
+size_t risa_mask_lanes_bytes(int mask_dtype, int cta_k, int64_t mask_stride_q, int64_t mask_stride_k,
+                             int batch, int q_heads, int mask_batch, int mask_heads, int q_len,
+                             int k_len) {
+  if (mask_dtype != risa::kBool || cta_k != 64 || mask_stride_q == 0 || mask_stride_k != 1) return 0;
+  if (batch <= 0 || q_heads <= 0 || mask_batch <= 0 || mask_heads <= 0 || q_len <= 0 || k_len <= 0) return 0;
+  // The conversion reads the mask once; it pays when several heads then share the words.
+  if (static_cast<int64_t>(batch) * q_heads < int64_t{4} * mask_batch * mask_heads) return 0;
+  return risa::mask_lane_words(mask_batch, mask_heads, q_len, k_len) * sizeof(uint64_t);
+}
+
+int risa_prepare_mask_lanes(const void* mask, uint64_t* lanes, int mask_batch, int mask_heads,
+                            int q_len, int k_len, int64_t stride_b, int64_t stride_h,
+                            int64_t stride_q, void* stream) {
+  if (mask == nullptr || lanes == nullptr || mask_batch <= 0 || mask_heads <= 0 || q_len <= 0 || k_len <= 0)
+    return risa::fail("risa_prepare_mask_lanes: bad extents");
+  if (!aligned(lanes, 8)) return risa::fail("risa_prepare_mask_lanes: lane words must be 8-byte aligned");
+  return risa::launch_mask_lanes(mask, lanes, mask_batch, mask_heads, q_len, k_len,
+                                 mask_batch > 1 ? stride_b : 0, mask_heads > 1 ? stride_h : 0, stride_q,
+                                 static_cast<hipStream_t>(stream));
+}
+
 int risa_lse_shift(const void* q, const void* k, const int32_t* anchors, float* out, int batch,
                    int q_heads, int kv_heads, int q_len, int head_dim, int64_t q_stride_b,
                    int64_t q_stride_h, int64_t q_stride_n, int64_t k_stride_b, int64_t k_stride_h,
@@ -365,11 +392,11 @@ namespace {
 // Sections of the risa_sdpa workspace, each aligned to 256 bytes.
 struct SdpaLayout {
   size_t q_codes, k_codes, v_codes, q_scale, k_scale, v_scale, v_center, tile_sum, anchors,
-      v_workspace, v_workspace_bytes, key_bias, key_tiles, bytes;
+      v_workspace, v_workspace_bytes, key_bias, key_tiles, mask_lanes, bytes;
 };
 
 SdpaLayout sdpa_layout(int batch, int q_heads, int q_len, int kv_heads, int k_len, int head_dim,
-                       int cta_k, bool affine, bool key_only_mask) {
+                       int cta_k, bool affine, bool key_only_mask, size_t mask_lanes_bytes) {
   SdpaLayout l{};
   size_t offset = 0;
   auto take = [&](size_t bytes) {
@@ -394,6 +421,7 @@ SdpaLayout sdpa_layout(int batch, int q_heads, int q_len, int kv_heads, int k_le
   l.v_workspace = take(l.v_workspace_bytes);
   l.key_bias = key_only_mask ? take(static_cast<size_t>(batch) * q_heads * padded * 4) : 0;
   l.key_tiles = key_only_mask ? take(static_cast<size_t>(batch) * q_heads * (tiles + 1) * 4) : 0;
+  l.mask_lanes = mask_lanes_bytes != 0 ? take(mask_lanes_bytes) : 0;
   l.bytes = offset;
   return l;
 }
@@ -403,12 +431,17 @@ SdpaLayout sdpa_layout(int batch, int q_heads, int q_len, int kv_heads, int k_le
 extern "C" {
 
 size_t risa_sdpa_workspace_bytes(int batch, int q_heads, int q_len, int kv_heads, int k_len,
-                                 int head_dim, int cta_k, int midpoint_affine, int key_only_mask) {
+                                 int head_dim, int cta_k, int midpoint_affine, int mask_dtype,
+                                 int64_t mask_stride_q, int64_t mask_stride_k, int mask_batch,
+                                 int mask_heads) {
   if (batch <= 0 || q_heads <= 0 || q_len <= 0 || kv_heads <= 0 || k_len <= 0 || head_dim <= 0 ||
       (cta_k != 64 && cta_k != 128))
     return 0;
+  const bool key_only = mask_dtype >= 0 && mask_stride_q == 0;
+  const size_t lanes = risa_mask_lanes_bytes(mask_dtype, cta_k, mask_stride_q, mask_stride_k, batch,
+                                             q_heads, mask_batch, mask_heads, q_len, k_len);
   return sdpa_layout(batch, q_heads, q_len, kv_heads, k_len, head_dim, cta_k, midpoint_affine != 0,
-                     key_only_mask != 0)
+                     key_only, lanes)
       .bytes;
 }
 
@@ -427,8 +460,16 @@ int risa_sdpa(const void* q, const void* k, const void* v, void* out, void* work
       (cta_k != 64 && cta_k != 128))
     return fail("risa_sdpa: extents must be positive and cta_k 64 or 128");
   const bool key_only = mask != nullptr && mask_stride_q == 0;
+  if (mask != nullptr) {
+    if (mask_batch != 1 && mask_batch != batch) return fail("risa_sdpa: mask batch extent");
+    if (mask_heads != 1 && mask_heads != q_heads) return fail("risa_sdpa: mask head extent");
+  }
+  const size_t lanes_bytes =
+      mask == nullptr ? 0
+                      : risa_mask_lanes_bytes(mask_dtype, cta_k, mask_stride_q, mask_stride_k, batch,
+                                              q_heads, mask_batch, mask_heads, q_len, k_len);
   const SdpaLayout l = sdpa_layout(batch, q_heads, q_len, kv_heads, k_len, head_dim, cta_k,
-                                   midpoint_affine != 0, key_only);
+                                   midpoint_affine != 0, key_only, lanes_bytes);
   if (workspace == nullptr || !aligned(workspace, 256) || workspace_bytes < l.bytes)
     return fail("risa_sdpa: workspace must be 256-byte aligned and hold risa_sdpa_workspace_bytes");
   auto* base = static_cast<unsigned char*>(workspace);
@@ -462,9 +503,19 @@ int risa_sdpa(const void* q, const void* k, const void* v, void* out, void* work
   const float* key_bias = nullptr;
   const int32_t* key_tiles = nullptr;
   int64_t bias_stride_b = 0, bias_stride_h = 0;
+  const uint64_t* mask_lanes = nullptr;
+  int64_t lanes_stride_b = 0, lanes_stride_h = 0;
+  if (lanes_bytes != 0) {
+    auto* words = reinterpret_cast<uint64_t*>(base + l.mask_lanes);
+    status = risa_prepare_mask_lanes(mask, words, mask_batch, mask_heads, q_len, k_len, mask_stride_b,
+                                     mask_stride_h, mask_stride_q, stream);
+    if (status != 0) return status;
+    mask_lanes = words;
+    const int64_t plane = static_cast<int64_t>(risa::mask_lane_words(1, 1, q_len, k_len));
+    lanes_stride_h = mask_heads > 1 ? plane : 0;
+    lanes_stride_b = mask_batch > 1 ? plane * mask_heads : 0;
+  }
   if (key_only) {
-    if (mask_batch != 1 && mask_batch != batch) return fail("risa_sdpa: mask batch extent");
-    if (mask_heads != 1 && mask_heads != q_heads) return fail("risa_sdpa: mask head extent");
     auto* bias = reinterpret_cast<float*>(base + l.key_bias);
     status = risa_prepare_key_bias(mask, bias, mask_batch, mask_heads, k_len, padded,
                                    mask_batch > 1 ? mask_stride_b : 0,
@@ -488,7 +539,8 @@ int risa_sdpa(const void* q, const void* k, const void* v, void* out, void* work
                         mask_stride_q, mask_stride_k, mask_dtype, cta_k, batch, q_len, k_len,
                         q_heads, kv_heads, head_dim, out_stride_b, out_stride_n, out_stride_h,
                         sm_scale, output_dtype, sparse_row_offsets, sparse_block_indices, nullptr,
-                        is_causal, nullptr, key_tiles, key_bias, bias_stride_b, bias_stride_h, stream);
+                        is_causal, nullptr, key_tiles, key_bias, bias_stride_b, bias_stride_h,
+                        mask_lanes, lanes_stride_b, lanes_stride_h, stream);
 }
 
 }  // extern "C"

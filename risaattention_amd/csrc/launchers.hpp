@@ -81,6 +81,8 @@ struct AttentionArgs {
   const int32_t* key_mask_tiles;
   const float* key_bias;  // [Bm,Hm,padded] from launch_key_bias, or null
   int64_t key_bias_stride_b, key_bias_stride_h;
+  const uint64_t* mask_lanes;  // lane words from launch_mask_lanes, or null
+  int64_t mask_lanes_stride_b, mask_lanes_stride_h;  // in words
 };
 int launch_attention(const AttentionArgs& args, hipStream_t stream);
 
@@ -105,6 +107,12 @@ int launch_key_mask_tiles(const void* mask, int32_t* tiles, int batch, int heads
 // Q/K/V preparation in two launches (short sequences, no permutation).
 bool can_prepare_fused(const QkArgs& qk, const ValueArgs& v);
 int launch_prepare_fused(const QkArgs& qk, const ValueArgs& v, hipStream_t stream);
+
+// Lane words of a boolean mask with 64-key tiles: [batch, heads, ceil(q_len/128)*4,
+// ceil(k_len/64), 32] 64-bit words, batch and heads being the mask's own extents.
+size_t mask_lane_words(int batch, int heads, int q_len, int k_len);
+int launch_mask_lanes(const void* mask, uint64_t* lanes, int batch, int heads, int q_len, int k_len,
+                      int64_t stride_b, int64_t stride_h, int64_t stride_q, hipStream_t stream);
 
 int launch_key_bias(const void* mask, float* bias, int batch, int heads, int length, int padded,
                     int64_t stride_b, int64_t stride_h, int64_t stride_k, int dtype,

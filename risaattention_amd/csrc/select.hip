@@ -214,7 +214,110 @@ __global__ __launch_bounds__(256) void key_bias_kernel(const void* __restrict__ 
   bias[(static_cast<int64_t>(blockIdx.z) * gridDim.y + blockIdx.y) * padded + key] = value;
 }
 
+
+// Lane words of a boolean mask (the form kMaskLanes of the attention kernel reads): for
+// every block of 32 queries and 64-key tile, 32 words; bit l of word 16*rb + i is the mask
+// element of query 32*block + l % 32 and key 64*tile + 32*rb + 8*(i / 4) + 4*(l / 32) + i % 4,
+// which is score (rb, i) of lane l in the attention kernel.  Rows past the last query and
+// keys past the last key have no bit set.
+//
+// grid (groups of 16 tiles, blocks of 32 queries, batch*heads of the mask), 256 threads: a
+// wavefront takes four consecutive key tiles of one query block (256 mask bytes per row, all
+// requested before the first is used).  Lane (row, half) reads, per tile and 32-key block,
+// the sixteen elements at keys 16*half .. 16*half+15 of the block (one 16-byte load when
+// ALIGNED): the eight-key groups b4 = 2*half and 2*half+1, both four-key halves of each.
+// A vote over element (b', h', r) of every lane therefore holds, in its low 32 bits, the
+// rows' decisions for group b' and, in its high 32 bits, those for group 2+b', four-key
+// half h' each; a lane word wants the two halves h' of one group side by side, which is a
+// regrouping of 32-bit scalar registers.  Lane s keeps word s, so the 32 words of a tile
+// leave in one 256-byte store.
+constexpr int kLaneTilesPerWave = 4;
+// A wave-uniform 32-bit value written into one lane of a vector register.
+__device__ __forceinline__ void write_lane(uint32_t& target, uint32_t uniform_value, int lane_index) {
+  asm("v_writelane_b32 %0, %1, %2" : "+v"(target) : "s"(uniform_value), "n"(lane_index));
+}
+template <bool ALIGNED>
+__global__ __launch_bounds__(256) void mask_lanes_kernel(const uint8_t* __restrict__ mask,
+                                                         uint64_t* __restrict__ lanes, int heads,
+                                                         int q_len, int k_len, int key_tiles,
+                                                         int query_waves, int64_t stride_b,
+                                                         int64_t stride_h, int64_t stride_q) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int query_wave = blockIdx.y, plane = blockIdx.z;
+  const int row = query_wave * 32 + (lane & 31), half = lane >> 5;
+  const bool row_ok = row < q_len;
+  const uint8_t* row_mask = mask + (plane / heads) * stride_b + (plane % heads) * stride_h +
+                            static_cast<int64_t>(row_ok ? row : q_len - 1) * stride_q;
+  uint64_t* out = lanes + (static_cast<int64_t>(plane) * query_waves + query_wave) * key_tiles * 32;
+  const int first_tile = (blockIdx.x * 4 + wave) * kLaneTilesPerWave;
+  typedef uint32_t v4u __attribute__((ext_vector_type(4)));
+  v4u chunk[kLaneTilesPerWave][2];
+#pragma unroll
+  for (int t = 0; t < kLaneTilesPerWave; ++t) {
+#pragma unroll
+    for (int rb = 0; rb < 2; ++rb) {
+      const int key = (first_tile + t) * 64 + rb * 32 + half * 16;
+      v4u words = {0u, 0u, 0u, 0u};
+      if (ALIGNED && key + 15 < k_len) {
+        words = *reinterpret_cast<const v4u*>(row_mask + key);
+      } else {
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+          if (key + j < k_len && row_mask[key + j] != 0) words[j >> 2] |= 1u << (8 * (j & 3));
+        }
+      }
+      if (!row_ok) words = v4u{0u, 0u, 0u, 0u};
+      chunk[t][rb] = words;
+    }
+  }
+#pragma unroll
+  for (int t = 0; t < kLaneTilesPerWave; ++t) {
+    if (first_tile + t >= key_tiles) break;  // wave-uniform
+    // word s of the tile goes to lane s, 32 bits at a time, straight from the scalar registers
+    uint32_t mine_low = 0, mine_high = 0;
+#pragma unroll
+    for (int rb = 0; rb < 2; ++rb) {
+#pragma unroll
+      for (int group = 0; group < 2; ++group) {  // b'
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const uint64_t first = __ballot(((chunk[t][rb][group * 2] >> (8 * r)) & 0xffu) != 0);
+          const uint64_t second = __ballot(((chunk[t][rb][group * 2 + 1] >> (8 * r)) & 0xffu) != 0);
+          const int low_slot = rb * 16 + group * 4 + r;        // b4 = b'
+          const int high_slot = rb * 16 + (2 + group) * 4 + r;  // b4 = 2 + b'
+          write_lane(mine_low, static_cast<uint32_t>(first), low_slot);
+          write_lane(mine_high, static_cast<uint32_t>(second), low_slot);
+          write_lane(mine_low, static_cast<uint32_t>(first >> 32), high_slot);
+          write_lane(mine_high, static_cast<uint32_t>(second >> 32), high_slot);
+        }
+      }
+    }
+    const uint64_t mine = mine_low | (static_cast<uint64_t>(mine_high) << 32);
+    if (lane < 32) out[static_cast<int64_t>(first_tile + t) * 32 + lane] = mine;
+  }
+}
+
 }  // namespace
+
+size_t mask_lane_words(int batch, int heads, int q_len, int k_len) {
+  const size_t query_waves = (static_cast<size_t>(q_len) + 127) / 128 * 4;
+  const size_t key_tiles = (static_cast<size_t>(k_len) + 63) / 64;
+  return static_cast<size_t>(batch) * heads * query_waves * key_tiles * 32;
+}
+
+int launch_mask_lanes(const void* mask, uint64_t* lanes, int batch, int heads, int q_len, int k_len,
+                      int64_t stride_b, int64_t stride_h, int64_t stride_q, hipStream_t stream) {
+  const int query_waves = (q_len + 127) / 128 * 4;
+  const int key_tiles = (k_len + 63) / 64;
+  if (query_waves > 65535 || static_cast<int64_t>(batch) * heads > 65535)
+    return fail("risa_prepare_mask_lanes: more query blocks or mask planes than one launch covers");
+  const dim3 grid((key_tiles + 4 * kLaneTilesPerWave - 1) / (4 * kLaneTilesPerWave), query_waves, batch * heads);
+  const bool aligned = reinterpret_cast<uintptr_t>(mask) % 16 == 0 && ((stride_b | stride_h | stride_q) & 15) == 0;
+  auto kernel = aligned ? mask_lanes_kernel<true> : mask_lanes_kernel<false>;
+  kernel<<<grid, 256, 0, stream>>>(static_cast<const uint8_t*>(mask), lanes, heads, q_len, k_len,
+                                   key_tiles, query_waves, stride_b, stride_h, stride_q);
+  return check_launch("risa_prepare_mask_lanes");
+}
 
 int launch_key_bias(const void* mask, float* bias, int batch, int heads, int length, int padded,
                     int64_t stride_b, int64_t stride_h, int64_t stride_k, int dtype,

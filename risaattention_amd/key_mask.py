@@ -36,6 +36,36 @@ def prepare_key_bias(mask, key_block_size):
     return bias, (bias.stride(0) if batch > 1 else 0), (bias.stride(1) if heads > 1 else 0)
 
 
+def prepare_mask_lanes(mask, key_block_size):
+    """Lane words of a boolean mask several heads share, ``(words, stride_b, stride_h)`` or ``None``.
+
+    ``mask`` is the expanded ``[B,Hq,Lq,Lk]`` view.  The library decides whether the form
+    applies (boolean, query-dependent, unit key stride, 64-key tiles, at least four
+    (batch, head) pairs per mask plane) by returning the size of the buffer or 0; the
+    attention kernel then takes one 64-lane word per score from scalar registers instead
+    of reading mask elements.
+    """
+    if mask is None or mask.dtype != torch.bool:
+        return None
+    batch, q_heads, q_len, k_len = mask.shape
+    planes_b = batch if mask.stride(0) != 0 else 1
+    planes_h = q_heads if mask.stride(1) != 0 else 1
+    lib = native.library()
+    size = lib.risa_mask_lanes_bytes(MASK_DTYPE_CODES[mask.dtype], key_block_size, mask.stride(2),
+                                     mask.stride(3), batch, q_heads, planes_b, planes_h, q_len, k_len)
+    if size == 0:
+        return None
+    words = torch.empty(size // 8, device=mask.device, dtype=torch.int64)
+    native.check(
+        lib.risa_prepare_mask_lanes(
+            mask.data_ptr(), words.data_ptr(), planes_b, planes_h, q_len, k_len,
+            mask.stride(0), mask.stride(1), mask.stride(2), native.current_stream(mask.device),
+        )
+    )
+    plane = words.numel() // (planes_b * planes_h)
+    return words, (plane * planes_h if planes_b > 1 else 0), (plane if planes_h > 1 else 0)
+
+
 def prepare_key_mask_tiles(mask, key_block_size, query_length, scale, is_causal):
     """int32 [B,Hq,tiles+1] (active tile ids, then the count) or None.
 

@@ -55,13 +55,18 @@ SIGNATURES = {
         + [_c_int] * 8
         + [_c_i64] * 3
         + [_c_f32, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr]
-        + [_c_ptr, _c_i64, _c_i64, _c_ptr],
+        + [_c_ptr, _c_i64, _c_i64, _c_ptr, _c_i64, _c_i64, _c_ptr],
+    ),
+    "risa_mask_lanes_bytes": (_c_size, [_c_int, _c_int, _c_i64, _c_i64] + [_c_int] * 6),
+    "risa_prepare_mask_lanes": (
+        _c_int,
+        [_c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_i64, _c_i64, _c_i64, _c_ptr],
     ),
     "risa_prepare_key_bias": (
         _c_int,
         [_c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_i64, _c_i64, _c_i64, _c_int, _c_ptr],
     ),
-    "risa_sdpa_workspace_bytes": (_c_size, [_c_int] * 9),
+    "risa_sdpa_workspace_bytes": (_c_size, [_c_int] * 9 + [_c_i64, _c_i64, _c_int, _c_int]),
     "risa_sdpa": (
         _c_int,
         [_c_ptr] * 5 + [_c_size] + [_c_int] * 7 + [_c_i64] * 12 + [_c_f32, _c_int, _c_int, _c_int]

@@ -407,3 +407,94 @@ def test_concurrent_host_threads_on_their_own_streams(risa):
         thread.join(timeout=100)
     assert not any(thread.is_alive() for thread in threads)
     assert not failures, failures
+
+
+def expected_lane_words(mask, q_len, k_len):
+    """Lane words of a [planes, q_len, k_len] boolean array, element by element: word
+    (plane, w, t, 16*rb + i) has bit l set when query 32*w + l % 32 may attend to key
+    64*t + 32*rb + 8*(i // 4) + 4*(l // 32) + i % 4."""
+    planes = mask.shape[0]
+    query_waves = -(-q_len // 128) * 4
+    key_tiles = -(-k_len // 64)
+    padded = np.zeros((planes, query_waves * 32, key_tiles * 64), dtype=bool)
+    padded[:, :q_len, :k_len] = mask
+    lane = np.arange(64)
+    slot = np.arange(32)
+    rows = lane % 32                                           # [64]
+    keys = (slot[:, None] // 16) * 32 + ((slot[:, None] % 16) // 4) * 8 + (lane[None, :] // 32) * 4 + slot[:, None] % 4
+    blocks = padded.reshape(planes, query_waves, 32, key_tiles, 64)
+    bits = blocks[:, :, rows[None, :], :, keys]                # [slot, lane, planes, waves, tiles]
+    bits = np.moveaxis(bits, (0, 1), (3, 4))                   # [planes, waves, tiles, slot, lane]
+    weights = (np.uint64(1) << lane.astype(np.uint64))
+    return (bits.astype(np.uint64) * weights).sum(-1, dtype=np.uint64)
+
+
+@pytest.mark.parametrize("q_len,k_len,aligned", [(300, 704, True), (300, 700, False), (129, 263, False), (64, 64, True)])
+def test_lane_words_of_a_boolean_mask(risa, q_len, k_len, aligned):
+    """The conversion a boolean mask shared by several heads goes through, bit for bit."""
+    from risaattention_amd.key_mask import prepare_mask_lanes
+
+    generator = torch.Generator().manual_seed(q_len + k_len)
+    planes = torch.rand((2, 1, q_len, k_len), generator=generator) > 0.5
+    planes[1, 0, 5] = False
+    mask = planes.cuda()
+    assert (mask.stride(2) % 16 == 0) == aligned  # rows the conversion can read 16 bytes at a time
+    words, stride_b, stride_h = prepare_mask_lanes(mask.expand(2, 8, q_len, k_len), 64)
+    expected = expected_lane_words(planes[:, 0].numpy(), q_len, k_len)
+    assert stride_h == 0 and stride_b == expected[0].size
+    assert np.array_equal(words.cpu().numpy().view(np.uint64).reshape(expected.shape), expected)
+    # one plane per head is not worth converting, nor is any other dtype or tile size
+    assert prepare_mask_lanes(mask.expand(2, 3, q_len, k_len), 64) is None
+    assert prepare_mask_lanes(mask.expand(2, 8, q_len, k_len), 128) is None
+    assert prepare_mask_lanes(mask.expand(2, 8, q_len, k_len).float(), 64) is None
+
+
+@pytest.mark.parametrize("dim", [64, 128, 256])
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("q_len,k_len", [(330, 400), (257, 263)])
+def test_shared_boolean_mask_equals_the_mask_per_head(risa, dim, causal, q_len, k_len):
+    """A boolean mask that broadcasts over heads is applied from lane words; the same mask
+    materialised per head is read element by element.  Same decisions, same arithmetic:
+    outputs and LSE are equal bit for bit, and both match the oracle."""
+    heads = 8
+    q = seeded((2, heads, q_len, dim), torch.float16, 171)
+    k = seeded((2, 2, k_len, dim), torch.float16, 172)
+    v = seeded((2, 2, k_len, dim), torch.float16, 173)
+    generator = torch.Generator().manual_seed(174)
+    shared = (torch.rand((2, 1, q_len, k_len), generator=generator) > 0.4).cuda()
+    shared[0, 0, 129] = False  # a fully hidden row
+    shared[1, 0, :, 64:128] = False  # a fully hidden key tile
+    per_head = shared.expand(2, heads, q_len, k_len).contiguous()
+    out, lse = risa.int8_attention(q, k, v, attn_mask=shared, is_causal=causal, return_lse=True)
+    out_heads, lse_heads = risa.int8_attention(q, k, v, attn_mask=per_head, is_causal=causal, return_lse=True)
+    assert torch.equal(out, out_heads)
+    assert torch.equal(lse, lse_heads)
+    assert torch.equal(out, risa.int8_attention(q, k, v, attn_mask=shared, is_causal=causal))  # the one-call route
+    prepared = oracle_prequantize(q[:1, :2], k[:1, :1], v[:1, :1], attn_mask=shared[:1], is_causal=causal,
+                                  return_lse=True)
+    expected, expected_lse, _ = oracle_pipeline.attend(prepared, return_lse=True)
+    assert relative_l2(to_numpy(out[:1, :2]), expected) < TOLERANCE
+    finite = np.isfinite(expected_lse)
+    assert np.array_equal(np.isfinite(to_numpy(lse[:1, :2])), finite)
+    assert relative_l2(to_numpy(lse[:1, :2])[finite], expected_lse[finite]) < TOLERANCE
+
+
+def test_shared_boolean_mask_in_the_sparse_path(risa):
+    """Pattern construction (capturing kernel) and reuse (tile lists) under lane words
+    give what they give under the mask read per head."""
+    heads, q_len, k_len, dim = 8, 512, 1500, 128
+    q = seeded((1, heads, q_len, dim), torch.bfloat16, 181)
+    k = seeded((1, 2, k_len, dim), torch.bfloat16, 182)
+    v = seeded((1, 2, k_len, dim), torch.bfloat16, 183)
+    generator = torch.Generator().manual_seed(184)
+    shared = (torch.rand((1, 1, q_len, k_len), generator=generator) > 0.3).cuda()
+    per_head = shared.expand(1, heads, q_len, k_len).contiguous()
+    out, pattern = risa.construct_sparse_int8_attention(q, k, v, theta=0.9, attn_mask=shared)
+    out_heads, pattern_heads = risa.construct_sparse_int8_attention(q, k, v, theta=0.9, attn_mask=per_head)
+    assert torch.equal(out, out_heads)
+    assert torch.equal(pattern.row_offsets, pattern_heads.row_offsets)
+    assert torch.equal(pattern.block_indices, pattern_heads.block_indices)
+    assert 0.05 < pattern.sparsity < 0.95
+    reuse = risa.sparse_int8_attention(q, k, v, pattern, attn_mask=shared)
+    reuse_heads = risa.sparse_int8_attention(q, k, v, pattern_heads, attn_mask=per_head)
+    assert torch.equal(reuse, reuse_heads)
