@@ -245,15 +245,16 @@ int risa_prepare_key_bias(const void* mask, float* bias, int batch, int heads, i
  * is set past the last query or key.  The attention kernel applies one word per score
  * from scalar registers.  risa_mask_lanes_bytes returns the size of the buffer, or 0
  * when the form does not apply or does not pay: the mask is not boolean, the tiles are
- * not 64 keys, the key stride is not 1, the query stride is 0, or fewer than four
+ * not 64 keys, the head dim is 256 (that kernel holds its scores in another layout), the
+ * key stride is not 1, the query stride is 0, or fewer than four
  * (batch, head) pairs share each mask plane (the conversion reads the mask once, the
  * attention kernel would read it once per pair).  No counterpart in the reference, whose
  * kernel reads the mask per score (csrc/kernels/attention_masks.cuh:27-164); the
  * decisions are the ones it takes.
  */
-size_t risa_mask_lanes_bytes(int mask_dtype, int cta_k, int64_t mask_stride_q, int64_t mask_stride_k,
-                             int batch, int q_heads, int mask_batch, int mask_heads, int q_len,
-                             int k_len);
+size_t risa_mask_lanes_bytes(int mask_dtype, int head_dim, int cta_k, int64_t mask_stride_q,
+                             int64_t mask_stride_k, int batch, int q_heads, int mask_batch,
+                             int mask_heads, int q_len, int k_len);
 int risa_prepare_mask_lanes(const void* mask, uint64_t* lanes, int mask_batch, int mask_heads,
                             int q_len, int k_len, int64_t stride_b, int64_t stride_h,
                             int64_t stride_q, void* stream);

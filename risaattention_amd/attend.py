@@ -145,7 +145,7 @@ def launch_attention(*, q_codes, k_codes, v_codes, output, q_scale, k_scale, v_s
     sums = ensure_tile_sums(v_codes, v_tile_sum, batch * kv_heads, dim, cta_k)
     key_bias = prepare_key_bias(attn_mask, cta_k)
     bias_args = (None, 0, 0) if key_bias is None else (key_bias[0].data_ptr(), key_bias[1], key_bias[2])
-    mask_lanes = prepare_mask_lanes(attn_mask, cta_k)
+    mask_lanes = prepare_mask_lanes(attn_mask, cta_k, dim)
     lane_args = (None, 0, 0) if mask_lanes is None else (mask_lanes[0].data_ptr(), mask_lanes[1], mask_lanes[2])
     out_b = output.stride(0) if batch > 1 else q_heads * q_len * dim
     out_n = output.stride(2) if q_len > 1 else dim

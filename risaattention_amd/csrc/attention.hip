@@ -12,8 +12,9 @@ namespace risa {
 
 template <> int launch_attention_variant<64>(const KernelParams&, int, bool, bool, bool, int, hipStream_t);
 template <> int launch_attention_variant<128>(const KernelParams&, int, bool, bool, bool, int, hipStream_t);
-template <> int launch_attention_variant<256>(const KernelParams&, int, bool, bool, bool, int, hipStream_t);
 int launch_attention_narrow(const KernelParams& p, int head_dim, int cta_k, hipStream_t stream);
+int launch_attention_wide_head(const KernelParams& p, int cta_k, bool fast, bool indexed, bool capture,
+                               int mask_mode, hipStream_t stream);
 int narrow_attention_limit();
 
 namespace {
@@ -128,7 +129,7 @@ int launch_attention(const AttentionArgs& a, hipStream_t stream) {
         mask_mode = kMaskStaged;
       }
     }
-    if (a.mask_lanes != nullptr) {
+    if (a.mask_lanes != nullptr && a.head_dim <= 128) {  // head dim 256 reads the mask itself
       if (a.mask_dtype != kBool || a.cta_k != 64 || a.mask_stride_q == 0)
         return fail("risa_attention: lane words go with a query-dependent boolean mask and 64-key tiles");
       if (reinterpret_cast<uintptr_t>(a.mask_lanes) % 8 != 0)
@@ -180,9 +181,9 @@ int launch_attention(const AttentionArgs& a, hipStream_t stream) {
 
   // A launch that cannot give every compute unit more than one workgroup runs the
   // raw-score path with sixteen queries per wavefront (two wavefronts per SIMD).  So does
-  // every launch with head dim 256: thirty-two queries of 256 channels per wavefront need
-  // some 380 registers, which leaves one wavefront per SIMD (1200 against 1630
-  // dense-equivalent TOPS at N=16K).
+  // every launch with head dim 256, masked, causal and capturing ones included: thirty-two
+  // queries of 256 channels per wavefront need some 380 registers, which leaves one
+  // wavefront per SIMD (1200 against 1630 dense-equivalent TOPS at N=16K).
   const int64_t workgroups = static_cast<int64_t>(p.n_qb) * a.q_heads * a.batch;
   const bool narrow = fast && p.index_mode != 2 && !capture &&
                       (a.head_dim > 128 || workgroups <= narrow_attention_limit());
@@ -195,7 +196,7 @@ int launch_attention(const AttentionArgs& a, hipStream_t stream) {
   else if (a.head_dim == 128)
     status = launch_attention_variant<128>(p, a.cta_k, fast, indexed, capture, mask_mode, stream);
   else if (a.head_dim == 256)
-    status = launch_attention_variant<256>(p, a.cta_k, fast, indexed, capture, mask_mode, stream);
+    status = launch_attention_wide_head(p, a.cta_k, fast, indexed, capture, mask_mode, stream);
   else
     return fail("risa_attention: unsupported head_dim");
   if (status != 0) return status;

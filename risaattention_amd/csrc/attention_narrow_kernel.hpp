@@ -46,15 +46,35 @@ template <int ROWBYTES> __device__ __forceinline__ int narrow_key_swizzle(int ro
 // the chain of dependent tiles of a short sequence.  The merge is the online-softmax
 // update applied once more, so only the FP32 rounding order differs.
 // INDEXED walks the key tiles listed for the 128-query block of the workgroup's queries
-// (the CSR pattern of the sparse path) instead of all of them; the last listed tile takes
-// the last-tile formulas, as in the wide kernel.
-template <int D, int CTA_K, int WAVES, int KSPLIT = 1, bool INDEXED = false>
+// (the CSR pattern of the sparse path, or the active tiles of a key-only mask) instead of
+// all of them; the last listed tile takes the last-tile formulas, as in the wide kernel.
+//
+// GENERAL is the pre-scaled path of the wide kernel (masks, causal, scale <= 0) with the
+// same decisions and arithmetic per score, CAPTURE its statistics stores; both run with
+// 128-query workgroups only.  MASK_DT as in the wide kernel (-1 none, kKeyBias for the
+// additive row of a key-only mask, else the element type of the mask tensor); MASK_VEC:
+// the four consecutive keys of a score group come from one load (unit key stride, aligned
+// rows).  They exist for head dim 256, where thirty-two queries per wavefront leave one
+// wavefront per SIMD.
+template <int D, int CTA_K, int MASK_DT = -1> using NarrowTileShape = TileShape<D, CTA_K, MASK_DT == kKeyBias ? CTA_K * 4 : 0>;
+
+__device__ __forceinline__ uint32_t sum_across_row_pairs(uint32_t x) {
+  const auto both = __builtin_amdgcn_permlane16_swap(x, x, false, false);
+  return both[0] + both[1];
+}
+
+template <int D, int CTA_K, int WAVES, int KSPLIT = 1, bool INDEXED = false, bool GENERAL = false,
+          bool CAPTURE = false, int MASK_DT = -1, bool MASK_VEC = false>
 __global__ __launch_bounds__(64 * WAVES * KSPLIT) void attention_narrow_kernel(const KernelParams p) {
   static_assert(WAVES == 8 || WAVES == 4 || WAVES == 2, "seeds and scales are copied by two different wavefronts");
   static_assert(KSPLIT == 1 || (KSPLIT == 2 && WAVES <= 4), "at most eight wavefronts per workgroup");
   static_assert(!INDEXED || KSPLIT == 1, "tile lists are not split");
+  static_assert(!(GENERAL || CAPTURE) || (WAVES == 8 && KSPLIT == 1), "masks and capture: 128-query workgroups");
+  static_assert(GENERAL || MASK_DT < 0, "the raw-score path takes no mask");
+  static_assert(!(CAPTURE && INDEXED), "statistics are captured on dense runs");
+  constexpr bool TENSOR_MASK = MASK_DT >= 0 && MASK_DT != kKeyBias;
   constexpr int QUERIES = 16 * WAVES;
-  using Shape = TileShape<D, CTA_K>;
+  using Shape = NarrowTileShape<D, CTA_K, MASK_DT>;
   constexpr int KB = CTA_K / 16;  // 16-key blocks per tile
   constexpr int SB = CTA_K / 64;  // 64-key steps of the P·V product
   constexpr int CB = D / 16;      // 16-channel blocks
@@ -72,10 +92,20 @@ __global__ __launch_bounds__(64 * WAVES * KSPLIT) void attention_narrow_kernel(c
   unsigned char* lds = lds_all + part * Shape::kLdsBytes;
 
   const int query_blocks = (p.q_len + QUERIES - 1) / QUERIES;
-  const int bx = blockIdx.x % query_blocks;
-  const int rest = blockIdx.x / query_blocks;
-  const int head = rest % p.q_heads;
-  const int batch = rest / p.q_heads;
+  int bx, head, batch;
+  if (GENERAL && p.causal) {
+    // longest query blocks first, across all heads (as in the wide kernel)
+    const int heads = p.q_heads * p.batch;
+    const int rest = blockIdx.x % heads;
+    bx = query_blocks - 1 - blockIdx.x / heads;
+    head = rest % p.q_heads;
+    batch = rest / p.q_heads;
+  } else {
+    bx = blockIdx.x % query_blocks;
+    const int rest = blockIdx.x / query_blocks;
+    head = rest % p.q_heads;
+    batch = rest / p.q_heads;
+  }
   const int kv_head = head / (p.q_heads / p.kv_heads);
   const int64_t bhk = static_cast<int64_t>(batch) * p.kv_heads + kv_head;
   const int64_t bhq = static_cast<int64_t>(batch) * p.q_heads + head;
@@ -84,6 +114,10 @@ __global__ __launch_bounds__(64 * WAVES * KSPLIT) void attention_narrow_kernel(c
   const int8_t* v_base = p.v + bhk * D * p.padded;
   const int32_t* sum_base = p.v_tile_sum + bhk * p.n_kb * D;
   const float* ks_base = p.k_scale + bhk * p.n_kb * 4;
+  [[maybe_unused]] const float* bias_base = nullptr;
+  if constexpr (MASK_DT == kKeyBias) {
+    bias_base = p.key_bias + batch * p.key_bias_stride_b + head * p.key_bias_stride_h;
+  }
 
   const int query = bx * QUERIES + wave * 16 + ql;
   const bool query_ok = query < p.q_len;
@@ -93,10 +127,20 @@ __global__ __launch_bounds__(64 * WAVES * KSPLIT) void attention_narrow_kernel(c
   const int first_tile = part == 0 ? 0 : p.n_kb - second_half;
   [[maybe_unused]] const int32_t* indices = nullptr;
   if constexpr (INDEXED) {
-    const int64_t row = bhq * p.n_qb + (bx * QUERIES) / kQueryBlock;
-    const int start = p.row_offsets[row];
-    n_it = __builtin_amdgcn_readfirstlane(p.row_offsets[row + 1] - start);
-    indices = p.tile_indices + start;
+    if (p.index_mode == 1) {
+      const int64_t row = bhq * p.n_qb + (bx * QUERIES) / kQueryBlock;
+      const int start = p.row_offsets[row];
+      n_it = __builtin_amdgcn_readfirstlane(p.row_offsets[row + 1] - start);
+      indices = p.tile_indices + start;
+    } else {
+      indices = p.tile_indices + bhq * (p.n_kb + 1);
+      n_it = __builtin_amdgcn_readfirstlane(indices[p.n_kb]);
+    }
+  } else if constexpr (GENERAL && !CAPTURE) {
+    if (p.causal) {
+      const int limit = min(p.k_len, (bx + 1) * QUERIES);
+      n_it = (limit + CTA_K - 1) / CTA_K;
+    }
   }
   auto tile_at = [&](int step) -> int {
     if constexpr (INDEXED) return __builtin_amdgcn_readfirstlane(indices[step]);
@@ -159,6 +203,12 @@ __global__ __launch_bounds__(64 * WAVES * KSPLIT) void attention_narrow_kernel(c
                               sl + Shape::kSeedBytes);
       }
     }
+    if constexpr (MASK_DT == kKeyBias) {
+      if (wave == WAVES - 3 && lane < CTA_K / 4) {
+        copy16_to_lds_uniform(reinterpret_cast<const int8_t*>(bias_base + static_cast<int64_t>(tile) * CTA_K),
+                              static_cast<uint32_t>(lane) * 16, lds + stage * Shape::kStageBytes + Shape::kMaskOffset);
+      }
+    }
   };
   // Read as a plain vector type: the compiler orders LDS reads it cannot classify
   // behind every outstanding copy into LDS, i.e. behind the next tile.
@@ -193,6 +243,56 @@ __global__ __launch_bounds__(64 * WAVES * KSPLIT) void attention_narrow_kernel(c
   float d_part = 0.0f;  // this lane's quarter of the row denominator
   float seed_value;
   asm volatile("v_mov_b32 %0, %1" : "=v"(seed_value) : "s"(kAccumulatorSeedBits));
+
+  // capture bookkeeping (layout of the wide kernel)
+  [[maybe_unused]] uint32_t* stats = nullptr;
+  [[maybe_unused]] uint64_t full_words = 0;
+  [[maybe_unused]] uint64_t stat_row = 0;
+  if constexpr (CAPTURE) {
+    const uint64_t mass_elements = static_cast<uint64_t>(p.batch) * p.q_heads * p.n_qb * p.n_kb;
+    stats = reinterpret_cast<uint32_t*>(p.workspace + mass_elements);
+    full_words = static_cast<uint64_t>(p.batch) * p.q_heads * p.q_len * (p.n_kb - 1) * 2;
+    stat_row = static_cast<uint64_t>(bhq) * p.q_len + query;
+  }
+  [[maybe_unused]] const int64_t mask_row =
+      TENSOR_MASK ? static_cast<int64_t>(batch) * p.mask_stride_b + static_cast<int64_t>(head) * p.mask_stride_h +
+                        static_cast<int64_t>(query) * p.mask_stride_q
+                  : 0;
+
+  // Mask elements of a full tile, requested before the next tile's copies: vector memory
+  // operations complete in order, so a mask load issued behind the copies could only be
+  // used once they have landed.  For masks that allow one load per four keys, with 64-key
+  // tiles (the tile of every query-dependent mask); other mask tensors are read inside the
+  // softmax and the next tile's copies are requested after it instead.
+  constexpr bool PRELOAD = TENSOR_MASK && MASK_VEC && CTA_K == 64;
+  constexpr bool LATE_COPIES = TENSOR_MASK && !PRELOAD;
+  constexpr int WORDS = MASK_DT == kF32 ? 4 : MASK_DT == kBool ? 1 : 2;  // 32-bit words per four keys
+  [[maybe_unused]] uint32_t mask_words[PRELOAD ? KB * WORDS : 1];
+  auto load_mask_words = [&](int tile) {
+    if constexpr (PRELOAD) {
+      constexpr int ES = MASK_DT == kF32 ? 4 : MASK_DT == kBool ? 1 : 2;
+      // rows past the last query read the last row; their results are never stored
+      const int64_t row = mask_row - static_cast<int64_t>(query_ok ? 0 : query - (p.q_len - 1)) * p.mask_stride_q;
+      const unsigned char* base = static_cast<const unsigned char*>(p.mask) +
+                                  (row + tile * CTA_K + 32 * (grp >> 1) + 4 * (grp & 1)) * ES;
+#pragma unroll
+      for (int kb = 0; kb < KB; ++kb) {
+        const unsigned char* at = base + ((kb >> 2) * 64 + (kb & 3) * 8) * ES;
+        uint32_t* words = mask_words + kb * WORDS;
+        if constexpr (WORDS == 1) {
+          words[0] = *reinterpret_cast<const uint32_t*>(at);
+        } else if constexpr (WORDS == 2) {
+          typedef uint32_t v2u __attribute__((ext_vector_type(2)));
+          const v2u w = *reinterpret_cast<const v2u*>(at);
+          words[0] = w[0], words[1] = w[1];
+        } else {
+          typedef uint32_t v4u __attribute__((ext_vector_type(4)));
+          const v4u w = *reinterpret_cast<const v4u*>(at);
+          words[0] = w[0], words[1] = w[1], words[2] = w[2], words[3] = w[3];
+        }
+      }
+    }
+  };
 
   // ---- S^T = K · Q^T ------------------------------------------------------------------
   const int key_row = 32 * (ql >> 3) + (ql & 7);  // row of this lane inside block (s, b): + 64*s + 8*b
@@ -229,13 +329,144 @@ __global__ __launch_bounds__(64 * WAVES * KSPLIT) void attention_narrow_kernel(c
   // Element (kb, i) is key tile*CTA_K + (kb/4)*64 + 32*(grp/2) + (kb%4)*8 + 4*(grp%2) + i,
   // K scale group (key % 8) / 2 = 2*(grp%2) + i/2.
   constexpr float kRescaleSlack = 8.0f;
-  auto softmax_tile = [&](auto last_tag, int tile, float ks0, float ks1, v4i (&s)[KB], v4i (&pk)[SB]) -> float {
+  auto softmax_tile = [&](auto last_tag, int it, int tile, float ks0, float ks1, v4i (&s)[KB], v4i (&pk)[SB]) -> float {
     constexpr bool LAST = decltype(last_tag)::value;
     const float sc0 = qs2 * (q_scale * ks0);
     const float sc1 = qs2 * (q_scale * ks1);
     float tile_m;
     uint32_t row_sum = 0;
-    if constexpr (!LAST) {
+    if constexpr (GENERAL) {
+      // Pre-scaled scores with masks: the decisions and the arithmetic per score of the wide
+      // kernel.  Whether a tile needs any masking is uniform over the wavefront.
+      const float neg_inf = -__builtin_inff();
+      const int first_query = bx * QUERIES + wave * 16;
+      const bool on_diagonal = p.causal && tile * CTA_K + CTA_K - 1 > first_query;
+      const bool partial = LAST && (tile + 1) * CTA_K > p.k_len;
+      const int key0 = tile * CTA_K + 32 * (grp >> 1) + 4 * (grp & 1);
+      float mx = kRowFloor;
+      if (MASK_DT < 0 && !on_diagonal && !partial) {
+#pragma unroll
+        for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const float value = score_value(s[kb][i]) * ((i & 2) ? sc1 : sc0);
+            s[kb][i] = __float_as_int(value);
+            mx = __builtin_fmaxf(mx, value);
+          }
+      } else {
+        auto masked_scores = [&](auto diagonal_tag) {
+          constexpr bool DIAGONAL = decltype(diagonal_tag)::value;
+          constexpr int ES = MASK_DT == kF32 ? 4 : MASK_DT == kBool ? 1 : 2;
+          [[maybe_unused]] const unsigned char* lane_mask = nullptr;
+          if constexpr (TENSOR_MASK) {
+            lane_mask = static_cast<const unsigned char*>(p.mask) +
+                        (mask_row + static_cast<int64_t>(key0) * p.mask_stride_k) * ES;
+          }
+          [[maybe_unused]] const float* bias_row = nullptr;
+          if constexpr (MASK_DT == kKeyBias) {
+            bias_row = reinterpret_cast<const float*>(lds + (it & 1) * Shape::kStageBytes + Shape::kMaskOffset) +
+                       32 * (grp >> 1) + 4 * (grp & 1);
+          }
+#pragma unroll
+          for (int kb = 0; kb < KB; ++kb) {
+            const int local = (kb >> 2) * 64 + (kb & 3) * 8;  // first of this lane's four consecutive keys
+            const int key = key0 + local;
+            bool keep[4] = {true, true, true, true};
+            float bias[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+            if constexpr (MASK_DT == kKeyBias) {
+              const v4f terms = *reinterpret_cast<const v4f*>(bias_row + local);
+              bias[0] = terms[0], bias[1] = terms[1], bias[2] = terms[2], bias[3] = terms[3];
+            } else if constexpr (PRELOAD && !LAST) {
+              const uint32_t* words = mask_words + kb * WORDS;
+              if constexpr (MASK_DT == kBool) {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) keep[r] = ((words[0] >> (8 * r)) & 0xffu) != 0;
+              } else if constexpr (MASK_DT == kF32) {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) bias[r] = __uint_as_float(words[r]);
+              } else {
+                const uint32_t bits16[4] = {words[0] & 0xffffu, words[0] >> 16, words[1] & 0xffffu, words[1] >> 16};
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                  bias[r] = MASK_DT == kF16 ? static_cast<float>(__builtin_bit_cast(_Float16, static_cast<uint16_t>(bits16[r])))
+                                            : __uint_as_float(bits16[r] << 16);
+                }
+              }
+              if constexpr (MASK_DT != kBool) {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) keep[r] = __builtin_isfinite(bias[r]);
+              }
+            } else if constexpr (TENSOR_MASK) {
+              if (!query_ok) {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) keep[r] = false;
+              } else if (MASK_VEC && key + 3 < p.k_len) {
+                const unsigned char* at = lane_mask + local * ES;
+                if constexpr (MASK_DT == kBool) {
+                  const uint32_t word = *reinterpret_cast<const uint32_t*>(at);
+#pragma unroll
+                  for (int r = 0; r < 4; ++r) keep[r] = ((word >> (8 * r)) & 0xffu) != 0;
+                } else if constexpr (MASK_DT == kF32) {
+                  const v4f w = *reinterpret_cast<const v4f*>(at);
+                  bias[0] = w[0], bias[1] = w[1], bias[2] = w[2], bias[3] = w[3];
+                } else {
+                  typedef uint32_t v2u __attribute__((ext_vector_type(2)));
+                  const v2u w = *reinterpret_cast<const v2u*>(at);
+                  const uint32_t bits16[4] = {w[0] & 0xffffu, w[0] >> 16, w[1] & 0xffffu, w[1] >> 16};
+#pragma unroll
+                  for (int r = 0; r < 4; ++r) {
+                    bias[r] = MASK_DT == kF16 ? static_cast<float>(__builtin_bit_cast(_Float16, static_cast<uint16_t>(bits16[r])))
+                                              : __uint_as_float(bits16[r] << 16);
+                  }
+                }
+              } else {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                  keep[r] = key + r < p.k_len;
+                  if (keep[r]) {
+                    const unsigned char* at = lane_mask + (local + r) * p.mask_stride_k * ES;
+                    if constexpr (MASK_DT == kBool) {
+                      keep[r] = *at != 0;
+                    } else {
+                      bias[r] = load1<MASK_DT>(at, 0);
+                    }
+                  }
+                }
+              }
+              if constexpr (MASK_DT != kBool) {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) keep[r] = keep[r] && __builtin_isfinite(bias[r]);
+              }
+            }
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+              float value = score_value(s[kb][r]) * ((r & 2) ? sc1 : sc0);
+              if constexpr (MASK_DT == kKeyBias) {
+                value += bias[r];
+              } else if constexpr (MASK_DT == kBool) {
+                value = keep[r] ? value : neg_inf;
+              } else if constexpr (TENSOR_MASK) {
+                value = keep[r] ? value + bias[r] * kLog2e : neg_inf;
+              }
+              if constexpr (DIAGONAL) {
+                if (key + r > query) value = neg_inf;
+              }
+              if constexpr (MASK_DT != kKeyBias) {
+                if (LAST && key + r >= p.k_len) value = neg_inf;
+              }
+              s[kb][r] = __float_as_int(value);
+              mx = __builtin_fmaxf(mx, value);
+            }
+          }
+        };
+        if (on_diagonal) {
+          masked_scores(std::true_type{});
+        } else {
+          masked_scores(std::false_type{});
+        }
+      }
+      tile_m = mx - kU8Offset;
+    } else if constexpr (!LAST) {
       int mx0 = s[0][0], mx1 = s[0][2];
 #pragma unroll
       for (int kb = 0; kb < KB; ++kb)
@@ -274,8 +505,13 @@ __global__ __launch_bounds__(64 * WAVES * KSPLIT) void attention_narrow_kernel(c
       uint32_t packed = 0;
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const float raw = LAST ? __int_as_float(s[kb][i]) : score_value(s[kb][i]);
-        const float x = __builtin_fmaf(raw, (i & 2) ? sc1 : sc0, neg_m);
+        float x;
+        if constexpr (GENERAL) {
+          x = __int_as_float(s[kb][i]) - tile_m;
+        } else {
+          const float raw = LAST ? __int_as_float(s[kb][i]) : score_value(s[kb][i]);
+          x = __builtin_fmaf(raw, (i & 2) ? sc1 : sc0, neg_m);
+        }
         packed = __builtin_amdgcn_cvt_pk_u8_f32(__builtin_amdgcn_exp2f(x), i, packed);
       }
       row_sum = __builtin_amdgcn_udot4(packed, 0x01010101u, row_sum, false);
@@ -296,6 +532,20 @@ __global__ __launch_bounds__(64 * WAVES * KSPLIT) void attention_narrow_kernel(c
     }
     const float t_scale = __builtin_amdgcn_exp2f(tile_m - m_run);
     d_part = __builtin_fmaf(static_cast<float>(row_sum), t_scale, d_part);
+    if constexpr (CAPTURE) {
+      const uint32_t numerator = sum_across_halves(sum_across_row_pairs(row_sum));
+      if (grp == 0 && query_ok) {
+        if constexpr (!LAST) {
+          const uint64_t offset = ((bhq * (p.n_kb - 1) + it) * static_cast<uint64_t>(p.q_len) + query) * 2;
+          stats[offset] = numerator;
+          stats[offset + 1] = __float_as_uint(tile_m);
+        } else {
+          const uint64_t offset = full_words + stat_row * 2;
+          stats[offset] = __float_as_uint(static_cast<float>(numerator));
+          stats[offset + 1] = __float_as_uint(tile_m);
+        }
+      }
+    }
     return t_scale;
   };
 
@@ -368,15 +618,23 @@ __global__ __launch_bounds__(64 * WAVES * KSPLIT) void attention_narrow_kernel(c
       __syncthreads();
       load_k_fragments(lds + stage * Shape::kStageBytes, 0, k_first);
       tile_scales(stage, ks0, ks1);
-      issue_tile(next_tile, stage ^ 1);
+      if constexpr (PRELOAD) {
+        load_mask_words(tile);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      if constexpr (!LATE_COPIES) issue_tile(next_tile, stage ^ 1);
       __builtin_amdgcn_s_setprio(0);  // vector phases before matrix phases, as in the wide kernel
       score_tile(stage, k_first, s);
       load_group(stage, 0, acc_first, v_first);
       __builtin_amdgcn_sched_barrier(0);
       __builtin_amdgcn_s_setprio(2);
-      const float t_scale = softmax_tile(std::false_type{}, tile, ks0, ks1, s, pk);
+      const float t_scale = softmax_tile(std::false_type{}, step, tile, ks0, ks1, s, pk);
       __builtin_amdgcn_s_setprio(1);
       __builtin_amdgcn_sched_barrier(0);
+      if constexpr (LATE_COPIES) {
+        issue_tile(next_tile, stage ^ 1);
+        __builtin_amdgcn_sched_barrier(0);
+      }
       value_tile(stage, pk, acc_first, v_first, t_scale);
       tile = next_tile;
     }
@@ -389,9 +647,9 @@ __global__ __launch_bounds__(64 * WAVES * KSPLIT) void attention_narrow_kernel(c
     // Only the last tile of the sequence takes the last-tile formulas.
     float t_scale;
     if (KSPLIT == 1 || part == KSPLIT - 1) {
-      t_scale = softmax_tile(std::true_type{}, tile, ks0, ks1, s, pk);
+      t_scale = softmax_tile(std::true_type{}, n_it - 1, tile, ks0, ks1, s, pk);
     } else {
-      t_scale = softmax_tile(std::false_type{}, tile, ks0, ks1, s, pk);
+      t_scale = softmax_tile(std::false_type{}, n_it - 1, tile, ks0, ks1, s, pk);
     }
     load_group(stage, 0, acc_first, v_first);
     value_tile(stage, pk, acc_first, v_first, t_scale);
@@ -437,7 +695,17 @@ __global__ __launch_bounds__(64 * WAVES * KSPLIT) void attention_narrow_kernel(c
   // ---- epilogue ---------------------------------------------------------------------------
   float d_total = d_part + __shfl_xor(d_part, 16);
   d_total += __shfl_xor(d_total, 32);
+  if constexpr (CAPTURE) {
+    if (grp == 0 && query_ok) {
+      const uint64_t query_rows = static_cast<uint64_t>(p.batch) * p.q_heads * p.q_len;
+      float* state = reinterpret_cast<float*>(stats + full_words + query_rows * 2);
+      state[stat_row * 2] = m_run;
+      state[stat_row * 2 + 1] = d_total;
+    }
+  }
   const float inv_d = 1.0f / d_total;
+  // rows without any visible key (masks, causal): zeros
+  const bool zero_row = GENERAL && (MASK_DT >= 0 || p.causal) && !(d_total > 0.0f);
   if (query_ok) {
     const float* vs = p.v_scale + bhk * D;
     const float* vc = p.v_center + bhk * D;
@@ -456,7 +724,10 @@ __global__ __launch_bounds__(64 * WAVES * KSPLIT) void attention_narrow_kernel(c
       value[3] = __builtin_fmaf(o_acc[cb][3] * inv_d, scale4.w, center4.w);
       uint32_t bits[4];
 #pragma unroll
-      for (int r = 0; r < 4; ++r) bits[r] = p.out_dtype == kF16 ? to_f16_bits(value[r]) : to_bf16_bits(value[r]);
+      for (int r = 0; r < 4; ++r) {
+        const float x = zero_row ? 0.0f : value[r];
+        bits[r] = p.out_dtype == kF16 ? to_f16_bits(x) : to_bf16_bits(x);
+      }
       uint2 word;
       word.x = bits[0] | (bits[1] << 16);
       word.y = bits[2] | (bits[3] << 16);

@@ -353,10 +353,11 @@ int risa_prepare_key_bias(const void* mask, float* bias, int batch, int heads, i
                                stride_h, stride_k, mask_dtype, static_cast<hipStream_t>(stream));
 }
 
-size_t risa_mask_lanes_bytes(int mask_dtype, int cta_k, int64_t mask_stride_q, int64_t mask_stride_k,
-                             int batch, int q_heads, int mask_batch, int mask_heads, int q_len,
-                             int k_len) {
+size_t risa_mask_lanes_bytes(int mask_dtype, int head_dim, int cta_k, int64_t mask_stride_q,
+                             int64_t mask_stride_k, int batch, int q_heads, int mask_batch,
+                             int mask_heads, int q_len, int k_len) {
   if (mask_dtype != risa::kBool || cta_k != 64 || mask_stride_q == 0 || mask_stride_k != 1) return 0;
+  if (head_dim > 128) return 0;  // the sixteen-query kernel of head dim 256 has another score layout
   if (batch <= 0 || q_heads <= 0 || mask_batch <= 0 || mask_heads <= 0 || q_len <= 0 || k_len <= 0) return 0;
   // The conversion reads the mask once; it pays when several heads then share the words.
   if (static_cast<int64_t>(batch) * q_heads < int64_t{4} * mask_batch * mask_heads) return 0;
@@ -438,8 +439,8 @@ size_t risa_sdpa_workspace_bytes(int batch, int q_heads, int q_len, int kv_heads
       (cta_k != 64 && cta_k != 128))
     return 0;
   const bool key_only = mask_dtype >= 0 && mask_stride_q == 0;
-  const size_t lanes = risa_mask_lanes_bytes(mask_dtype, cta_k, mask_stride_q, mask_stride_k, batch,
-                                             q_heads, mask_batch, mask_heads, q_len, k_len);
+  const size_t lanes = risa_mask_lanes_bytes(mask_dtype, head_dim, cta_k, mask_stride_q, mask_stride_k,
+                                             batch, q_heads, mask_batch, mask_heads, q_len, k_len);
   return sdpa_layout(batch, q_heads, q_len, kv_heads, k_len, head_dim, cta_k, midpoint_affine != 0,
                      key_only, lanes)
       .bytes;
@@ -466,8 +467,8 @@ int risa_sdpa(const void* q, const void* k, const void* v, void* out, void* work
   }
   const size_t lanes_bytes =
       mask == nullptr ? 0
-                      : risa_mask_lanes_bytes(mask_dtype, cta_k, mask_stride_q, mask_stride_k, batch,
-                                              q_heads, mask_batch, mask_heads, q_len, k_len);
+                      : risa_mask_lanes_bytes(mask_dtype, head_dim, cta_k, mask_stride_q, mask_stride_k,
+                                              batch, q_heads, mask_batch, mask_heads, q_len, k_len);
   const SdpaLayout l = sdpa_layout(batch, q_heads, q_len, kv_heads, k_len, head_dim, cta_k,
                                    midpoint_affine != 0, key_only, lanes_bytes);
   if (workspace == nullptr || !aligned(workspace, 256) || workspace_bytes < l.bytes)

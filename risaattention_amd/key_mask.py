@@ -36,12 +36,12 @@ def prepare_key_bias(mask, key_block_size):
     return bias, (bias.stride(0) if batch > 1 else 0), (bias.stride(1) if heads > 1 else 0)
 
 
-def prepare_mask_lanes(mask, key_block_size):
+def prepare_mask_lanes(mask, key_block_size, head_dim):
     """Lane words of a boolean mask several heads share, ``(words, stride_b, stride_h)`` or ``None``.
 
     ``mask`` is the expanded ``[B,Hq,Lq,Lk]`` view.  The library decides whether the form
-    applies (boolean, query-dependent, unit key stride, 64-key tiles, at least four
-    (batch, head) pairs per mask plane) by returning the size of the buffer or 0; the
+    applies (boolean, query-dependent, unit key stride, 64-key tiles, head dim up to 128,
+    at least four (batch, head) pairs per mask plane) by returning the size of the buffer or 0; the
     attention kernel then takes one 64-lane word per score from scalar registers instead
     of reading mask elements.
     """
@@ -51,7 +51,7 @@ def prepare_mask_lanes(mask, key_block_size):
     planes_b = batch if mask.stride(0) != 0 else 1
     planes_h = q_heads if mask.stride(1) != 0 else 1
     lib = native.library()
-    size = lib.risa_mask_lanes_bytes(MASK_DTYPE_CODES[mask.dtype], key_block_size, mask.stride(2),
+    size = lib.risa_mask_lanes_bytes(MASK_DTYPE_CODES[mask.dtype], head_dim, key_block_size, mask.stride(2),
                                      mask.stride(3), batch, q_heads, planes_b, planes_h, q_len, k_len)
     if size == 0:
         return None

@@ -57,7 +57,7 @@ SIGNATURES = {
         + [_c_f32, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr]
         + [_c_ptr, _c_i64, _c_i64, _c_ptr, _c_i64, _c_i64, _c_ptr],
     ),
-    "risa_mask_lanes_bytes": (_c_size, [_c_int, _c_int, _c_i64, _c_i64] + [_c_int] * 6),
+    "risa_mask_lanes_bytes": (_c_size, [_c_int, _c_int, _c_int, _c_i64, _c_i64] + [_c_int] * 6),
     "risa_prepare_mask_lanes": (
         _c_int,
         [_c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_i64, _c_i64, _c_i64, _c_ptr],

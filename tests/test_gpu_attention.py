@@ -439,14 +439,15 @@ def test_lane_words_of_a_boolean_mask(risa, q_len, k_len, aligned):
     planes[1, 0, 5] = False
     mask = planes.cuda()
     assert (mask.stride(2) % 16 == 0) == aligned  # rows the conversion can read 16 bytes at a time
-    words, stride_b, stride_h = prepare_mask_lanes(mask.expand(2, 8, q_len, k_len), 64)
+    words, stride_b, stride_h = prepare_mask_lanes(mask.expand(2, 8, q_len, k_len), 64, 128)
     expected = expected_lane_words(planes[:, 0].numpy(), q_len, k_len)
     assert stride_h == 0 and stride_b == expected[0].size
     assert np.array_equal(words.cpu().numpy().view(np.uint64).reshape(expected.shape), expected)
     # one plane per head is not worth converting, nor is any other dtype or tile size
-    assert prepare_mask_lanes(mask.expand(2, 3, q_len, k_len), 64) is None
-    assert prepare_mask_lanes(mask.expand(2, 8, q_len, k_len), 128) is None
-    assert prepare_mask_lanes(mask.expand(2, 8, q_len, k_len).float(), 64) is None
+    assert prepare_mask_lanes(mask.expand(2, 3, q_len, k_len), 64, 128) is None
+    assert prepare_mask_lanes(mask.expand(2, 8, q_len, k_len), 128, 128) is None
+    assert prepare_mask_lanes(mask.expand(2, 8, q_len, k_len), 64, 256) is None
+    assert prepare_mask_lanes(mask.expand(2, 8, q_len, k_len).float(), 64, 128) is None
 
 
 @pytest.mark.parametrize("dim", [64, 128, 256])
@@ -479,12 +480,14 @@ def test_shared_boolean_mask_equals_the_mask_per_head(risa, dim, causal, q_len, 
     assert relative_l2(to_numpy(lse[:1, :2])[finite], expected_lse[finite]) < TOLERANCE
 
 
-def test_shared_boolean_mask_in_the_sparse_path(risa):
-    """Pattern construction (capturing kernel) and reuse (tile lists) under lane words
-    give what they give under the mask read per head."""
-    heads, q_len, k_len, dim = 8, 512, 1500, 128
-    q = seeded((1, heads, q_len, dim), torch.bfloat16, 181)
-    k = seeded((1, 2, k_len, dim), torch.bfloat16, 182)
+@pytest.mark.parametrize("dim", [128, 256])
+def test_shared_boolean_mask_in_the_sparse_path(risa, dim):
+    """Pattern construction (capturing kernel) and reuse (tile lists) under a query-dependent
+    boolean mask: shared over heads (lane words up to head dim 128) they give what they give
+    with the mask read per head, and both follow the oracle walking the same lists."""
+    heads, q_len, k_len = 8, 512, 1500
+    q = seeded((1, heads, q_len, dim), torch.bfloat16, 181, scale=2.0)
+    k = seeded((1, 2, k_len, dim), torch.bfloat16, 182, scale=2.0)
     v = seeded((1, 2, k_len, dim), torch.bfloat16, 183)
     generator = torch.Generator().manual_seed(184)
     shared = (torch.rand((1, 1, q_len, k_len), generator=generator) > 0.3).cuda()
@@ -498,3 +501,9 @@ def test_shared_boolean_mask_in_the_sparse_path(risa):
     reuse = risa.sparse_int8_attention(q, k, v, pattern, attn_mask=shared)
     reuse_heads = risa.sparse_int8_attention(q, k, v, pattern_heads, attn_mask=per_head)
     assert torch.equal(reuse, reuse_heads)
+    prepared = oracle_prequantize(q, k, v, attn_mask=shared)
+    expected, _, _ = oracle_pipeline.attend(prepared)
+    assert relative_l2(to_numpy(out), expected) < TOLERANCE
+    lists = (pattern.row_offsets.cpu().numpy(), pattern.block_indices.cpu().numpy())
+    expected_reuse, _, _ = oracle_pipeline.attend(prepared, pattern=lists)
+    assert relative_l2(to_numpy(reuse), expected_reuse) < TOLERANCE
