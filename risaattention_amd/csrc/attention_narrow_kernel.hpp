@@ -1,9 +1,10 @@
-// Raw-score attention kernel for launches with fewer workgroups than compute units.
+// Attention kernel with sixteen queries per wavefront: launches with fewer workgroups
+// than compute units, and every launch with head dim 256.
 //
-// Same arithmetic as risa::attention_kernel<D, CTA_K, true, false, false, -1>
-// (reference csrc/kernels/attention_int8.cuh:145-1026, unmasked non-causal path) on the
-// same operands, with the 128 queries of a workgroup spread over eight wavefronts of
-// sixteen queries instead of four of thirty-two.  A lone 256-thread workgroup leaves
+// Same arithmetic as risa::attention_kernel (reference csrc/kernels/attention_int8.cuh:
+// 145-1026; the raw-score path, and for head dim 256 also the pre-scaled path with masks,
+// the causal rule and the capture stores) on the same operands, with the 128 queries of a
+// workgroup spread over eight wavefronts of sixteen queries instead of four of thirty-two.  A lone 256-thread workgroup leaves
 // one wavefront per SIMD, which issues a vector instruction only every other slot;
 // eight wavefronts put two on every SIMD with half the work each.  Measured on
 // B=1, H=16, D=128: 19 -> 17 us at 512 tokens, 29 -> 27.5 us at 1024, 47 -> 40.5 us at
