@@ -69,46 +69,78 @@ template <int BIT> __device__ __forceinline__ float dpp_partner(float value) {
   }
 }
 
-// One Hadamard butterfly level between lanes l and l xor BIT for COUNT values of a lane: the
-// lane with the bit clear keeps a + b, the other b - a (other - v on the lanes with the bit
-// set, other + v on the rest: one exact sign flip and one addition instead of both results and
-// a select).  All values of the lane pass a level together, so that the exchanges of one value
-// (which must wait two cycles for the instruction that produced their operand) issue between
-// those of the others.
+// One Hadamard butterfly level between lanes l and l xor BIT for COUNT values of a lane.  The
+// reference keeps a + b on the lane with the bit clear and a - b on the other (a: the value of
+// the lane with the bit clear).  Here every lane computes own + beta * partner in one fused
+// multiply-add whose DPP operand is the partner (beta = -1 on the lanes with the bit set, a
+// product that is exact): the lane with the bit set ends up with b - a, the exact negative of
+// the reference's value (IEEE addition is symmetric in sign).  Partners of a later level differ
+// in that level's bit only, so both carry the same sign and the recurrence holds at every
+// level; after all levels lane j holds the reference's values times (-1)^popcount(j), which the
+// caller folds into the final scaling.  All values of the lane pass a level together, so that
+// the exchanges of one value (which must wait two cycles for the instruction that produced
+// their operand) issue between those of the others.
+//
+// The multiply-adds are written out (four values per block): the compiler selects the VOP3
+// form of a fused multiply-add, which takes no DPP operand, and would spend a separate move
+// per exchange.  Every instruction of a block reads and writes its own value only, and a
+// value was last written a whole level earlier, which is what an instruction with a DPP
+// operand requires (two wait states after the write of its source); the s_nop in front of a
+// level's first block covers whatever the compiler placed ahead of it.
+#define RISA_BUTTERFLY_BLOCK(NOP, CONTROL)                                                   \
+  asm volatile(NOP                                                                           \
+               "v_fmac_f32_dpp %0, %0, %4 " CONTROL " row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t" \
+               "v_fmac_f32_dpp %1, %1, %4 " CONTROL " row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t" \
+               "v_fmac_f32_dpp %2, %2, %4 " CONTROL " row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t" \
+               "v_fmac_f32_dpp %3, %3, %4 " CONTROL " row_mask:0xf bank_mask:0xf bound_ctrl:1"       \
+               : "+v"(*values[n]), "+v"(*values[n + 1]), "+v"(*values[n + 2]), "+v"(*values[n + 3]) \
+               : "v"(beta))
 template <int BIT, int COUNT> __device__ __forceinline__ void butterfly_level(float* (&values)[COUNT], int sub) {
-  const uint32_t flip = (sub & BIT) ? 0x80000000u : 0u;
-  // The sign flips first, all of them: an instruction with a DPP operand must not follow the
-  // instruction that wrote any of its registers by less than two cycles.
-  float flipped[COUNT];
+  static_assert(BIT == 1 || BIT == 2 || BIT == 4 || BIT == 8, "DPP reaches partners inside a row of sixteen lanes");
+  static_assert(COUNT % 4 == 0, "values come in runs of four channels");
+  const float beta = (sub & BIT) ? -1.0f : 1.0f;
 #pragma unroll
-  for (int n = 0; n < COUNT; ++n) flipped[n] = __uint_as_float(__float_as_uint(*values[n]) ^ flip);
-  asm volatile("" ::: "memory");
-  if constexpr (BIT == 4) {
-    // l xor 4 = (l xor 3) xor 7: the reversal of every quad, then the reversal of every eight
-    // lanes; the second move joins the addition.  (A row shift reaches l xor 4 only for half
-    // of the lanes, which takes two moves that cannot join it.)
-    int reversed[COUNT];
-#pragma unroll
-    for (int n = 0; n < COUNT; ++n)
-      reversed[n] = __builtin_amdgcn_update_dpp(0, __float_as_int(*values[n]), 0x1B, 0xf, 0xf, true);  // quad_perm [3,2,1,0]
-    asm volatile("" ::: "memory");
-#pragma unroll
-    for (int n = 0; n < COUNT; ++n)
-      *values[n] = __int_as_float(__builtin_amdgcn_update_dpp(0, reversed[n], 0x141, 0xf, 0xf, true)) +  // row_half_mirror
-                   flipped[n];
-  } else {
-#pragma unroll
-    for (int n = 0; n < COUNT; ++n) {
-      float other;
-      if constexpr (BIT < 16) {
-        other = dpp_partner<BIT>(*values[n]);
+  for (int n = 0; n < COUNT; n += 4) {
+    if constexpr (BIT == 1) {
+      if (n == 0) {
+        RISA_BUTTERFLY_BLOCK("s_nop 1\n\t", "quad_perm:[1,0,3,2]");
       } else {
-        other = __shfl_xor(*values[n], BIT);
+        RISA_BUTTERFLY_BLOCK("", "quad_perm:[1,0,3,2]");
       }
-      *values[n] = other + flipped[n];
+    } else if constexpr (BIT == 2) {
+      if (n == 0) {
+        RISA_BUTTERFLY_BLOCK("s_nop 1\n\t", "quad_perm:[2,3,0,1]");
+      } else {
+        RISA_BUTTERFLY_BLOCK("", "quad_perm:[2,3,0,1]");
+      }
+    } else if constexpr (BIT == 8) {
+      // rotating a row of sixteen lanes by eight swaps its halves
+      if (n == 0) {
+        RISA_BUTTERFLY_BLOCK("s_nop 1\n\t", "row_ror:8");
+      } else {
+        RISA_BUTTERFLY_BLOCK("", "row_ror:8");
+      }
+    } else {
+      // l xor 4 = (l xor 3) xor 7: the reversal of every quad, then the reversal of every eight
+      // lanes; the second move joins the multiply-add.  (A row shift reaches l xor 4 only for
+      // half of the lanes, which takes two moves that cannot join it.)
+      float r0, r1, r2, r3;
+      asm volatile("s_nop 1\n\t"
+                   "v_mov_b32_dpp %4, %0 quad_perm:[3,2,1,0] row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+                   "v_mov_b32_dpp %5, %1 quad_perm:[3,2,1,0] row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+                   "v_mov_b32_dpp %6, %2 quad_perm:[3,2,1,0] row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+                   "v_mov_b32_dpp %7, %3 quad_perm:[3,2,1,0] row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+                   "v_fmac_f32_dpp %0, %4, %8 row_half_mirror row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+                   "v_fmac_f32_dpp %1, %5, %8 row_half_mirror row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+                   "v_fmac_f32_dpp %2, %6, %8 row_half_mirror row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+                   "v_fmac_f32_dpp %3, %7, %8 row_half_mirror row_mask:0xf bank_mask:0xf bound_ctrl:1"
+                   : "+v"(*values[n]), "+v"(*values[n + 1]), "+v"(*values[n + 2]), "+v"(*values[n + 3]),
+                     "=&v"(r0), "=&v"(r1), "=&v"(r2), "=&v"(r3)
+                   : "v"(beta));
     }
   }
 }
+#undef RISA_BUTTERFLY_BLOCK
 
 // Rotation of the channels one lane holds of SETS 128-channel blocks (64 channels for head
 // dim 64), SETS = tokens x blocks the lane works on.  Sixteen lanes share a token; lane j
@@ -149,9 +181,11 @@ template <int ROT, int GROUPS, int SETS> __device__ __forceinline__ void rotate(
   butterfly_level<2, COUNT>(values, j);
   butterfly_level<4, COUNT>(values, j);
   butterfly_level<8, COUNT>(values, j);
+  // the scaling of the transform, with the sign the butterfly levels left on this lane
   constexpr float factor = ROT == kRot64 ? 0.25f : 0.1767766952966369f;
+  const float lane_factor = (__builtin_popcount(j & 15) & 1) ? -factor : factor;
 #pragma unroll
-  for (int n = 0; n < COUNT; ++n) *values[n] *= factor;
+  for (int n = 0; n < COUNT; ++n) *values[n] *= lane_factor;
 }
 
 // Maximum over the 32 lanes of a half wavefront, in every lane: one lane swap for the
