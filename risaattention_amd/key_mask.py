@@ -41,7 +41,7 @@ def prepare_mask_lanes(mask, key_block_size, head_dim):
 
     ``mask`` is the expanded ``[B,Hq,Lq,Lk]`` view.  The library decides whether the form
     applies (boolean, query-dependent, unit key stride, 64-key tiles, head dim up to 128,
-    at least four (batch, head) pairs per mask plane) by returning the size of the buffer or 0; the
+    at least eight (batch, head) pairs per mask plane) by returning the size of the buffer or 0; the
     attention kernel then takes one 64-lane word per score from scalar registers instead
     of reading mask elements.
     """
