@@ -358,6 +358,9 @@ size_t risa_mask_lanes_bytes(int mask_dtype, int head_dim, int cta_k, int64_t ma
                              int mask_heads, int q_len, int k_len) {
   if (mask_dtype != risa::kBool || cta_k != 64 || mask_stride_q == 0 || mask_stride_k != 1) return 0;
   if (head_dim > 128) return 0;  // the sixteen-query kernel of head dim 256 has another score layout
+  // one conversion launch: blocks of 32 queries and mask planes are grid dimensions
+  if ((static_cast<int64_t>(q_len) + 127) / 128 * 4 > 65535 || static_cast<int64_t>(mask_batch) * mask_heads > 65535)
+    return 0;
   if (batch <= 0 || q_heads <= 0 || mask_batch <= 0 || mask_heads <= 0 || q_len <= 0 || k_len <= 0) return 0;
   // The conversion reads the mask once; it pays when several heads then share the words.
   if (static_cast<int64_t>(batch) * q_heads < int64_t{8} * mask_batch * mask_heads) return 0;
