@@ -246,7 +246,8 @@ int risa_prepare_key_bias(const void* mask, float* bias, int batch, int heads, i
  * from scalar registers.  risa_mask_lanes_bytes returns the size of the buffer, or 0
  * when the form does not apply or does not pay: the mask is not boolean, the tiles are
  * not 64 keys, the head dim is 256 (that kernel holds its scores in another layout), the
- * key stride is not 1, the query stride is 0, or fewer than eight
+ * key stride is not 1, the query stride is 0, the launch has at most 256 workgroups of 128
+ * queries (it runs the sixteen-query kernel), or fewer than eight
  * (batch, head) pairs share each mask plane (the conversion reads the mask once, the
  * attention kernel would read it once per pair).  No counterpart in the reference, whose
  * kernel reads the mask per score (csrc/kernels/attention_masks.cuh:27-164); the

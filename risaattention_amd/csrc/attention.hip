@@ -13,8 +13,8 @@ namespace risa {
 template <> int launch_attention_variant<64>(const KernelParams&, int, bool, bool, bool, int, hipStream_t);
 template <> int launch_attention_variant<128>(const KernelParams&, int, bool, bool, bool, int, hipStream_t);
 int launch_attention_narrow(const KernelParams& p, int head_dim, int cta_k, hipStream_t stream);
-int launch_attention_wide_head(const KernelParams& p, int cta_k, bool fast, bool indexed, bool capture,
-                               int mask_mode, hipStream_t stream);
+int launch_attention_narrow_general(const KernelParams& p, int head_dim, int cta_k, bool fast, bool indexed,
+                                    bool capture, int mask_mode, hipStream_t stream);
 int narrow_attention_limit();
 
 namespace {
@@ -129,7 +129,7 @@ int launch_attention(const AttentionArgs& a, hipStream_t stream) {
         mask_mode = kMaskStaged;
       }
     }
-    if (a.mask_lanes != nullptr && a.head_dim <= 128) {  // head dim 256 reads the mask itself
+    if (a.mask_lanes != nullptr && a.head_dim <= 128) {  // the sixteen-query kernel of head dim 256 reads the mask itself
       if (a.mask_dtype != kBool || a.cta_k != 64 || a.mask_stride_q == 0)
         return fail("risa_attention: lane words go with a query-dependent boolean mask and 64-key tiles");
       if (reinterpret_cast<uintptr_t>(a.mask_lanes) % 8 != 0)
@@ -188,15 +188,20 @@ int launch_attention(const AttentionArgs& a, hipStream_t stream) {
   const bool narrow = fast && p.index_mode != 2 && !capture &&
                       (a.head_dim > 128 || workgroups <= narrow_attention_limit());
 
+  // The other launches of that size (masked, causal, capturing, key-mask tile lists) and all of
+  // head dim 256 take the same kernel with 128-query workgroups; lane words, when given, keep
+  // the 32-query kernel that reads them.
+  const bool narrow_general = !narrow && mask_mode != kMaskLanes &&
+                              (a.head_dim > 128 || workgroups <= narrow_attention_limit());
   int status;
   if (narrow)
     status = launch_attention_narrow(p, a.head_dim, a.cta_k, stream);
+  else if (narrow_general)
+    status = launch_attention_narrow_general(p, a.head_dim, a.cta_k, fast, indexed, capture, mask_mode, stream);
   else if (a.head_dim == 64)
     status = launch_attention_variant<64>(p, a.cta_k, fast, indexed, capture, mask_mode, stream);
   else if (a.head_dim == 128)
     status = launch_attention_variant<128>(p, a.cta_k, fast, indexed, capture, mask_mode, stream);
-  else if (a.head_dim == 256)
-    status = launch_attention_wide_head(p, a.cta_k, fast, indexed, capture, mask_mode, stream);
   else
     return fail("risa_attention: unsupported head_dim");
   if (status != 0) return status;

@@ -741,4 +741,28 @@ __global__ __launch_bounds__(64 * WAVES * KSPLIT) void attention_narrow_kernel(c
   }
 }
 
+// Launch of one variant: grid of ceil(q_len / (16 * WAVES)) * heads * batch workgroups.
+template <int D, int CTA_K, int WAVES, int KSPLIT, bool INDEXED = false, bool GENERAL = false,
+          bool CAPTURE = false, int MASK_DT = -1, bool MASK_VEC = false>
+int launch_narrow_block(const KernelParams& p, hipStream_t stream) {
+  using Shape = NarrowTileShape<D, CTA_K, MASK_DT>;
+  constexpr int kLdsBytes = Shape::kLdsBytes * KSPLIT;
+  auto kernel = attention_narrow_kernel<D, CTA_K, WAVES, KSPLIT, INDEXED, GENERAL, CAPTURE, MASK_DT, MASK_VEC>;
+  static thread_local int configured_device = -1;
+  int device = -1;
+  if (hipGetDevice(&device) != hipSuccess) return fail("risa_attention: hipGetDevice failed");
+  if (device != configured_device) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes) != hipSuccess) {
+      return fail("risa_attention: cannot reserve " + std::to_string(kLdsBytes) + " bytes of LDS");
+    }
+    configured_device = device;
+  }
+  constexpr int QUERIES = 16 * WAVES;
+  const unsigned query_blocks = static_cast<unsigned>((p.q_len + QUERIES - 1) / QUERIES);
+  const dim3 grid(query_blocks * p.q_heads * p.batch);
+  kernel<<<grid, 64 * WAVES * KSPLIT, kLdsBytes, stream>>>(p);
+  return 0;
+}
+
 }  // namespace risa

@@ -358,6 +358,9 @@ size_t risa_mask_lanes_bytes(int mask_dtype, int head_dim, int cta_k, int64_t ma
                              int mask_heads, int q_len, int k_len) {
   if (mask_dtype != risa::kBool || cta_k != 64 || mask_stride_q == 0 || mask_stride_k != 1) return 0;
   if (head_dim > 128) return 0;  // the sixteen-query kernel of head dim 256 has another score layout
+  // A launch of at most one workgroup per compute unit (256 on the MI355X) runs the
+  // sixteen-query kernel, and the conversion would be a launch of its own next to a short kernel.
+  if (static_cast<int64_t>(batch) * q_heads * ((q_len + 127) / 128) <= 256) return 0;
   // one conversion launch: blocks of 32 queries and mask planes are grid dimensions
   if ((static_cast<int64_t>(q_len) + 127) / 128 * 4 > 65535 || static_cast<int64_t>(mask_batch) * mask_heads > 65535)
     return 0;
