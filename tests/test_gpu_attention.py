@@ -473,6 +473,15 @@ def test_shared_boolean_mask_equals_the_mask_per_head(risa, dim, causal, q_len, 
     out_heads, lse_heads = risa.int8_attention(q, k, v, attn_mask=per_head, is_causal=causal, return_lse=True)
     assert torch.equal(out, out_heads)
     assert torch.equal(lse, lse_heads)
+    # the same mask as a window of a wider tensor: rows 13 elements apart from a multiple of
+    # 16, base address odd (the conversion then reads it element by element)
+    wider = torch.zeros((2, 1, q_len, k_len + 13), dtype=torch.bool, device="cuda")
+    window = wider[..., 5:5 + k_len]
+    window.copy_(shared)
+    assert window.data_ptr() % 2 == 1 and not window.is_contiguous()
+    out_window, lse_window = risa.int8_attention(q, k, v, attn_mask=window, is_causal=causal, return_lse=True)
+    assert torch.equal(out_window, out)
+    assert torch.equal(lse_window, lse)
     assert torch.equal(out, risa.int8_attention(q, k, v, attn_mask=shared, is_causal=causal))  # the one-call route
     prepared = oracle_prequantize(q[:1, :2], k[:1, :1], v[:1, :1], attn_mask=shared[:1], is_causal=causal,
                                   return_lse=True)
