@@ -98,11 +98,11 @@ __global__ __launch_bounds__(256) void prepare_stage2_kernel(const FusedArgs a) 
     }
     block -= residual_blocks;
   }
-  const int x = block % a.code_blocks_x;
-  const int rest = block / a.code_blocks_x;
+  int position_block, bh, channel_block;
+  code_block_coordinates(block, a.code_blocks_x, a.kv, a.v.head_dim / 32, position_block, bh, channel_block);
   value_codes_block<DT, CTA_K, PARAMS>(a.v.v, a.v.codes, a.v.tile_sum, a.inverse, a.midpoint, a.v.length,
                                        a.v.padded, a.v.head_dim, a.v.heads, a.v.stride_b, a.v.stride_h,
-                                       a.v.stride_n, a.v.permutation, fused, x, rest % a.kv, rest / a.kv);
+                                       a.v.stride_n, a.v.permutation, fused, position_block, bh, channel_block);
 }
 
 template <int DT, int DK, int CTA_K, int ROT>

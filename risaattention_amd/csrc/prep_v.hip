@@ -31,11 +31,12 @@ template <int DT> int run(const ValueArgs& a, hipStream_t stream) {
       value_params_kernel<false><<<(groups + 3) / 4, 256, 0, stream>>>(
           w.part_max, w.part_min, a.scale, a.center, w.inverse, w.midpoint, a.head_dim, chunks, groups);
   }
-  dim3 code_grid((a.padded + 255) / 256, bh, a.head_dim / 32);
+  const int position_blocks = (a.padded + 255) / 256;
+  const dim3 code_grid(static_cast<unsigned>(position_blocks) * bh * (a.head_dim / 32));
 #define RISA_CODES(TILE, PARAMS)                                                                   \
   value_codes_kernel<DT, TILE, PARAMS><<<code_grid, 256, 0, stream>>>(                             \
       a.v, a.codes, a.tile_sum, w.inverse, w.midpoint, a.length, a.padded, a.head_dim, a.heads,    \
-      a.stride_b, a.stride_h, a.stride_n, a.permutation, fused)
+      a.stride_b, a.stride_h, a.stride_n, a.permutation, fused, position_blocks, bh)
   if (a.cta_k == 128) {
     if (!fuse_params)
       RISA_CODES(128, kParamsStored);

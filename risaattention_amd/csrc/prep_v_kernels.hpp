@@ -311,6 +311,31 @@ __device__ __forceinline__ void value_codes_block(const void* __restrict__ v, in
   }
 }
 
+// Launch order of the code workgroups.  A workgroup reads 32 of a token row's channels (64 of
+// its 256 bytes for a 16-bit input with 128 channels), so the workgroups of the other channel
+// blocks read the other parts of the same cache lines: they follow each other eight
+// workgroups apart -- consecutive workgroups go to the eight XCDs in turn, eight apart is the
+// same XCD and its L2 -- instead of a whole sweep over positions and heads later, when the
+// lines would come from HBM again.  `pairs` = position blocks x (batch, head) pairs.
+__device__ __forceinline__ void code_block_coordinates(int block, int position_blocks, int bh_count,
+                                                       int channel_blocks, int& position_block, int& bh,
+                                                       int& channel_block) {
+  const int pairs = position_blocks * bh_count;
+  const int grouped = pairs / 8 * 8;
+  int pair;
+  if (block < grouped * channel_blocks) {
+    const int step = block / 8;
+    channel_block = step % channel_blocks;
+    pair = step / channel_blocks * 8 + block % 8;
+  } else {
+    const int rest = pairs - grouped, local = block - grouped * channel_blocks;
+    channel_block = local / rest;
+    pair = grouped + local % rest;
+  }
+  position_block = pair % position_blocks;
+  bh = pair / position_blocks;
+}
+
 template <int DT, int CTA_K, int PARAMS>
 __global__ __launch_bounds__(256) void value_codes_kernel(const void* __restrict__ v,
                                                           int8_t* __restrict__ codes,
@@ -321,10 +346,13 @@ __global__ __launch_bounds__(256) void value_codes_kernel(const void* __restrict
                                                           int64_t stride_b, int64_t stride_h,
                                                           int64_t stride_n,
                                                           const int32_t* __restrict__ permutation,
-                                                          FusedParams fused) {
+                                                          FusedParams fused, int position_blocks,
+                                                          int bh_count) {
+  int position_block, bh, channel_block;
+  code_block_coordinates(blockIdx.x, position_blocks, bh_count, dim / 32, position_block, bh, channel_block);
   value_codes_block<DT, CTA_K, PARAMS>(v, codes, tile_sum, inverse, midpoint, length, padded, dim,
                                        heads, stride_b, stride_h, stride_n, permutation, fused,
-                                       blockIdx.x, blockIdx.y, blockIdx.z);
+                                       position_block, bh, channel_block);
 }
 
 // grid (T / (256/quads), B*H), 256 threads: thread = (summation thread t, four channels);
