@@ -9,6 +9,11 @@
   variant is compared with the oracle to the 1e-3 relative-L2 bar.
 * Video-DiT scale: H=40, N=32760 (last query block and last key tile hold 120 rows):
   closed forms, the last block against FP32, construction + reuse, packed replay.
+* Sparse reuse on block-structured Q/K: B=1, Hq=16, Hkv=4, D=128, N=32768, 64 contiguous
+  groups (centroid x 3 + unit noise), theta 0.99, five reuse calls under 0.05 drift: the
+  constructed tile sets of a slice against the oracle's capture, block masses and selector,
+  the structure the inputs force (a query block keeps the tiles of its own group), and every
+  reuse against the oracle walking the same lists.
 """
 
 from dataclasses import replace
@@ -17,7 +22,9 @@ import numpy as np
 import pytest
 import torch
 
+from oracle import attention as oracle_attention
 from oracle import pipeline as oracle_pipeline
+from oracle import selection as oracle_selection
 from tests.helpers import oracle_prequantize, relative_l2, to_numpy
 
 pytestmark = pytest.mark.gpu
@@ -236,3 +243,73 @@ def test_video_scale_configuration_full_size(risa):
         prepared = oracle_prequantize(q[:, head_pair, rows], k[:, head_pair], v[:, head_pair])
         expected, _, _ = oracle_pipeline.attend(prepared, pattern=(sliced_offsets, np.concatenate(lists)))
         assert relative_l2(to_numpy(sparse[:, head_pair, rows]), expected) < TOLERANCE, block
+
+
+def block_structured_inputs(length, groups, seed):
+    """Tokens in `groups` contiguous groups; Q and K are their group's centroid (N(0,1) x 3,
+    one per KV head, shared by its query heads) plus unit noise, V is unit noise
+    (the recipe of bench.py's sparse workload)."""
+    generator = torch.Generator(device="cuda").manual_seed(seed)
+    centroids = torch.randn(1, 4, groups, 128, generator=generator, device="cuda") * 3
+    per_token = centroids.repeat_interleave(length // groups, dim=2)
+    k = per_token + torch.randn(1, 4, length, 128, generator=generator, device="cuda")
+    q = per_token.repeat_interleave(4, dim=1) + torch.randn(1, 16, length, 128, generator=generator, device="cuda")
+    v = torch.randn(1, 4, length, 128, generator=generator, device="cuda")
+    return q.bfloat16(), k.bfloat16(), v.bfloat16()
+
+
+def test_block_structured_sparse_configuration_full_size(risa):
+    length, groups, theta = 32768, 64, 0.99
+    query_blocks, tiles_per_group = length // 128, length // groups // 128
+    q, k, v = block_structured_inputs(length, groups, seed=0)
+    built, pattern = risa.construct_sparse_int8_attention(q, k, v, theta=theta)
+    dense = risa.int8_attention(q, k, v)
+    torch.testing.assert_close(built, dense, atol=0.03, rtol=0.01)
+    assert pattern.measured_retained_mass >= theta
+    # a query block attends to its own group: four of the 256 key tiles
+    assert pattern.coverage == pytest.approx(tiles_per_group / query_blocks, rel=0.05)
+    offsets = pattern.row_offsets.cpu().numpy()
+    indices = pattern.block_indices.cpu().numpy()
+    assert offsets.shape == (16 * query_blocks + 1,) and offsets[-1] == indices.shape[0]
+    own_group = 0
+    for row in range(16 * query_blocks):
+        block = row % query_blocks
+        group_tiles = set(range(block // tiles_per_group * tiles_per_group, (block // tiles_per_group + 1) * tiles_per_group))
+        own_group += set(indices[offsets[row]:offsets[row + 1]].tolist()) == group_tiles
+    assert own_group >= 0.99 * 16 * query_blocks
+
+    # the tile sets of two heads x two query blocks against the oracle's capture, masses and selector
+    heads = slice(4, 6)  # both read KV head 1
+    for block in (3, query_blocks - 1):
+        rows = slice(block * 128, block * 128 + 128)
+        prepared = oracle_prequantize(q[:, heads, rows], k[:, 1:2], v[:, 1:2])
+        expected, _, capture = oracle_pipeline.attend(prepared, capture=True)
+        assert relative_l2(to_numpy(built[:, heads, rows]), expected) < TOLERANCE
+        masses = oracle_attention.block_mass(capture, 1, 2, 128)
+        want_offsets, want_indices, _, _ = oracle_selection.select_retained_mass(masses, theta)
+        for local, head in enumerate((4, 5)):
+            row = head * query_blocks + block
+            got = set(indices[offsets[row]:offsets[row + 1]].tolist())
+            want = set(want_indices[want_offsets[local]:want_offsets[local + 1]].tolist())
+            if got != want:  # documented tie: only tiles whose mass is within FP32 noise of the cut
+                cut = min(masses[local, tile] for tile in want)
+                for tile in got ^ want:
+                    assert abs(masses[local, tile] - cut) <= 1e-4 * max(cut, 1e-6) + 1e-6, (head, block, tile)
+
+    # five reuse calls while Q, K and V drift
+    generator = torch.Generator(device="cuda").manual_seed(1)
+    for step in range(5):
+        q, k, v = [(t.float() + 0.05 * torch.randn(t.shape, generator=generator, device="cuda")).bfloat16()
+                   for t in (q, k, v)]
+        sparse = risa.sparse_int8_attention(q, k, v, pattern)
+        dense = risa.int8_attention(q, k, v)
+        difference = (sparse.float() - dense.float()).abs()
+        sqnr = (10 * torch.log10(dense.float().pow(2).mean() / difference.pow(2).mean())).item()
+        print(f"block-structured reuse {step}: SQNR vs dense {sqnr:.1f} dB", flush=True)
+        assert sqnr > 25.0
+        rows = slice(3 * 128, 4 * 128)
+        lists = [indices[offsets[h * query_blocks + 3]:offsets[h * query_blocks + 3 + 1]] for h in (4, 5)]
+        sliced_offsets = np.concatenate([[0], np.cumsum([len(entry) for entry in lists])]).astype(np.int32)
+        prepared = oracle_prequantize(q[:, heads, rows], k[:, 1:2], v[:, 1:2])
+        expected, _, _ = oracle_pipeline.attend(prepared, pattern=(sliced_offsets, np.concatenate(lists)))
+        assert relative_l2(to_numpy(sparse[:, heads, rows]), expected) < TOLERANCE, step
