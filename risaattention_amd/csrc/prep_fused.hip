@@ -98,11 +98,9 @@ __global__ __launch_bounds__(256) void prepare_stage2_kernel(const FusedArgs a) 
     }
     block -= residual_blocks;
   }
-  int position_block, bh, channel_block;
-  code_block_coordinates(block, a.code_blocks_x, a.kv, a.v.head_dim / 32, position_block, bh, channel_block);
-  value_codes_block<DT, CTA_K, PARAMS>(a.v.v, a.v.codes, a.v.tile_sum, a.inverse, a.midpoint, a.v.length,
-                                       a.v.padded, a.v.head_dim, a.v.heads, a.v.stride_b, a.v.stride_h,
-                                       a.v.stride_n, a.v.permutation, fused, position_block, bh, channel_block);
+  value_codes_block<DT, CTA_K, PARAMS, DK>(a.v.v, a.v.codes, a.v.tile_sum, a.inverse, a.midpoint, a.v.length,
+                                           a.v.padded, a.v.heads, a.v.stride_b, a.v.stride_h, a.v.stride_n,
+                                           a.v.permutation, fused, block % a.code_blocks_x, block / a.code_blocks_x);
 }
 
 template <int DT, int DK, int CTA_K, int ROT>
@@ -116,7 +114,7 @@ void launch_stages(const FusedArgs& a, hipStream_t stream) {
   with_center.residual_blocks_x =
       merged_residual ? summation_threads(a.v.length) / (256 / (a.v.head_dim / 4)) : 0;
   const int stage2_blocks = a.key_blocks + with_center.center_blocks + with_center.residual_blocks_x * a.kv +
-                            a.code_blocks_x * a.kv * (a.v.head_dim / 32);
+                            a.code_blocks_x * a.kv;
   const int groups = a.kv * a.v.head_dim / 8;
   if (a.v.midpoint_affine) {
     prepare_stage1_kernel<DT, DK, ROT, true><<<stage1_blocks, 256, 0, stream>>>(a);
@@ -226,7 +224,7 @@ int launch_prepare_fused(const QkArgs& qk, const ValueArgs& v, hipStream_t strea
   a.range_groups = (a.chunks + 3) / 4;
   a.key_tiles = (qk.k_len + qk.cta_k - 1) / qk.cta_k;
   a.key_blocks = 2 * a.key_tiles * a.kv;  // half a tile per workgroup
-  a.code_blocks_x = (v.padded + 255) / 256;
+  a.code_blocks_x = (v.padded + kCodeBlockPositions - 1) / kCodeBlockPositions;
   a.q_wide = rows_are_16_byte_aligned(qk.q, qk.q_stride_b, qk.q_stride_h, qk.q_stride_n, qk.dtype);
   a.k_wide = rows_are_16_byte_aligned(qk.k, qk.k_stride_b, qk.k_stride_h, qk.k_stride_n, qk.dtype);
   if (qk.dtype == kF32)

@@ -31,12 +31,21 @@ template <int DT> int run(const ValueArgs& a, hipStream_t stream) {
       value_params_kernel<false><<<(groups + 3) / 4, 256, 0, stream>>>(
           w.part_max, w.part_min, a.scale, a.center, w.inverse, w.midpoint, a.head_dim, chunks, groups);
   }
-  const int position_blocks = (a.padded + 255) / 256;
-  const dim3 code_grid(static_cast<unsigned>(position_blocks) * bh * (a.head_dim / 32));
+  const int position_blocks = (a.padded + kCodeBlockPositions - 1) / kCodeBlockPositions;
+  const dim3 code_grid(static_cast<unsigned>(position_blocks) * bh);
+#define RISA_CODES_DIM(TILE, PARAMS, DIM)                                                          \
+  value_codes_kernel<DT, TILE, PARAMS, DIM><<<code_grid, 256, 0, stream>>>(                        \
+      a.v, a.codes, a.tile_sum, w.inverse, w.midpoint, a.length, a.padded, a.heads, a.stride_b,    \
+      a.stride_h, a.stride_n, a.permutation, fused, position_blocks)
 #define RISA_CODES(TILE, PARAMS)                                                                   \
-  value_codes_kernel<DT, TILE, PARAMS><<<code_grid, 256, 0, stream>>>(                             \
-      a.v, a.codes, a.tile_sum, w.inverse, w.midpoint, a.length, a.padded, a.head_dim, a.heads,    \
-      a.stride_b, a.stride_h, a.stride_n, a.permutation, fused, position_blocks, bh)
+  do {                                                                                             \
+    if (a.head_dim == 64)                                                                          \
+      RISA_CODES_DIM(TILE, PARAMS, 64);                                                            \
+    else if (a.head_dim == 128)                                                                    \
+      RISA_CODES_DIM(TILE, PARAMS, 128);                                                           \
+    else                                                                                           \
+      RISA_CODES_DIM(TILE, PARAMS, 256);                                                           \
+  } while (0)
   if (a.cta_k == 128) {
     if (!fuse_params)
       RISA_CODES(128, kParamsStored);
@@ -52,6 +61,7 @@ template <int DT> int run(const ValueArgs& a, hipStream_t stream) {
     else
       RISA_CODES(64, kParamsAbsmax);
   }
+#undef RISA_CODES_DIM
 #undef RISA_CODES
   if (a.midpoint_affine) {
     if (a.length <= kFusedCenterMaxLength) {

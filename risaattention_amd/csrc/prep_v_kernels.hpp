@@ -193,16 +193,30 @@ __global__ __launch_bounds__(256) void value_params_kernel(const float* __restri
   }
 }
 
-// grid (ceil(padded/256), B*H, dim/32), 256 threads.  Lane l of every wave owns the
-// four packed positions 256*blockIdx.x + 4*l .. +3 (four consecutive tokens); wave
-// w of the workgroup takes the eight channels 32*blockIdx.z + 8*w .. +7.
+// grid (ceil(padded/128) * B*H), 256 threads: a workgroup turns 128 packed positions (128
+// tokens) of every channel into codes.
+//   * Loads cover whole token rows: the dim/8 lanes next to each other read the 16-byte
+//     pieces of one row, so a load instruction of a wavefront touches 64/(dim/8) rows and
+//     every cache line once (a lane-per-token mapping touches 64 rows for 16 bytes each and
+//     is limited by the address rate of the load path: 4.0 TB/s where Q and K reach 5.7-6.1).
+//     A thread owns four consecutive positions (four consecutive tokens) of eight channels,
+//     32/(256/(dim/8)) such quads; all its loads are issued before any is used.
+//   * The four codes of a channel become one 32-bit word, which goes to LDS at
+//     [channel row][position quad]; after a barrier two threads per channel row read 64 bytes
+//     each and store them: every store instruction of a wavefront writes whole cache lines of
+//     the packed transposed matrix, and the same words give the accumulator seeds of the
+//     tile(s) (a 128-key tile is the workgroup's 128 positions, a 64-key tile one half).
+//   * LDS rows are 36 words apart and channel 8*o + i sits in row i*(dim/8) + o: the words a
+//     wavefront writes at once (fixed i, all o, four quads) then fall into different banks
+//     two by two, and so do the 16-byte reads of neighbouring rows.
 //
 // PARAMS says where the per-channel scale and midpoint come from: kParamsStored reads
 // what value_params_kernel left; kParamsAbsmax / kParamsAffine reduce the partial
-// ranges (at most 64 of them, one per lane) inside every wavefront, which saves a
-// launch for short sequences; the workgroups of the first 256 positions also store
+// ranges (at most 64 of them) inside every workgroup, one thread per channel, which saves a
+// launch for short sequences; the workgroups of the first 128 positions also store
 // the parameters for the kernels that follow.
 constexpr int kParamsStored = 0, kParamsAbsmax = 1, kParamsAffine = 2;
+constexpr int kCodeBlockPositions = 128;
 
 struct FusedParams {
   const float* part_max;
@@ -214,145 +228,170 @@ struct FusedParams {
   int chunks;
 };
 
-template <int DT, int CTA_K, int PARAMS>
+template <int DT, int CTA_K, int PARAMS, int DK>
 __device__ __forceinline__ void value_codes_block(const void* __restrict__ v, int8_t* __restrict__ codes,
                                                   int32_t* __restrict__ tile_sum,
                                                   const float* __restrict__ inverse,
                                                   const float* __restrict__ midpoint, int length,
-                                                  int padded, int dim, int heads, int64_t stride_b,
+                                                  int padded, int heads, int64_t stride_b,
                                                   int64_t stride_h, int64_t stride_n,
                                                   const int32_t* __restrict__ permutation,
-                                                  const FusedParams& fused, int position_block, int bh,
-                                                  int channel_block) {
+                                                  const FusedParams& fused, int position_block, int bh) {
+  constexpr int OCTETS = DK / 8;        // lanes per token row
+  constexpr int SLOTS = 256 / OCTETS;   // quads of positions in flight per load
+  constexpr int QUADS = 32 / SLOTS;     // quads per thread
+  constexpr int BATCH = QUADS < 2 ? QUADS : 2;  // quads whose loads are in flight together
+  constexpr int PITCH = 36;             // words between LDS rows (16-byte aligned, 4 banks apart)
+  typedef uint32_t v4u __attribute__((ext_vector_type(4)));
+  __shared__ __attribute__((aligned(16))) uint32_t transposed[DK * PITCH];
+  __shared__ float channel_inverse[DK], channel_midpoint[DK];
+  [[maybe_unused]] __shared__ float partial_max[256 / DK][DK], partial_min[256 / DK][DK];
   const int b = bh / heads, h = bh - b * heads;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int p0 = position_block * 256 + lane * 4;
-  const int n0 = first_token_of_positions(p0);
+  const int tid = threadIdx.x;
+  const int octet = tid % OCTETS, slot = tid / OCTETS;
   const int64_t base = static_cast<int64_t>(b) * stride_b + static_cast<int64_t>(h) * stride_h;
+  const int64_t row0 = static_cast<int64_t>(bh) * DK;
   const int tiles = padded / CTA_K;
-  {
-    const int octet = channel_block * 4 + wave;
-    const int64_t row0 = static_cast<int64_t>(bh) * dim + octet * 8;
-    float inv[8], mid[8];
-    if constexpr (PARAMS == kParamsStored) {
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        inv[i] = inverse[row0 + i];
-        mid[i] = midpoint[row0 + i];
-      }
-    } else {
-      constexpr bool AFFINE = PARAMS == kParamsAffine;
-      float mx[8], mn[8];
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        mx[i] = AFFINE ? -FLT_MAX : 0.0f;
-        mn[i] = FLT_MAX;
-      }
-      if (lane < fused.chunks) {
-        const int64_t slot = (static_cast<int64_t>(bh) * fused.chunks + lane) * dim + octet * 8;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-          mx[i] = fused.part_max[slot + i];
-          if constexpr (AFFINE) mn[i] = fused.part_min[slot + i];
-        }
-      }
-#pragma unroll
-      for (int offset = 32; offset > 0; offset >>= 1) {
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-          mx[i] = __builtin_fmaxf(mx[i], __shfl_xor(mx[i], offset));
-          if constexpr (AFFINE) mn[i] = __builtin_fminf(mn[i], __shfl_xor(mn[i], offset));
-        }
-      }
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        mid[i] = AFFINE ? 0.5f * (mn[i] + mx[i]) : 0.0f;
-        const float radius = AFFINE ? 0.5f * (mx[i] - mn[i]) : mx[i];
-        const float sc = __builtin_fmaxf(radius * (1.0f / 127.0f), 1e-12f);
-        inv[i] = 1.0f / sc;
-        if (position_block == 0 && lane == i) {
-          fused.scale[row0 + i] = sc;
-          fused.inverse[row0 + i] = inv[i];
-          fused.midpoint[row0 + i] = mid[i];
-          if constexpr (!AFFINE) fused.center[row0 + i] = 0.0f;
-        }
-      }
-    }
-    // The four token loads are issued together, outside any branch; tokens past the end
-    // read the last row and their codes are zeroed.
-    float q[8][4];  // codes as magic sums (round_to_code)
-    int from[4];
-#pragma unroll
-    for (int r = 0; r < 4; ++r) from[r] = min(n0 + r, length - 1);
-    if (permutation != nullptr) {
-#pragma unroll
-      for (int r = 0; r < 4; ++r) from[r] = permutation[static_cast<int64_t>(bh) * length + from[r]];
-    }
-    float x[4][8];
-#pragma unroll
-    for (int r = 0; r < 4; ++r) load8<DT>(v, base + static_cast<int64_t>(from[r]) * stride_n + octet * 8, x[r]);
-#pragma unroll
-    for (int r = 0; r < 4; ++r)
-#pragma unroll
-      for (int i = 0; i < 8; ++i)
-        q[i][r] = n0 + r < length ? round_to_code((x[r][i] - mid[i]) * inv[i]) : kRoundMagic;
+  const int first_position = position_block * kCodeBlockPositions;
+
+  float inv[8], mid[8];
+  if constexpr (PARAMS == kParamsStored) {
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-      const uint32_t word = pack_codes(q[i][0], q[i][1], q[i][2], q[i][3]);
-      if (p0 < padded) *reinterpret_cast<uint32_t*>(codes + (row0 + i) * padded + p0) = word;
-      int sum = sum_of_codes(word);
+      inv[i] = inverse[row0 + octet * 8 + i];
+      mid[i] = midpoint[row0 + octet * 8 + i];
+    }
+  } else {
+    constexpr bool AFFINE = PARAMS == kParamsAffine;
+    // All 256 threads walk the (at most 64) partial ranges: thread (channel, part) takes every
+    // PARTS-th one.  The loads are independent of each other and of the token loads below and
+    // sit in no branch (a range past the last one reads the last one again, which changes
+    // neither a maximum nor a minimum), so all of them are in flight together.
+    constexpr int PARTS = 256 / DK;
+    constexpr int PER_PART = 64 / PARTS;
+    {
+      const int channel = tid % DK, part = tid / DK;
+      float mx = AFFINE ? -FLT_MAX : 0.0f, mn = FLT_MAX;
 #pragma unroll
-      for (int offset = CTA_K / 8; offset > 0; offset >>= 1) sum += __shfl_xor(sum, offset);
-      if ((lane & (CTA_K / 4 - 1)) == 0 && p0 < padded) {
-        tile_sum[(static_cast<int64_t>(bh) * tiles + p0 / CTA_K) * dim + octet * 8 + i] =
+      for (int k = 0; k < PER_PART; ++k) {
+        const int chunk = min(k * PARTS + part, fused.chunks - 1);
+        const int64_t at = (static_cast<int64_t>(bh) * fused.chunks + chunk) * DK + channel;
+        mx = __builtin_fmaxf(mx, fused.part_max[at]);
+        if constexpr (AFFINE) mn = __builtin_fminf(mn, fused.part_min[at]);
+      }
+      partial_max[part][channel] = mx;
+      if constexpr (AFFINE) partial_min[part][channel] = mn;
+    }
+    __syncthreads();
+    if (tid < DK) {
+      float mx = partial_max[0][tid], mn = AFFINE ? partial_min[0][tid] : FLT_MAX;
+#pragma unroll
+      for (int part = 1; part < PARTS; ++part) {
+        mx = __builtin_fmaxf(mx, partial_max[part][tid]);
+        if constexpr (AFFINE) mn = __builtin_fminf(mn, partial_min[part][tid]);
+      }
+      const float middle = AFFINE ? 0.5f * (mn + mx) : 0.0f;
+      const float radius = AFFINE ? 0.5f * (mx - mn) : mx;
+      const float sc = __builtin_fmaxf(radius * (1.0f / 127.0f), 1e-12f);
+      const float reciprocal = 1.0f / sc;
+      channel_inverse[tid] = reciprocal;
+      channel_midpoint[tid] = middle;
+      if (position_block == 0) {
+        fused.scale[row0 + tid] = sc;
+        fused.inverse[row0 + tid] = reciprocal;
+        fused.midpoint[row0 + tid] = middle;
+        if constexpr (!AFFINE) fused.center[row0 + tid] = 0.0f;
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      inv[i] = channel_inverse[octet * 8 + i];
+      mid[i] = channel_midpoint[octet * 8 + i];
+    }
+  }
+
+#pragma unroll
+  for (int first = 0; first < QUADS; first += BATCH) {
+    // The loads of a batch are issued together, outside any branch; tokens past the end
+    // read the last row and their codes are zeroed.
+    int from[BATCH][4];
+#pragma unroll
+    for (int j = 0; j < BATCH; ++j) {
+      const int n0 = first_token_of_positions(first_position + (slot + SLOTS * (first + j)) * 4);
+#pragma unroll
+      for (int r = 0; r < 4; ++r) from[j][r] = min(n0 + r, length - 1);
+    }
+    if (permutation != nullptr) {
+#pragma unroll
+      for (int j = 0; j < BATCH; ++j)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) from[j][r] = permutation[static_cast<int64_t>(bh) * length + from[j][r]];
+    }
+    float x[BATCH][4][8];
+#pragma unroll
+    for (int j = 0; j < BATCH; ++j)
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        load8<DT>(v, base + static_cast<int64_t>(from[j][r]) * stride_n + octet * 8, x[j][r]);
+#pragma unroll
+    for (int j = 0; j < BATCH; ++j) {
+      const int quad = slot + SLOTS * (first + j);
+      const int n0 = first_token_of_positions(first_position + quad * 4);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        float q[4];  // codes as magic sums (round_to_code)
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          q[r] = n0 + r < length ? round_to_code((x[j][r][i] - mid[i]) * inv[i]) : kRoundMagic;
+        transposed[(i * OCTETS + octet) * PITCH + quad] = pack_codes(q[0], q[1], q[2], q[3]);
+      }
+    }
+  }
+  __syncthreads();
+
+  // Two threads per LDS row: 64 positions (bytes) each.  Row r holds channel 8*(r % OCTETS) + r / OCTETS.
+#pragma unroll
+  for (int task = tid; task < DK * 2; task += 256) {
+    const int row = task >> 1, half = task & 1;
+    const int channel = (row % OCTETS) * 8 + row / OCTETS;
+    const int position = first_position + half * 64;
+    const v4u* source = reinterpret_cast<const v4u*>(transposed + row * PITCH + half * 16);
+    v4u words[4];
+#pragma unroll
+    for (int n = 0; n < 4; ++n) words[n] = source[n];
+    int sum = 0;
+#pragma unroll
+    for (int n = 0; n < 4; ++n)
+#pragma unroll
+      for (int w = 0; w < 4; ++w) sum += sum_of_codes(words[n][w]);
+    if constexpr (CTA_K == 128) sum += __shfl_xor(sum, 1);
+    if (position < padded) {
+      v4u* target = reinterpret_cast<v4u*>(codes + (row0 + channel) * padded + position);
+#pragma unroll
+      for (int n = 0; n < 4; ++n) target[n] = words[n];
+      if (CTA_K == 64 || half == 0) {
+        tile_sum[(static_cast<int64_t>(bh) * tiles + position / CTA_K) * DK + channel] =
             sum * 128 + kAccumulatorSeedBits;
       }
     }
   }
 }
 
-// Launch order of the code workgroups.  A workgroup reads 32 of a token row's channels (64 of
-// its 256 bytes for a 16-bit input with 128 channels), so the workgroups of the other channel
-// blocks read the other parts of the same cache lines: they follow each other eight
-// workgroups apart -- consecutive workgroups go to the eight XCDs in turn, eight apart is the
-// same XCD and its L2 -- instead of a whole sweep over positions and heads later, when the
-// lines would come from HBM again.  `pairs` = position blocks x (batch, head) pairs.
-__device__ __forceinline__ void code_block_coordinates(int block, int position_blocks, int bh_count,
-                                                       int channel_blocks, int& position_block, int& bh,
-                                                       int& channel_block) {
-  const int pairs = position_blocks * bh_count;
-  const int grouped = pairs / 8 * 8;
-  int pair;
-  if (block < grouped * channel_blocks) {
-    const int step = block / 8;
-    channel_block = step % channel_blocks;
-    pair = step / channel_blocks * 8 + block % 8;
-  } else {
-    const int rest = pairs - grouped, local = block - grouped * channel_blocks;
-    channel_block = local / rest;
-    pair = grouped + local % rest;
-  }
-  position_block = pair % position_blocks;
-  bh = pair / position_blocks;
-}
-
-template <int DT, int CTA_K, int PARAMS>
+template <int DT, int CTA_K, int PARAMS, int DK>
 __global__ __launch_bounds__(256) void value_codes_kernel(const void* __restrict__ v,
                                                           int8_t* __restrict__ codes,
                                                           int32_t* __restrict__ tile_sum,
                                                           const float* __restrict__ inverse,
                                                           const float* __restrict__ midpoint,
-                                                          int length, int padded, int dim, int heads,
+                                                          int length, int padded, int heads,
                                                           int64_t stride_b, int64_t stride_h,
                                                           int64_t stride_n,
                                                           const int32_t* __restrict__ permutation,
-                                                          FusedParams fused, int position_blocks,
-                                                          int bh_count) {
-  int position_block, bh, channel_block;
-  code_block_coordinates(blockIdx.x, position_blocks, bh_count, dim / 32, position_block, bh, channel_block);
-  value_codes_block<DT, CTA_K, PARAMS>(v, codes, tile_sum, inverse, midpoint, length, padded, dim,
-                                       heads, stride_b, stride_h, stride_n, permutation, fused,
-                                       position_block, bh, channel_block);
+                                                          FusedParams fused, int position_blocks) {
+  value_codes_block<DT, CTA_K, PARAMS, DK>(v, codes, tile_sum, inverse, midpoint, length, padded, heads,
+                                           stride_b, stride_h, stride_n, permutation, fused,
+                                           blockIdx.x % position_blocks, blockIdx.x / position_blocks);
 }
 
 // grid (T / (256/quads), B*H), 256 threads: thread = (summation thread t, four channels);
