@@ -26,6 +26,33 @@ def test_library_exports_every_declared_symbol():
     assert native.library().risa_last_error() == b""
 
 
+def test_lane_word_size_query_rules():
+    """risa_mask_lanes_bytes is a host function: the size of the lane words of a boolean mask
+    that enough heads share, 0 wherever the attention kernel reads the mask itself."""
+    lib = native.library()
+    BOOL, F32 = 3, 0
+
+    def size(dtype=BOOL, head_dim=128, cta_k=64, stride_q=4608, stride_k=1, batch=2, heads=24,
+             mask_batch=2, mask_heads=1, q_len=4096, k_len=4608):
+        return lib.risa_mask_lanes_bytes(dtype, head_dim, cta_k, stride_q, stride_k, batch, heads,
+                                         mask_batch, mask_heads, q_len, k_len)
+
+    # [mask batch, mask heads, blocks of 32 queries padded to 128, 64-key tiles, 32 words] x 8 bytes
+    assert size() == 2 * 1 * (4096 // 32) * (4608 // 64) * 32 * 8
+    assert size(q_len=4000, k_len=4600) == 2 * (32 * 4) * 72 * 32 * 8  # ragged extents round up
+    assert size(head_dim=64) == size()
+    assert size(dtype=F32) == 0            # values, not decisions
+    assert size(cta_k=128) == 0            # query-dependent masks run 64-key tiles
+    assert size(head_dim=256) == 0         # the sixteen-query kernel has another score layout
+    assert size(stride_q=0) == 0           # key-only masks have their bias row
+    assert size(stride_k=2) == 0
+    assert size(mask_heads=24) == 0        # a plane per head: nobody to share with
+    assert size(heads=7) == 0 and size(heads=8) > 0  # eight (batch, head) pairs per mask plane
+    assert size(batch=1, heads=8, mask_batch=1, q_len=4096) == 0   # 256 workgroups: a small launch
+    assert size(batch=1, heads=8, mask_batch=1, q_len=4224) > 0
+    assert size(q_len=0) == 0
+
+
 def test_host_only_entry_points():
     assert native.unpack_order() == layout.position_to_token()
     assert sorted(native.unpack_order()) == list(range(32))
