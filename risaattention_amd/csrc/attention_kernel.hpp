@@ -89,13 +89,21 @@ template <int ROWBYTES> __device__ __forceinline__ int swizzled(int row, int chu
   return row * ROWBYTES + ((chunk ^ ((row / ROWS_PER_256) & (CH - 1))) << 4);
 }
 
-__device__ __forceinline__ uint16_t to_bf16_bits(float x) {
-  uint32_t bits = __float_as_uint(x);
-  const uint32_t rounded = bits + 0x7fffu + ((bits >> 16) & 1u);
-  return static_cast<uint16_t>((x != x ? (bits | 0x400000u) : rounded) >> 16);
+// Two FP32 values as a pair of 16-bit floats in one word (first value in the low half), round
+// to nearest even: one v_cvt_pk_bf16_f32 for bfloat16, two conversions and a pack for half.
+__device__ __forceinline__ uint32_t to_bf16_pair(float low, float high) {
+  typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+  typedef float f32x2 __attribute__((ext_vector_type(2)));
+  const f32x2 values = {low, high};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(values, bf16x2));
 }
-__device__ __forceinline__ uint16_t to_f16_bits(float x) {
-  return __builtin_bit_cast(uint16_t, static_cast<_Float16>(x));
+__device__ __forceinline__ uint32_t to_f16_pair(float low, float high) {
+  typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+  const f16x2 values = {static_cast<_Float16>(low), static_cast<_Float16>(high)};
+  return __builtin_bit_cast(uint32_t, values);
+}
+__device__ __forceinline__ uint32_t to_output_pair(float low, float high, int out_dtype) {
+  return out_dtype == kF16 ? to_f16_pair(low, high) : to_bf16_pair(low, high);
 }
 
 // Copies 16 bytes per lane from global memory to LDS without touching VGPRs:
@@ -528,7 +536,11 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void attention_kernel(cons
     float tile_m;
     uint32_t row_sum = 0;
 
-    if constexpr (FAST && !LAST) {
+    // Raw scores of a tile without keys past the end: maxima of the seeded integers, one FMA
+    // per score.  FLOORED applies the last-tile rule that a scale group's maximum starts from
+    // -50000 (a clamp of the converted maximum: the conversion is exact and monotone).
+    auto raw_score_tile = [&](auto floored_tag) {
+      constexpr bool FLOORED = decltype(floored_tag)::value;
       int mx0 = s[0][0], mx1 = s[0][2];
 #pragma unroll
       for (int rb = 0; rb < RB; ++rb)
@@ -539,8 +551,12 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void attention_kernel(cons
           else
             mx0 = max(mx0, s[rb][i]);
         }
-      tile_m = __builtin_fmaxf(__builtin_fmaf(score_value(mx0), sc0, -kU8Offset),
-                               __builtin_fmaf(score_value(mx1), sc1, -kU8Offset));
+      float top0 = score_value(mx0), top1 = score_value(mx1);
+      if constexpr (FLOORED) {
+        top0 = __builtin_fmaxf(kRowFloor, top0);
+        top1 = __builtin_fmaxf(kRowFloor, top1);
+      }
+      tile_m = __builtin_fmaxf(__builtin_fmaf(top0, sc0, -kU8Offset), __builtin_fmaf(top1, sc1, -kU8Offset));
       tile_m = max_across_halves(tile_m);
       const float neg_m = -tile_m;
 #pragma unroll
@@ -556,6 +572,12 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void attention_kernel(cons
           row_sum = __builtin_amdgcn_udot4(packed, 0x01010101u, row_sum, false);
           pk[rb][b4] = static_cast<int>(packed ^ 0x80808080u);
         }
+    };
+    if constexpr (FAST && !LAST) {
+      raw_score_tile(std::false_type{});
+    } else if (FAST && (tile + 1) * CTA_K <= p.k_len) {
+      // the last listed tile, all of its keys in range: the same values as the formulas below
+      raw_score_tile(std::true_type{});
     } else if constexpr (FAST) {
       // Last listed tile of the raw-score path: out-of-range keys become -1e30
       // and every scale group's maximum starts from -50000 before scaling.
@@ -1043,15 +1065,11 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void attention_kernel(cons
         value[1] = __builtin_fmaf(o_acc[cb][b4 * 4 + 1] * inv_d, scale4.y, center4.y);
         value[2] = __builtin_fmaf(o_acc[cb][b4 * 4 + 2] * inv_d, scale4.z, center4.z);
         value[3] = __builtin_fmaf(o_acc[cb][b4 * 4 + 3] * inv_d, scale4.w, center4.w);
-        uint32_t bits[4];
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const float x = zero_row ? 0.0f : value[r];
-          bits[r] = p.out_dtype == kF16 ? to_f16_bits(x) : to_bf16_bits(x);
-        }
+        for (int r = 0; r < 4; ++r) value[r] = zero_row ? 0.0f : value[r];
         uint2 word;
-        word.x = bits[0] | (bits[1] << 16);
-        word.y = bits[2] | (bits[3] << 16);
+        word.x = to_output_pair(value[0], value[1], p.out_dtype);
+        word.y = to_output_pair(value[2], value[3], p.out_dtype);
         *reinterpret_cast<uint2*>(out_row + 2 * c) = word;
       }
     if (p.lse != nullptr && half == 0) {

@@ -480,6 +480,23 @@ __global__ __launch_bounds__(64 * WAVES * KSPLIT) void attention_narrow_kernel(c
         }
       tile_m = __builtin_fmaxf(__builtin_fmaf(score_value(mx0), sc0, -kU8Offset),
                                __builtin_fmaf(score_value(mx1), sc1, -kU8Offset));
+    } else if ((tile + 1) * CTA_K <= p.k_len) {
+      // Last listed tile with all of its keys in range: the values of the formulas below from
+      // the maxima of the seeded integers (the conversion is exact and monotone, the floor of
+      // -50000 becomes a clamp of the converted maximum).
+      int mx0 = s[0][0], mx1 = s[0][2];
+#pragma unroll
+      for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          if (i & 2)
+            mx1 = max(mx1, s[kb][i]);
+          else
+            mx0 = max(mx0, s[kb][i]);
+          s[kb][i] = __float_as_int(score_value(s[kb][i]));
+        }
+      tile_m = __builtin_fmaxf(__builtin_fmaf(__builtin_fmaxf(kRowFloor, score_value(mx0)), sc0, -kU8Offset),
+                               __builtin_fmaf(__builtin_fmaxf(kRowFloor, score_value(mx1)), sc1, -kU8Offset));
     } else {
       // Last tile: out-of-range keys become -1e30 and every scale group's maximum
       // starts from -50000 before scaling.
@@ -723,15 +740,11 @@ __global__ __launch_bounds__(64 * WAVES * KSPLIT) void attention_narrow_kernel(c
       value[1] = __builtin_fmaf(o_acc[cb][1] * inv_d, scale4.y, center4.y);
       value[2] = __builtin_fmaf(o_acc[cb][2] * inv_d, scale4.z, center4.z);
       value[3] = __builtin_fmaf(o_acc[cb][3] * inv_d, scale4.w, center4.w);
-      uint32_t bits[4];
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const float x = zero_row ? 0.0f : value[r];
-        bits[r] = p.out_dtype == kF16 ? to_f16_bits(x) : to_bf16_bits(x);
-      }
+      for (int r = 0; r < 4; ++r) value[r] = zero_row ? 0.0f : value[r];
       uint2 word;
-      word.x = bits[0] | (bits[1] << 16);
-      word.y = bits[2] | (bits[3] << 16);
+      word.x = to_output_pair(value[0], value[1], p.out_dtype);
+      word.y = to_output_pair(value[2], value[3], p.out_dtype);
       *reinterpret_cast<uint2*>(out_row + 2 * c) = word;
     }
     if (p.lse != nullptr && grp == 0) {
