@@ -241,6 +241,22 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void attention_kernel(cons
   const int query = bx * kQueryBlock + wave * 32 + l32;
   const bool query_ok = query < p.q_len;
 
+  // --- Q operand and scales ------------------------------------------------
+  // Requested before the tile list is read: the list's first entries are needed at once and
+  // would otherwise keep these loads waiting behind their round trip.
+  v4i qreg[KK];
+  {
+    const int8_t* q_row = p.q + (bhq * p.q_len + query) * D;
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) {
+      qreg[kk] = query_ok ? *reinterpret_cast<const v4i*>(q_row + kk * 32 + half * 16) : v4i{0, 0, 0, 0};
+    }
+  }
+  constexpr int W = D == 256 ? 16 : 32;
+  const int q_groups = (p.q_len + 127) / 128 * (128 / W) * 8;
+  const float q_scale = query_ok ? p.q_scale[bhq * q_groups + (query / W) * 8 + (query & 7)] : 1.0f;
+  const float qs2 = p.sm2;
+
   // --- tile list -----------------------------------------------------------
   int n_it;
   const int32_t* indices = nullptr;
@@ -383,20 +399,6 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void attention_kernel(cons
       }
     }
   };
-
-  // --- Q operand and scales ------------------------------------------------
-  v4i qreg[KK];
-  {
-    const int8_t* q_row = p.q + (bhq * p.q_len + query) * D;
-#pragma unroll
-    for (int kk = 0; kk < KK; ++kk) {
-      qreg[kk] = query_ok ? *reinterpret_cast<const v4i*>(q_row + kk * 32 + half * 16) : v4i{0, 0, 0, 0};
-    }
-  }
-  constexpr int W = D == 256 ? 16 : 32;
-  const int q_groups = (p.q_len + 127) / 128 * (128 / W) * 8;
-  const float q_scale = query_ok ? p.q_scale[bhq * q_groups + (query / W) * 8 + (query & 7)] : 1.0f;
-  const float qs2 = p.sm2;
 
   float o_acc[CB][16];
 #pragma unroll
