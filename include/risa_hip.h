@@ -139,7 +139,8 @@ void risa_unpack_order(int32_t* order);
  * risa_sdpa_prequantized (csrc/bindings.cpp:277-461).
  *   q_int8/k_int8 contiguous [B,H,L,D]; v_int8 [B*Hkv*D, padded];
  *   out [B,Hq,Lq,D] fp16/bf16 with the given batch/token/head strides (last
- *   dim contiguous); mask (nullable) expanded to [B,Hq,Lq,Lk] with its strides,
+ *   dim contiguous; base 16-byte aligned, strides multiples of 8 elements: rows
+ *   are written 16 bytes per lane); mask (nullable) expanded to [B,Hq,Lq,Lk] with its strides,
  *   query stride 0 selecting the key-only path; sparse_row_offsets int32
  *   [B*Hq*ceil(Lq/128)+1] and sparse_block_indices int32 (both or neither);
  *   block_mass (nullable) float32 workspace laid out as mass

@@ -92,6 +92,9 @@ int launch_attention(const AttentionArgs& a, hipStream_t stream) {
   if (capture && sparse) return fail("risa_attention: block mass requires dense attention");
   if (a.v_tile_sum == nullptr) return fail("risa_attention: V tile sums are required");
   if (a.q_heads % a.kv_heads != 0) return fail("risa_attention: head counts are incompatible");
+  // output rows leave the kernels in 16-byte pieces
+  if (reinterpret_cast<uintptr_t>(a.out) % 16 != 0 || ((a.out_stride_b | a.out_stride_h | a.out_stride_n) & 7) != 0)
+    return fail("risa_attention: the output must be 16-byte aligned, with strides that are multiples of 8 elements");
   const int64_t padded_keys = static_cast<int64_t>((a.k_len + a.cta_k - 1) / a.cta_k) * a.cta_k;
   if (padded_keys * a.head_dim >= (int64_t{1} << 32) || static_cast<int64_t>(a.k_len) * a.head_dim >= (int64_t{1} << 31))
     return fail("risa_attention: one head of K or V exceeds the 32-bit tile offsets of the kernel");

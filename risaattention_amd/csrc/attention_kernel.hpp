@@ -577,41 +577,23 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void attention_kernel(cons
     };
     if constexpr (FAST && !LAST) {
       raw_score_tile(std::false_type{});
-    } else if (FAST && (tile + 1) * CTA_K <= p.k_len) {
-      // the last listed tile, all of its keys in range: the same values as the formulas below
-      raw_score_tile(std::true_type{});
     } else if constexpr (FAST) {
-      // Last listed tile of the raw-score path: out-of-range keys become -1e30
-      // and every scale group's maximum starts from -50000 before scaling.
-      float mx0 = kRowFloor, mx1 = kRowFloor;
+      // Last listed tile of the raw-score path: every scale group's maximum starts from
+      // -50000, and keys past the end count as -1e30.  Their seeded scores are replaced by
+      // the bit pattern of -1e30: a negative integer, so it never wins the integer maximum
+      // (a group made of such keys alone ends at the -50000 clamp), and removing the seed
+      // from it leaves -1e30 exactly.
+      if ((tile + 1) * CTA_K > p.k_len) {
+        constexpr int kPastEndBits = static_cast<int>(0xF149F2CAu);  // -1e30f
 #pragma unroll
-      for (int rb = 0; rb < RB; ++rb)
+        for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          const int key = key0 + rb * 32 + (i >> 2) * 8 + (i & 3);
-          const float raw = key < p.k_len ? score_value(s[rb][i]) : -1.0e30f;
-          s[rb][i] = __float_as_int(raw);
-          if (i & 2)
-            mx1 = __builtin_fmaxf(mx1, raw);
-          else
-            mx0 = __builtin_fmaxf(mx0, raw);
-        }
-      tile_m = __builtin_fmaxf(__builtin_fmaf(mx0, sc0, -kU8Offset), __builtin_fmaf(mx1, sc1, -kU8Offset));
-      tile_m = max_across_halves(tile_m);
-      const float neg_m = -tile_m;
-#pragma unroll
-      for (int rb = 0; rb < RB; ++rb)
-#pragma unroll
-        for (int b4 = 0; b4 < 4; ++b4) {
-          uint32_t packed = 0;
-#pragma unroll
-          for (int r = 0; r < 4; ++r) {
-            const float x = __builtin_fmaf(__int_as_float(s[rb][b4 * 4 + r]), (r & 2) ? sc1 : sc0, neg_m);
-            packed = __builtin_amdgcn_cvt_pk_u8_f32(__builtin_amdgcn_exp2f(x), r, packed);
+          for (int i = 0; i < 16; ++i) {
+            const int key = key0 + rb * 32 + (i >> 2) * 8 + (i & 3);
+            s[rb][i] = key < p.k_len ? s[rb][i] : kPastEndBits;
           }
-          row_sum = __builtin_amdgcn_udot4(packed, 0x01010101u, row_sum, false);
-          pk[rb][b4] = static_cast<int>(packed ^ 0x80808080u);
-        }
+      }
+      raw_score_tile(std::true_type{});
     } else {
       // Pre-scaled scores with masks.  Whether a tile needs any masking at all is
       // uniform over the wavefront: tiles below the causal diagonal, inside the key
@@ -972,11 +954,17 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void attention_kernel(cons
     load_lane_words(tile, 0);
     float ks0 = ks_base[tile * 4 + 2 * half];
     float ks1 = ks_base[tile * 4 + 2 * half + 1];
+    // Listed tiles: the entry after the next one is requested a whole tile before it is
+    // needed, ahead of the copies (read where it is needed, its round trip would be
+    // waited for in every tile).
+    [[maybe_unused]] int listed_next = INDEXED && n_it > 1 ? tile_at(1) : 0;
     for (int it = 0; it < n_it - 1; ++it) {
       const int stage = it & 1;
-      const int next_tile = tile_at(it + 1);
+      const int next_tile = INDEXED ? listed_next : it + 1;
       __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
       __syncthreads();
+      [[maybe_unused]] int listed_after_next = 0;
+      if constexpr (INDEXED) listed_after_next = indices[min(it + 2, n_it - 1)];
       load_k_fragments(lds + stage * Shape::kStageBytes, 0, k_first);
       if constexpr (PRELOAD) {
         load_mask_words(tile);
@@ -1023,6 +1011,7 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void attention_kernel(cons
       tile = next_tile;
       ks0 = next_ks0;
       ks1 = next_ks1;
+      if constexpr (INDEXED) listed_next = __builtin_amdgcn_readfirstlane(listed_after_next);
     }
     const int stage = (n_it - 1) & 1;
     __builtin_amdgcn_s_waitcnt(0x0f70);
@@ -1036,8 +1025,8 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void attention_kernel(cons
   }
 
   // ---- epilogue --------------------------------------------------------------
-  const float d_total = d_part + __shfl_xor(d_part, 32);
   if constexpr (CAPTURE) {
+    const float d_total = d_part + __shfl_xor(d_part, 32);
     if (half == 0 && query_ok) {
       const uint64_t query_rows = static_cast<uint64_t>(p.batch) * p.q_heads * p.q_len;
       float* state = reinterpret_cast<float*>(stats + full_words + query_rows * 2);
@@ -1045,39 +1034,57 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void attention_kernel(cons
       state[stat_row * 2 + 1] = d_total;
     }
   }
+  // A lane owns one query and, per instruction, four channels of it: stored from there, an
+  // instruction would write 16 bytes into each of 32 rows, and a launch with short tile
+  // lists spends more time on such stores than on its tiles (40 heads x 32K tokens, one
+  // listed tile per query block: 155 of 264 us).  The rows go through LDS instead (every
+  // wavefront has left the tiles by then; 64 * D bytes per wavefront) and leave as whole
+  // rows, 16 bytes per lane.
+  __syncthreads();  // no wavefront reads a tile any more
+  constexpr int ROW_BYTES = D * 2;
+  constexpr int CHUNKS = ROW_BYTES / 16;  // 16-byte pieces of a row
+  constexpr int ROWS_PER_STORE = 64 / CHUNKS;
+  constexpr int STORES = 32 / ROWS_PER_STORE;
+  const float d_total = d_part + __shfl_xor(d_part, 32);
   const bool guard_empty = !FAST && (MASK_DT >= 0 || p.causal);
   const bool row_valid = d_total > 0.0f;
   const float inv_d = 1.0f / d_total;
-  if (query_ok) {
-    const float* vs = p.v_scale + bhk * D;
-    const float* vc = p.v_center + bhk * D;
-    unsigned char* out_row = static_cast<unsigned char*>(p.out) +
+  const bool zero_row = guard_empty && !row_valid;
+  unsigned char* mine = lds + wave * (32 * ROW_BYTES);
+  const int first_query = bx * kQueryBlock + wave * 32;
+  unsigned char* out_block = static_cast<unsigned char*>(p.out) +
                              2 * (batch * p.out_stride_b + head * p.out_stride_h +
-                                  static_cast<int64_t>(query) * p.out_stride_n);
-    const bool zero_row = guard_empty && !row_valid;
+                                  static_cast<int64_t>(first_query) * p.out_stride_n);
 #pragma unroll
-    for (int cb = 0; cb < CB; ++cb)
+  for (int cb = 0; cb < CB; ++cb)
 #pragma unroll
-      for (int b4 = 0; b4 < 4; ++b4) {
-        const int c = cb * 32 + b4 * 8 + half * 4;
-        const float4 scale4 = *reinterpret_cast<const float4*>(vs + c);
-        const float4 center4 = *reinterpret_cast<const float4*>(vc + c);
-        float value[4];
-        value[0] = __builtin_fmaf(o_acc[cb][b4 * 4 + 0] * inv_d, scale4.x, center4.x);
-        value[1] = __builtin_fmaf(o_acc[cb][b4 * 4 + 1] * inv_d, scale4.y, center4.y);
-        value[2] = __builtin_fmaf(o_acc[cb][b4 * 4 + 2] * inv_d, scale4.z, center4.z);
-        value[3] = __builtin_fmaf(o_acc[cb][b4 * 4 + 3] * inv_d, scale4.w, center4.w);
+    for (int b4 = 0; b4 < 4; ++b4) {
+      const int c = cb * 32 + b4 * 8 + half * 4;
+      const v4f scale4 = *reinterpret_cast<const v4f*>(p.v_scale + bhk * D + c);
+      const v4f center4 = *reinterpret_cast<const v4f*>(p.v_center + bhk * D + c);
+      float value[4];
 #pragma unroll
-        for (int r = 0; r < 4; ++r) value[r] = zero_row ? 0.0f : value[r];
-        uint2 word;
-        word.x = to_output_pair(value[0], value[1], p.out_dtype);
-        word.y = to_output_pair(value[2], value[3], p.out_dtype);
-        *reinterpret_cast<uint2*>(out_row + 2 * c) = word;
+      for (int r = 0; r < 4; ++r) {
+        value[r] = __builtin_fmaf(o_acc[cb][b4 * 4 + r] * inv_d, scale4[r], center4[r]);
+        value[r] = zero_row ? 0.0f : value[r];
       }
-    if (p.lse != nullptr && half == 0) {
-      p.lse[bhq * p.q_len + query] =
-          row_valid ? (__builtin_amdgcn_logf(d_total) + m_run) / kLog2e : -__builtin_inff();
+      typedef uint32_t v2u __attribute__((ext_vector_type(2)));
+      v2u word;
+      word.x = to_output_pair(value[0], value[1], p.out_dtype);
+      word.y = to_output_pair(value[2], value[3], p.out_dtype);
+      *reinterpret_cast<v2u*>(mine + swizzled<ROW_BYTES>(l32, cb * 4 + b4) + half * 8) = word;
     }
+#pragma unroll
+  for (int i = 0; i < STORES; ++i) {
+    const int row = i * ROWS_PER_STORE + lane / CHUNKS, chunk = lane % CHUNKS;
+    const v4i piece = *reinterpret_cast<const v4i*>(mine + swizzled<ROW_BYTES>(row, chunk));
+    if (first_query + row < p.q_len) {
+      *reinterpret_cast<v4i*>(out_block + 2 * static_cast<int64_t>(row) * p.out_stride_n + chunk * 16) = piece;
+    }
+  }
+  if (p.lse != nullptr && half == 0 && query_ok) {
+    p.lse[bhq * p.q_len + query] =
+        row_valid ? (__builtin_amdgcn_logf(d_total) + m_run) / kLog2e : -__builtin_inff();
   }
 }
 
