@@ -1074,6 +1074,7 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void attention_kernel(cons
       word.y = to_output_pair(value[2], value[3], p.out_dtype);
       *reinterpret_cast<v2u*>(mine + swizzled<ROW_BYTES>(l32, cb * 4 + b4) + half * 8) = word;
     }
+  asm volatile("" ::: "memory");  // the pieces below are read from other lanes' writes
 #pragma unroll
   for (int i = 0; i < STORES; ++i) {
     const int row = i * ROWS_PER_STORE + lane / CHUNKS, chunk = lane % CHUNKS;

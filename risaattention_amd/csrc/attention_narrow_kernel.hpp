@@ -629,11 +629,16 @@ __global__ __launch_bounds__(64 * WAVES * KSPLIT) void attention_narrow_kernel(c
     float ks0, ks1;
     int tile = tile_at(0);
     issue_tile(tile, 0);
+    // Listed tiles: the entry after the next one is requested a whole tile before it is
+    // needed, ahead of the copies (its round trip would otherwise be waited for in every tile).
+    [[maybe_unused]] int listed_next = INDEXED && n_it > 1 ? tile_at(1) : 0;
     for (int step = 0; step < n_it - 1; ++step) {
       const int stage = step & 1;
-      const int next_tile = tile_at(step + 1);
+      const int next_tile = INDEXED ? listed_next : tile_at(step + 1);
       __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
       __syncthreads();
+      [[maybe_unused]] int listed_after_next = 0;
+      if constexpr (INDEXED) listed_after_next = indices[min(step + 2, n_it - 1)];
       load_k_fragments(lds + stage * Shape::kStageBytes, 0, k_first);
       tile_scales(stage, ks0, ks1);
       if constexpr (PRELOAD) {
@@ -655,6 +660,7 @@ __global__ __launch_bounds__(64 * WAVES * KSPLIT) void attention_narrow_kernel(c
       }
       value_tile(stage, pk, acc_first, v_first, t_scale);
       tile = next_tile;
+      if constexpr (INDEXED) listed_next = __builtin_amdgcn_readfirstlane(listed_after_next);
     }
     const int stage = (n_it - 1) & 1;
     __builtin_amdgcn_s_waitcnt(0x0f70);
@@ -724,6 +730,12 @@ __global__ __launch_bounds__(64 * WAVES * KSPLIT) void attention_narrow_kernel(c
   const float inv_d = 1.0f / d_total;
   // rows without any visible key (masks, causal): zeros
   const bool zero_row = GENERAL && (MASK_DT >= 0 || p.causal) && !(d_total > 0.0f);
+  // A lane owns one query and four channels per 16-channel block: stored from there, an
+  // instruction would write 32 bytes into each of 16 rows.  Two blocks are exchanged between
+  // neighbouring rows of lanes first (v_permlane16_swap: the odd rows of one register for the
+  // even rows of the other), after which a lane holds eight consecutive channels and an
+  // instruction writes 64 contiguous bytes of each row.  (The four lanes of a query are
+  // active or inactive together, so the exchange stays inside the branch.)
   if (query_ok) {
     const float* vs = p.v_scale + bhk * D;
     const float* vc = p.v_center + bhk * D;
@@ -731,21 +743,29 @@ __global__ __launch_bounds__(64 * WAVES * KSPLIT) void attention_narrow_kernel(c
                              2 * (batch * p.out_stride_b + head * p.out_stride_h +
                                   static_cast<int64_t>(query) * p.out_stride_n);
 #pragma unroll
-    for (int cb = 0; cb < CB; ++cb) {
-      const int c = cb * 16 + grp * 4;
-      const float4 scale4 = *reinterpret_cast<const float4*>(vs + c);
-      const float4 center4 = *reinterpret_cast<const float4*>(vc + c);
-      float value[4];
-      value[0] = __builtin_fmaf(o_acc[cb][0] * inv_d, scale4.x, center4.x);
-      value[1] = __builtin_fmaf(o_acc[cb][1] * inv_d, scale4.y, center4.y);
-      value[2] = __builtin_fmaf(o_acc[cb][2] * inv_d, scale4.z, center4.z);
-      value[3] = __builtin_fmaf(o_acc[cb][3] * inv_d, scale4.w, center4.w);
+    for (int cb = 0; cb < CB; cb += 2) {
+      uint32_t word[2][2];  // [block of the pair][channel pair]
 #pragma unroll
-      for (int r = 0; r < 4; ++r) value[r] = zero_row ? 0.0f : value[r];
-      uint2 word;
-      word.x = to_output_pair(value[0], value[1], p.out_dtype);
-      word.y = to_output_pair(value[2], value[3], p.out_dtype);
-      *reinterpret_cast<uint2*>(out_row + 2 * c) = word;
+      for (int j = 0; j < 2; ++j) {
+        const int c = (cb + j) * 16 + grp * 4;
+        const v4f scale4 = *reinterpret_cast<const v4f*>(vs + c);
+        const v4f center4 = *reinterpret_cast<const v4f*>(vc + c);
+        float value[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          value[r] = __builtin_fmaf(o_acc[cb + j][r] * inv_d, scale4[r], center4[r]);
+          value[r] = zero_row ? 0.0f : value[r];
+        }
+        word[j][0] = to_output_pair(value[0], value[1], p.out_dtype);
+        word[j][1] = to_output_pair(value[2], value[3], p.out_dtype);
+      }
+      // even rows of lanes end with channels 8*(grp/2) .. +7 of the first block, odd rows
+      // with the same channels of the second block
+      const auto low = __builtin_amdgcn_permlane16_swap(word[0][0], word[1][0], false, false);
+      const auto high = __builtin_amdgcn_permlane16_swap(word[0][1], word[1][1], false, false);
+      const v4i piece = {static_cast<int>(low[0]), static_cast<int>(high[0]), static_cast<int>(low[1]),
+                         static_cast<int>(high[1])};
+      *reinterpret_cast<v4i*>(out_row + (cb + (grp & 1)) * 32 + (grp >> 1) * 16) = piece;
     }
     if (p.lse != nullptr && grp == 0) {
       p.lse[bhq * p.q_len + query] =
