@@ -3,6 +3,7 @@ relative L2 (the tolerance the task states for floating-point results), plus the
 closed-form contracts of the reference's own CUDA tests."""
 
 from dataclasses import replace
+import math
 
 import numpy as np
 import pytest
@@ -523,3 +524,38 @@ def test_shared_boolean_mask_in_the_sparse_path(risa, dim):
     lists = (row_offsets, pattern.block_indices.cpu().numpy()[:row_offsets[-1]])
     expected_reuse, _, _ = oracle_pipeline.attend(prepared, pattern=lists)
     assert relative_l2(to_numpy(reuse[:, :4]), expected_reuse) < TOLERANCE
+
+
+@pytest.mark.parametrize("dim", [64, 128, 256])
+@pytest.mark.parametrize("heads,q_len", [(3, 77), (130, 200)])
+def test_output_rows_in_both_layouts_and_misaligned_outputs(risa, dim, heads, q_len):
+    """Output rows are written 16 bytes per lane, whole rows at a time (both kernels:
+    the few-workgroup launch and the large one).  The sequence-major layout must hold the
+    same values as the head-major one, rows past a ragged query length must stay untouched,
+    and an output that is not 16-byte aligned is refused instead of written."""
+    from risaattention_amd.attend import launch_attention
+
+    q = seeded((2, heads, q_len, dim), torch.bfloat16, 71)
+    k = seeded((2, 1, 300, dim), torch.bfloat16, 72)
+    v = seeded((2, 1, 300, dim), torch.bfloat16, 73, offset=0.25)
+    packed = risa.prequantize_int8_attention(q, k, v)
+    head_major = risa.int8_attention_from_prequantized(packed)
+    sequence_major = risa.int8_attention_from_prequantized(packed, output_layout="nhd")
+    assert sequence_major.transpose(1, 2).is_contiguous()
+    assert torch.equal(head_major, sequence_major)
+    expected, _, _ = oracle_pipeline.attend(oracle_prequantize(q[:1, :2], k[:1], v[:1]))
+    assert relative_l2(to_numpy(head_major[:1, :2]), expected) < TOLERANCE
+
+    # written through the wrapper into a buffer with a sentinel tail: nothing lands past the
+    # last row, and the same buffer shifted by 8 bytes is refused
+    shape = tuple(head_major.shape[:3]) + (packed.q.shape[-1],)
+    count = math.prod(shape)
+    buffer = torch.full((count + 64,), 7.0, dtype=torch.bfloat16, device="cuda")
+    arguments = dict(q_codes=packed.q, k_codes=packed.k, v_codes=packed.v, q_scale=packed.q_scale,
+                     k_scale=packed.k_scale, v_scale=packed.v_scale, v_center=packed.v_center, v_tile_sum=None,
+                     cta_k=packed.cta_k, sm_scale=packed.attention_scale)
+    launch_attention(output=buffer[:count].view(shape), **arguments)
+    assert torch.equal(buffer[:count].view(shape)[..., : head_major.shape[-1]], head_major)
+    assert torch.equal(buffer[count:], torch.full_like(buffer[count:], 7.0))
+    with pytest.raises(RuntimeError, match="16-byte aligned"):
+        launch_attention(output=buffer[4 : count + 4].view(shape), **arguments)
