@@ -355,3 +355,44 @@ def test_reuse_matches_oracle_at_every_launch_size(risa, dim, k_len):
         out = risa.sparse_int8_attention(q_all[:, :heads], k, v, pattern_for(heads))
         assert relative_l2(to_numpy(out[:, :oracle_heads]), expected) < 1e-3, heads
         assert relative_l2(to_numpy(out), to_numpy(largest[:, :heads])) < 1e-4, heads
+
+
+@pytest.mark.parametrize("dim", [64, 128, 256])
+@pytest.mark.parametrize("heads,output_dtype", [(2, torch.bfloat16), (130, torch.float16)])
+def test_short_tile_lists_match_oracle(risa, dim, heads, output_dtype):
+    """Hand-made lists of one to three tiles per query block, the partial tail tile among
+    them (always last: lists are ascending), through both kernels (few and many workgroups):
+    the listed tile after the next one is read a tile ahead, the last listed tile takes the
+    last-tile formulas, and keys past the end must not count."""
+    from risaattention_amd.types import RetainedMassPattern
+
+    q_len, k_len = 300, 1100
+    q = seeded((1, heads, q_len, dim), output_dtype, 81)
+    k = seeded((1, 1, k_len, dim), output_dtype, 82)
+    v = seeded((1, 1, k_len, dim), output_dtype, 83, offset=0.5)
+    packed = risa.prequantize_int8_attention(q, k, v, return_lse=True)
+    tiles = -(-k_len // packed.cta_k)
+    choices = [[tiles - 1], [0], [0, tiles - 1], [1, 2, tiles - 1], [tiles - 3, tiles - 2], [2]]
+    query_blocks = -(-q_len // 128)
+    lists = [choices[(head * query_blocks + block) % len(choices)] for head in range(heads) for block in range(query_blocks)]
+    offsets = np.cumsum([0] + [len(entry) for entry in lists]).astype(np.int32)
+    indices = np.concatenate(lists).astype(np.int32)
+    pattern = RetainedMassPattern(torch.from_numpy(offsets).cuda(), torch.from_numpy(indices).cuda(), 1, heads, q_len,
+                                  k_len, 128, packed.cta_k, packed.attention_scale, 0.5, 0.5)
+    out, lse = risa.int8_attention_from_prequantized(packed, sparse_pattern=pattern, return_lse=True)
+    checked = 2  # heads compared with the oracle
+    rows = checked * query_blocks
+    prepared = oracle_prequantize(q[:, :checked], k, v, return_lse=True)
+    expected, expected_lse, _ = oracle_pipeline.attend(prepared, pattern=(offsets[: rows + 1], indices[: offsets[rows]]),
+                                                       return_lse=True)
+    assert relative_l2(to_numpy(out[:, :checked]), expected) < 1e-3
+    assert relative_l2(to_numpy(lse[:, :checked]), expected_lse) < 1e-3
+    # heads with the same lists and inputs give the same rows whichever kernel ran
+    period = len(choices)
+    if heads > period * 2:
+        twin = risa.int8_attention_from_prequantized(
+            risa.prequantize_int8_attention(q[:, :2], k, v),
+            sparse_pattern=RetainedMassPattern(pattern.row_offsets[: rows + 1].clone(),
+                                               pattern.block_indices[: int(offsets[rows])].clone(), 1, 2, q_len, k_len,
+                                               128, packed.cta_k, packed.attention_scale, 0.5, 0.5))
+        assert relative_l2(to_numpy(twin), to_numpy(out[:, :2])) < 1e-4
