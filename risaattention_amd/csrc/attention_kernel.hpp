@@ -278,8 +278,14 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void attention_kernel(cons
     }
   }
   n_it = __builtin_amdgcn_readfirstlane(n_it);
+  // Entry `it` of the tile list through the scalar cache (the address is uniform): the first
+  // entries are needed before anything else can start, and as a vector load their wait would
+  // include the Q rows requested above (vector memory returns in order).
   auto tile_at = [&](int it) -> int {
-    if constexpr (INDEXED) return __builtin_amdgcn_readfirstlane(indices[it]);
+    if constexpr (INDEXED) {
+      typedef const __attribute__((address_space(4))) int32_t* UniformEntries;
+      return ((UniformEntries)(reinterpret_cast<uintptr_t>(indices)))[it];
+    }
     return it;
   };
 

@@ -143,8 +143,13 @@ __global__ __launch_bounds__(64 * WAVES * KSPLIT) void attention_narrow_kernel(c
       n_it = (limit + CTA_K - 1) / CTA_K;
     }
   }
+  // listed tiles come through the scalar cache (uniform address; as vector loads their wait
+  // would include every vector load requested before them)
   auto tile_at = [&](int step) -> int {
-    if constexpr (INDEXED) return __builtin_amdgcn_readfirstlane(indices[step]);
+    if constexpr (INDEXED) {
+      typedef const __attribute__((address_space(4))) int32_t* UniformEntries;
+      return ((UniformEntries)(reinterpret_cast<uintptr_t>(indices)))[step];
+    }
     return first_tile + step;
   };
 
