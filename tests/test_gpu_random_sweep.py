@@ -85,3 +85,51 @@ def test_random_configuration_matches_oracle(risa, seed):
     expected, expected_lse, _ = oracle_pipeline.attend(prepared, return_lse=True)
     assert relative_l2(to_numpy(out[:, :checked]), expected) < 1e-3
     assert relative_l2(to_numpy(lse[:, :checked]), expected_lse) < 1e-3
+
+
+def draw_preparation(seed):
+    rng = np.random.default_rng(5000 + seed)
+    kv_heads = int(rng.choice([1, 2, 3]))
+    return dict(
+        dim=int(rng.choice([40, 64, 96, 128, 256])),  # 40 and 96 are padded to 64 and 128
+        batch=int(rng.choice([1, 2])), kv_heads=kv_heads, heads=kv_heads * int(rng.choice([1, 2, 5])),
+        q_len=int(rng.integers(1, 500)), k_len=int(rng.choice([rng.integers(1, 900), rng.integers(4097, 6000)])),
+        dtype=DTYPES[int(rng.integers(0, 3))], mode=str(rng.choice(["absmax", "midpoint_affine"])),
+        key_offset=float(rng.choice([0.0, 0.0, 3.0])), layout=str(rng.choice(["hnd", "nhd"])),
+        query_mask=bool(rng.integers(0, 3) == 0),
+    )
+
+
+@pytest.mark.parametrize("seed", range(20))
+def test_random_preparation_matches_oracle_bit_for_bit(risa, seed):
+    """Codes, scales, centre, tile sums, anchor shift: bit for bit, over drawn shapes, padded
+    head dims, dtypes, V modes, memory layouts, shifted keys and both tile policies."""
+    from oracle import prepare as oracle_prepare
+    from risaattention_amd.layout import unpack_values
+
+    c = draw_preparation(seed)
+    print("configuration:", {key: str(value) for key, value in c.items()}, flush=True)
+
+    def tensor(heads, length, tensor_seed, **kwargs):
+        if c["layout"] == "nhd":  # sequence-major storage behind the [B,H,L,D] view
+            return seeded((c["batch"], length, heads, c["dim"]), c["dtype"], tensor_seed, **kwargs).transpose(1, 2)
+        return seeded((c["batch"], heads, length, c["dim"]), c["dtype"], tensor_seed, **kwargs)
+
+    q = tensor(c["heads"], c["q_len"], 7 * seed + 1)
+    k = tensor(c["kv_heads"], c["k_len"], 7 * seed + 2, offset=c["key_offset"], scale=0.2 if c["key_offset"] else 1.0)
+    v = tensor(c["kv_heads"], c["k_len"], 7 * seed + 3, offset=-0.7, scale=1.5)
+    mask = torch.ones((c["q_len"], c["k_len"]), dtype=torch.bool, device="cuda") if c["query_mask"] else None
+    packed = risa.prequantize_int8_attention(q, k, v, attn_mask=mask, v_quantization=c["mode"], return_lse=True)
+    expected = oracle_prequantize(q, k, v, attn_mask=mask, v_quantization=c["mode"], return_lse=True)
+    assert packed.cta_k == expected.cta_k
+    np.testing.assert_array_equal(packed.q.cpu().numpy(), expected.q)
+    np.testing.assert_array_equal(packed.q_scale.cpu().numpy(), expected.q_scale)
+    np.testing.assert_array_equal(packed.k.cpu().numpy(), expected.k)
+    np.testing.assert_array_equal(packed.k_scale.cpu().numpy(), expected.k_scale)
+    np.testing.assert_array_equal(unpack_values(packed.v).cpu().numpy(), expected.v)
+    np.testing.assert_array_equal(packed.v_scale.cpu().numpy(), expected.v_scale)
+    np.testing.assert_array_equal(packed.v_center.cpu().numpy(), expected.v_center)
+    sums = oracle_prepare.value_tile_sums(expected.v, expected.cta_k)
+    got = packed.v_tile_sum.cpu().numpy().transpose(0, 2, 1).reshape(expected.v.shape[0], -1)
+    np.testing.assert_array_equal(got, sums * 128 + 0x4B400000)
+    np.testing.assert_array_equal(to_numpy(packed.lse_shift), expected.lse_shift)
