@@ -133,3 +133,58 @@ def test_random_preparation_matches_oracle_bit_for_bit(risa, seed):
     got = packed.v_tile_sum.cpu().numpy().transpose(0, 2, 1).reshape(expected.v.shape[0], -1)
     np.testing.assert_array_equal(got, sums * 128 + 0x4B400000)
     np.testing.assert_array_equal(to_numpy(packed.lse_shift), expected.lse_shift)
+
+
+@pytest.mark.parametrize("seed", range(10))
+def test_random_sparse_construction_and_reuse_match_oracle(risa, seed):
+    """Pattern construction (outputs, selected tile sets up to mass ties, measured mass) and
+    reuse with the oracle's own pattern on drifted inputs, over drawn shapes and thetas."""
+    from dataclasses import replace
+
+    from oracle import attention as oracle_attention
+    from oracle import selection as oracle_selection
+
+    rng = np.random.default_rng(9000 + seed)
+    dim = int(rng.choice([64, 128, 256]))
+    kv_heads = int(rng.choice([1, 2]))
+    heads = kv_heads * int(rng.choice([1, 2, 3]))
+    q_len, k_len = int(rng.integers(129, 700)), int(rng.integers(1100, 1900))
+    theta = float(rng.choice([0.5, 0.9, 0.99]))
+    mode = str(rng.choice(["absmax", "midpoint_affine"]))
+    dtype = DTYPES[int(rng.integers(0, 2))]
+    print("configuration:", dim, heads, kv_heads, q_len, k_len, theta, mode, dtype, flush=True)
+    # keys in clusters so that the retained mass concentrates on some tiles
+    generator = torch.Generator(device="cpu").manual_seed(seed)
+    centres = torch.randn((1, kv_heads, 8, dim), generator=generator) * 2.5
+    k = (centres.repeat_interleave(-(-k_len // 8), dim=2)[:, :, :k_len]
+         + torch.randn((1, kv_heads, k_len, dim), generator=generator)).to(dtype).cuda()
+    picks = torch.randint(0, 8, (q_len,), generator=generator)
+    q = (centres[:, :, picks].repeat_interleave(heads // kv_heads, dim=1)
+         + torch.randn((1, heads, q_len, dim), generator=generator)).to(dtype).cuda()
+    v = torch.randn((1, kv_heads, k_len, dim), generator=generator).to(dtype).cuda()
+
+    out, pattern = risa.construct_sparse_int8_attention(q, k, v, theta=theta, v_quantization=mode)
+    prepared = oracle_prequantize(q, k, v, v_quantization=mode)
+    expected_out, _, captured = oracle_pipeline.attend(prepared, capture=True)
+    masses = oracle_attention.block_mass(captured, 1, heads, q_len)
+    row_offsets, block_indices, measured, _ = oracle_selection.select_retained_mass(masses, theta)
+    assert relative_l2(to_numpy(out), expected_out) < 1e-3
+    got_offsets = pattern.row_offsets.cpu().numpy()
+    got_indices = pattern.block_indices.cpu().numpy()
+    assert len(got_offsets) == len(row_offsets)
+    for row in range(len(row_offsets) - 1):
+        got = set(got_indices[got_offsets[row]:got_offsets[row + 1]].tolist())
+        want = set(block_indices[row_offsets[row]:row_offsets[row + 1]].tolist())
+        if got != want:  # only tiles whose mass ties with the cut may differ
+            cut = min(masses[row, tile] for tile in want)
+            for tile in got ^ want:
+                assert abs(masses[row, tile] - cut) <= 1e-4 * max(cut, 1e-6) + 1e-6, (row, tile)
+    assert pattern.measured_retained_mass == pytest.approx(measured, abs=1e-4)
+
+    drifted = [t + 0.05 * torch.randn(t.shape, generator=generator).to(t.dtype).cuda() for t in (q, k, v)]
+    oracle_pattern = replace(pattern, row_offsets=torch.from_numpy(row_offsets).cuda(),
+                             block_indices=torch.from_numpy(block_indices).cuda())
+    sparse = risa.sparse_int8_attention(*drifted, oracle_pattern, v_quantization=mode)
+    prepared_drifted = oracle_prequantize(*drifted, v_quantization=mode)
+    expected_sparse, _, _ = oracle_pipeline.attend(prepared_drifted, pattern=(row_offsets, block_indices))
+    assert relative_l2(to_numpy(sparse), expected_sparse) < 1e-3
