@@ -5,6 +5,7 @@ Host-side counterpart of reference src/risa_attention/_execution.py:28-328.
 
 from __future__ import annotations
 
+import functools
 import math
 
 import torch
@@ -163,6 +164,13 @@ def launch_attention(*, q_codes, k_codes, v_codes, output, q_scale, k_scale, v_s
     )
 
 
+@functools.lru_cache(maxsize=256)
+def sdpa_workspace_bytes(*extents) -> int:
+    """``risa_sdpa_workspace_bytes`` of the library (a pure function of its integer
+    arguments), remembered per argument tuple: serving loops ask for the same few shapes."""
+    return native.library().risa_sdpa_workspace_bytes(*extents)
+
+
 def execute_dense_attention(
     q: torch.Tensor,
     k: torch.Tensor,
@@ -209,9 +217,8 @@ def execute_dense_attention(
                      batch if attn_mask.stride(0) != 0 else 1, q_heads if attn_mask.stride(1) != 0 else 1)
     # the size query takes the mask's dtype, query and key strides and own extents
     workspace = torch.empty(
-        lib.risa_sdpa_workspace_bytes(batch, q_heads, q_len, kv_heads, k_len, dim, cta_k,
-                                      int(use_midpoint_affine), mask_args[5], mask_args[3], mask_args[4],
-                                      mask_args[6], mask_args[7]),
+        sdpa_workspace_bytes(batch, q_heads, q_len, kv_heads, k_len, dim, cta_k, int(use_midpoint_affine),
+                             mask_args[5], mask_args[3], mask_args[4], mask_args[6], mask_args[7]),
         dtype=torch.uint8, device=q.device)
     native.check(
         lib.risa_sdpa(

@@ -1,4 +1,5 @@
-// Q/K/V preparation in two launches (three beyond 4096 tokens).
+// Q/K/V preparation in two launches (three beyond 4096 tokens, one up to 1024 tokens with
+// absmax values).
 //
 // The separate preparation kernels (prep_qk.hip, prep_v.hip) are five to seven
 // launches whose order is fixed by data: anchor -> K codes, V range -> V parameters
@@ -70,7 +71,7 @@ __global__ __launch_bounds__(256) void prepare_stage2_kernel(const FusedArgs a) 
     const int part = block & 1;
     const int tile = (block >> 1) % a.key_tiles;
     const int rest = (block >> 1) / a.key_tiles;
-    quantize_k_block<DT, DK, CTA_K, ROT>(a.qk.k, a.qk.k_codes, a.qk.k_scale, a.qk.anchors, a.qk.k_len,
+    quantize_k_block<DT, DK, CTA_K, ROT>(a.qk.k, a.qk.k_codes, a.qk.k_scale, a.qk.anchors[rest], a.qk.k_len,
                                          a.qk.kv_heads, a.key_tiles * 4, a.qk.k_stride_b, a.qk.k_stride_h,
                                          a.qk.k_stride_n, a.k_wide, a.qk.permutation, tile, part,
                                          rest % a.qk.kv_heads, rest / a.qk.kv_heads);
@@ -103,8 +104,59 @@ __global__ __launch_bounds__(256) void prepare_stage2_kernel(const FusedArgs a) 
                                            a.v.permutation, fused, block % a.code_blocks_x, block / a.code_blocks_x);
 }
 
+// Short absmax problems in one launch: nothing waits for another workgroup.  A K workgroup
+// finds the anchor of its (batch, head) itself (nine sampled rows), a V workgroup walks the
+// whole sequence of its (batch, head) for the channel maxima; both repeat work that a first
+// launch would do once, which at this size costs less than the launch (about 5 us between two
+// dependent kernels).  Same device functions as the two-stage path: bit-identical tensors.
+template <int DT, int DK, int CTA_K, int ROT>
+__global__ __launch_bounds__(256) void prepare_single_kernel(const FusedArgs a) {
+  int block = blockIdx.x;
+  if (block < a.key_blocks) {
+    const int part = block & 1;
+    const int tile = (block >> 1) % a.key_tiles;
+    const int rest = (block >> 1) / a.key_tiles;
+    const int h = rest % a.qk.kv_heads, b = rest / a.qk.kv_heads;
+    const int anchor = detect_anchor_value<DT>(a.qk.k, a.qk.k_len, a.qk.head_dim, a.qk.kv_heads, a.qk.k_stride_b,
+                                               a.qk.k_stride_h, a.qk.k_stride_n, a.qk.permutation, h, b);
+    if (tile == 0 && part == 0 && threadIdx.x == 0) a.qk.anchors[rest] = anchor;  // for the LSE shift
+    quantize_k_block<DT, DK, CTA_K, ROT>(a.qk.k, a.qk.k_codes, a.qk.k_scale, anchor, a.qk.k_len, a.qk.kv_heads,
+                                         a.key_tiles * 4, a.qk.k_stride_b, a.qk.k_stride_h, a.qk.k_stride_n,
+                                         a.k_wide, a.qk.permutation, tile, part, h, b);
+    return;
+  }
+  block -= a.key_blocks;
+  const int code_blocks = a.code_blocks_x * a.kv;
+  if (block < code_blocks) {
+    const FusedParams fused{a.part_max, a.part_min, a.v.scale, a.v.center, a.inverse, a.midpoint, a.chunks};
+    value_codes_block<DT, CTA_K, kParamsWalk, DK>(a.v.v, a.v.codes, a.v.tile_sum, a.inverse, a.midpoint, a.v.length,
+                                                  a.v.padded, a.v.heads, a.v.stride_b, a.v.stride_h, a.v.stride_n,
+                                                  a.v.permutation, fused, block % a.code_blocks_x,
+                                                  block / a.code_blocks_x);
+    return;
+  }
+  block -= code_blocks;
+  const int slice = block % a.q_slices;
+  const int rest = block / a.q_slices;
+  quantize_q_block<DT, DK, ROT>(a.qk.q, a.qk.q_codes, a.qk.q_scale, a.qk.q_len, a.qk.q_heads,
+                                a.q_slices * 8, a.qk.q_stride_b, a.qk.q_stride_h, a.qk.q_stride_n,
+                                a.q_wide, slice, rest % a.qk.q_heads, rest / a.qk.q_heads);
+}
+
+// One launch while the repeated reads stay small: every V workgroup (128 positions) reads its
+// whole (batch, head), so V is read once per position block; up to 1024 tokens and 16 MiB of
+// such reads (out of L2) that is cheaper than a second launch.
+constexpr int kSingleLaunchMaxLength = 1024;
+constexpr int64_t kSingleLaunchMaxBytes = int64_t{16} << 20;
+
 template <int DT, int DK, int CTA_K, int ROT>
 void launch_stages(const FusedArgs& a, hipStream_t stream) {
+  const int64_t walked_bytes = static_cast<int64_t>(a.kv) * a.v.length * DK * (DT == kF32 ? 4 : 2) * a.code_blocks_x;
+  if (!a.v.midpoint_affine && a.v.length <= kSingleLaunchMaxLength && walked_bytes <= kSingleLaunchMaxBytes) {
+    const int blocks = a.key_blocks + a.code_blocks_x * a.kv + a.q_blocks;
+    prepare_single_kernel<DT, DK, CTA_K, ROT><<<blocks, 256, 0, stream>>>(a);
+    return;
+  }
   const int stage1_blocks = a.q_blocks + a.anchor_blocks + a.range_groups * a.kv;
   const bool stored_params = a.chunks > 64;
   const bool merged_center = a.v.midpoint_affine && !stored_params && a.v.length <= kFusedCenterMaxLength;

@@ -377,9 +377,8 @@ __global__ __launch_bounds__(256) void quantize_q_kernel(const void* __restrict_
 // CTA_K / 4, and twice as many wavefronts stand behind every tile.
 template <int DT, int DK, int CTA_K, int ROT>
 __device__ __forceinline__ void quantize_k_block(const void* __restrict__ k, int8_t* __restrict__ codes,
-                                                 float* __restrict__ scales,
-                                                 const int* __restrict__ anchors, int length, int heads,
-                                                 int scales_per_head, int64_t stride_b,
+                                                 float* __restrict__ scales, int anchor, int length,
+                                                 int heads, int scales_per_head, int64_t stride_b,
                                                  int64_t stride_h, int64_t stride_n, int wide,
                                                  const int32_t* __restrict__ permutation, int tile,
                                                  int part, int h, int b) {
@@ -391,7 +390,6 @@ __device__ __forceinline__ void quantize_k_block(const void* __restrict__ k, int
   const int first_index = (wave & 1) * NTOK;  // this wavefront's share of the group's CTA_K / 4 tokens
   const int64_t in_base = static_cast<int64_t>(b) * stride_b + static_cast<int64_t>(h) * stride_h;
   const int64_t bh = static_cast<int64_t>(b) * heads + h;
-  const int anchor = anchors[b * heads + h];
   const int32_t* source = permutation != nullptr ? permutation + bh * length : nullptr;
   // element offset of the anchor row (subtracted from every key) when one was chosen
   const int anchor_row = anchor >= 0 && source != nullptr ? source[anchor] : anchor;
@@ -414,9 +412,9 @@ __global__ __launch_bounds__(256) void quantize_k_kernel(const void* __restrict_
                                                          int64_t stride_b, int64_t stride_h,
                                                          int64_t stride_n, int wide,
                                                          const int32_t* __restrict__ permutation) {
-  quantize_k_block<DT, DK, CTA_K, ROT>(k, codes, scales, anchors, length, heads, scales_per_head,
-                                       stride_b, stride_h, stride_n, wide, permutation, blockIdx.x >> 1,
-                                       blockIdx.x & 1, blockIdx.y, blockIdx.z);
+  quantize_k_block<DT, DK, CTA_K, ROT>(k, codes, scales, anchors[blockIdx.z * heads + blockIdx.y], length, heads,
+                                       scales_per_head, stride_b, stride_h, stride_n, wide, permutation,
+                                       blockIdx.x >> 1, blockIdx.x & 1, blockIdx.y, blockIdx.z);
 }
 
 // ---------------------------------------------------------------------------
@@ -442,12 +440,11 @@ __device__ __forceinline__ float segment_down_sum(float value) {
 }
 __device__ __forceinline__ float segment_down_max(float value) { return half_wave_max(value); }
 
+// Returns the anchor row of (b, h), or -1, to every thread of the workgroup.
 template <int DT>
-__device__ __forceinline__ void detect_anchor_block(const void* __restrict__ k, int* __restrict__ anchors,
-                                                    int length, int dim, int heads, int64_t stride_b,
-                                                    int64_t stride_h, int64_t stride_n,
-                                                    const int32_t* __restrict__ permutation, int h,
-                                                    int b) {
+__device__ __forceinline__ int detect_anchor_value(const void* __restrict__ k, int length, int dim, int heads,
+                                                   int64_t stride_b, int64_t stride_h, int64_t stride_n,
+                                                   const int32_t* __restrict__ permutation, int h, int b) {
   __shared__ float samples[kSamples * 256];
   __shared__ float seg_energy[4], seg_max[4], seg_dist[kSamples][4], seg_best_energy[4],
       seg_best_max[4];
@@ -534,9 +531,20 @@ __device__ __forceinline__ void detect_anchor_block(const void* __restrict__ k, 
       m1 = __builtin_fmaxf(m1, seg_best_max[w]);
     }
     const bool improves = e1 < e0 && m1 <= m0 * 1.125f;
-    anchors[b * heads + h] =
-        improves ? static_cast<int>(static_cast<int64_t>(best) * (length - 1) / (kSamples - 1)) : -1;
+    chosen = improves ? static_cast<int>(static_cast<int64_t>(best) * (length - 1) / (kSamples - 1)) : -1;
   }
+  __syncthreads();
+  return chosen;
+}
+
+template <int DT>
+__device__ __forceinline__ void detect_anchor_block(const void* __restrict__ k, int* __restrict__ anchors,
+                                                    int length, int dim, int heads, int64_t stride_b,
+                                                    int64_t stride_h, int64_t stride_n,
+                                                    const int32_t* __restrict__ permutation, int h,
+                                                    int b) {
+  const int anchor = detect_anchor_value<DT>(k, length, dim, heads, stride_b, stride_h, stride_n, permutation, h, b);
+  if (threadIdx.x == 0) anchors[b * heads + h] = anchor;
 }
 
 

@@ -214,8 +214,10 @@ __global__ __launch_bounds__(256) void value_params_kernel(const float* __restri
 // what value_params_kernel left; kParamsAbsmax / kParamsAffine reduce the partial
 // ranges (at most 64 of them) inside every workgroup, one thread per channel, which saves a
 // launch for short sequences; the workgroups of the first 128 positions also store
-// the parameters for the kernels that follow.
-constexpr int kParamsStored = 0, kParamsAbsmax = 1, kParamsAffine = 2;
+// the parameters for the kernels that follow.  kParamsWalk (absmax, short sequences) takes
+// no partial ranges at all: every workgroup walks the whole sequence of its (batch, head)
+// for the channel maxima itself, which leaves the preparation without a launch to wait for.
+constexpr int kParamsStored = 0, kParamsAbsmax = 1, kParamsAffine = 2, kParamsWalk = 3;
 constexpr int kCodeBlockPositions = 128;
 
 struct FusedParams {
@@ -246,6 +248,7 @@ __device__ __forceinline__ void value_codes_block(const void* __restrict__ v, in
   __shared__ __attribute__((aligned(16))) uint32_t transposed[DK * PITCH];
   __shared__ float channel_inverse[DK], channel_midpoint[DK];
   [[maybe_unused]] __shared__ float partial_max[256 / DK][DK], partial_min[256 / DK][DK];
+  [[maybe_unused]] __shared__ float walked_max[PARAMS == kParamsWalk ? SLOTS : 1][DK];
   const int b = bh / heads, h = bh - b * heads;
   const int tid = threadIdx.x;
   const int octet = tid % OCTETS, slot = tid / OCTETS;
@@ -260,6 +263,46 @@ __device__ __forceinline__ void value_codes_block(const void* __restrict__ v, in
     for (int i = 0; i < 8; ++i) {
       inv[i] = inverse[row0 + octet * 8 + i];
       mid[i] = midpoint[row0 + octet * 8 + i];
+    }
+  } else if constexpr (PARAMS == kParamsWalk) {
+    // Thread (octet, slot) takes the rows slot, slot + SLOTS, ... of the whole sequence; rows
+    // past the end read the last one again (a repeated element does not change a maximum), so
+    // the loads sit in no branch.  The maximum does not depend on the order.
+    float mx[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) mx[i] = 0.0f;
+    const int passes = (length + SLOTS - 1) / SLOTS;
+#pragma unroll 8
+    for (int pass = 0; pass < passes; ++pass) {
+      const int n = min(pass * SLOTS + slot, length - 1);
+      float x[8];
+      load8<DT>(v, base + static_cast<int64_t>(n) * stride_n + octet * 8, x);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) mx[i] = __builtin_fmaxf(mx[i], __builtin_fabsf(x[i]));
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) walked_max[slot][octet * 8 + i] = mx[i];
+    __syncthreads();
+    if (tid < DK) {
+      float top = walked_max[0][tid];
+#pragma unroll
+      for (int part = 1; part < SLOTS; ++part) top = __builtin_fmaxf(top, walked_max[part][tid]);
+      const float sc = __builtin_fmaxf(top * (1.0f / 127.0f), 1e-12f);
+      const float reciprocal = 1.0f / sc;
+      channel_inverse[tid] = reciprocal;
+      channel_midpoint[tid] = 0.0f;
+      if (position_block == 0) {
+        fused.scale[row0 + tid] = sc;
+        fused.inverse[row0 + tid] = reciprocal;
+        fused.midpoint[row0 + tid] = 0.0f;
+        fused.center[row0 + tid] = 0.0f;
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      inv[i] = channel_inverse[octet * 8 + i];
+      mid[i] = channel_midpoint[octet * 8 + i];
     }
   } else {
     constexpr bool AFFINE = PARAMS == kParamsAffine;

@@ -121,16 +121,16 @@ def _require_device(device: torch.device) -> None:
 
 def validate_inputs(q, k, v, attn_mask):
     """Check Q, K, V and the mask; return the mask as a ``[B, Hq, Lq, Lk]`` broadcast view."""
-    operands = (q, k, v)
-    if any(t.ndim != 4 for t in operands):
+    if q.ndim != 4 or k.ndim != 4 or v.ndim != 4:
         raise _violation("rank")
-    if q.dtype not in DTYPE_CODES:
-        raise _violation("dtype", dtype=q.dtype)
-    if any(t.dtype != q.dtype for t in operands):
-        raise _violation("same_dtype", q=q.dtype, k=k.dtype, v=v.dtype)
-    if not q.is_cuda or any(t.device != q.device for t in operands):
+    dtype, device = q.dtype, q.device
+    if dtype not in DTYPE_CODES:
+        raise _violation("dtype", dtype=dtype)
+    if k.dtype != dtype or v.dtype != dtype:
+        raise _violation("same_dtype", q=dtype, k=k.dtype, v=v.dtype)
+    if not q.is_cuda or k.device != device or v.device != device:
         raise _violation("device")
-    _require_device(q.device)
+    _require_device(device)
 
     batch, q_heads, q_len, head_dim = q.shape
     kv_heads, k_len = k.shape[1], k.shape[2]
@@ -144,7 +144,7 @@ def validate_inputs(q, k, v, attn_mask):
         raise _violation("groups", q=q_heads, kv=kv_heads)
     if not 1 <= head_dim <= 256:
         raise _violation("head_dim", head_dim=head_dim)
-    if any(t.stride(-1) != 1 for t in operands):
+    if q.stride(-1) != 1 or k.stride(-1) != 1 or v.stride(-1) != 1:
         raise _violation("stride")
 
     if attn_mask is None:
