@@ -1,5 +1,4 @@
-// Q/K/V preparation in two launches (three beyond 4096 tokens, one up to 1024 tokens with
-// absmax values).
+// Q/K/V preparation in two launches (three beyond 4096 tokens, one up to 1024 tokens).
 //
 // The separate preparation kernels (prep_qk.hip, prep_v.hip) are five to seven
 // launches whose order is fixed by data: anchor -> K codes, V range -> V parameters
@@ -104,12 +103,12 @@ __global__ __launch_bounds__(256) void prepare_stage2_kernel(const FusedArgs a) 
                                            a.v.permutation, fused, block % a.code_blocks_x, block / a.code_blocks_x);
 }
 
-// Short absmax problems in one launch: nothing waits for another workgroup.  A K workgroup
+// Short problems in one launch: nothing waits for another workgroup.  A K workgroup
 // finds the anchor of its (batch, head) itself (nine sampled rows), a V workgroup walks the
 // whole sequence of its (batch, head) for the channel maxima; both repeat work that a first
 // launch would do once, which at this size costs less than the launch (about 5 us between two
 // dependent kernels).  Same device functions as the two-stage path: bit-identical tensors.
-template <int DT, int DK, int CTA_K, int ROT>
+template <int DT, int DK, int CTA_K, int ROT, bool AFFINE>
 __global__ __launch_bounds__(256) void prepare_single_kernel(const FusedArgs a) {
   int block = blockIdx.x;
   if (block < a.key_blocks) {
@@ -126,10 +125,20 @@ __global__ __launch_bounds__(256) void prepare_single_kernel(const FusedArgs a) 
     return;
   }
   block -= a.key_blocks;
+  const FusedParams fused{a.part_max, a.part_min, a.v.scale, a.v.center, a.inverse, a.midpoint, a.chunks};
+  if constexpr (AFFINE) {
+    // the centre blocks: each walks the whole sequence of its eight channels, twice
+    if (block < a.center_blocks) {
+      const int octets = a.v.head_dim / 8;
+      value_center_block<DT, true>(a.v.v, fused, a.v.length, a.v.head_dim, a.v.heads, a.v.stride_b, a.v.stride_h,
+                                   a.v.stride_n, a.v.permutation, block % octets, block / octets);
+      return;
+    }
+    block -= a.center_blocks;
+  }
   const int code_blocks = a.code_blocks_x * a.kv;
   if (block < code_blocks) {
-    const FusedParams fused{a.part_max, a.part_min, a.v.scale, a.v.center, a.inverse, a.midpoint, a.chunks};
-    value_codes_block<DT, CTA_K, kParamsWalk, DK>(a.v.v, a.v.codes, a.v.tile_sum, a.inverse, a.midpoint, a.v.length,
+    value_codes_block<DT, CTA_K, AFFINE ? kParamsWalkAffine : kParamsWalk, DK>(a.v.v, a.v.codes, a.v.tile_sum, a.inverse, a.midpoint, a.v.length,
                                                   a.v.padded, a.v.heads, a.v.stride_b, a.v.stride_h, a.v.stride_n,
                                                   a.v.permutation, fused, block % a.code_blocks_x,
                                                   block / a.code_blocks_x);
@@ -152,9 +161,16 @@ constexpr int64_t kSingleLaunchMaxBytes = int64_t{16} << 20;
 template <int DT, int DK, int CTA_K, int ROT>
 void launch_stages(const FusedArgs& a, hipStream_t stream) {
   const int64_t walked_bytes = static_cast<int64_t>(a.kv) * a.v.length * DK * (DT == kF32 ? 4 : 2) * a.code_blocks_x;
-  if (!a.v.midpoint_affine && a.v.length <= kSingleLaunchMaxLength && walked_bytes <= kSingleLaunchMaxBytes) {
-    const int blocks = a.key_blocks + a.code_blocks_x * a.kv + a.q_blocks;
-    prepare_single_kernel<DT, DK, CTA_K, ROT><<<blocks, 256, 0, stream>>>(a);
+  if (a.v.length <= kSingleLaunchMaxLength && walked_bytes <= kSingleLaunchMaxBytes) {
+    if (a.v.midpoint_affine) {
+      FusedArgs with_center = a;
+      with_center.center_blocks = a.kv * (a.v.head_dim / 8);
+      const int blocks = a.key_blocks + with_center.center_blocks + a.code_blocks_x * a.kv + a.q_blocks;
+      prepare_single_kernel<DT, DK, CTA_K, ROT, true><<<blocks, 256, 0, stream>>>(with_center);
+    } else {
+      const int blocks = a.key_blocks + a.code_blocks_x * a.kv + a.q_blocks;
+      prepare_single_kernel<DT, DK, CTA_K, ROT, false><<<blocks, 256, 0, stream>>>(a);
+    }
     return;
   }
   const int stage1_blocks = a.q_blocks + a.anchor_blocks + a.range_groups * a.kv;

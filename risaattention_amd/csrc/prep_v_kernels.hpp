@@ -214,10 +214,11 @@ __global__ __launch_bounds__(256) void value_params_kernel(const float* __restri
 // what value_params_kernel left; kParamsAbsmax / kParamsAffine reduce the partial
 // ranges (at most 64 of them) inside every workgroup, one thread per channel, which saves a
 // launch for short sequences; the workgroups of the first 128 positions also store
-// the parameters for the kernels that follow.  kParamsWalk (absmax, short sequences) takes
-// no partial ranges at all: every workgroup walks the whole sequence of its (batch, head)
-// for the channel maxima itself, which leaves the preparation without a launch to wait for.
-constexpr int kParamsStored = 0, kParamsAbsmax = 1, kParamsAffine = 2, kParamsWalk = 3;
+// the parameters for the kernels that follow.  kParamsWalk / kParamsWalkAffine (short
+// sequences) take no partial ranges at all: every workgroup walks the whole sequence of its
+// (batch, head) for the channel ranges itself, which leaves the preparation without a launch
+// to wait for.
+constexpr int kParamsStored = 0, kParamsAbsmax = 1, kParamsAffine = 2, kParamsWalk = 3, kParamsWalkAffine = 4;
 constexpr int kCodeBlockPositions = 128;
 
 struct FusedParams {
@@ -248,7 +249,9 @@ __device__ __forceinline__ void value_codes_block(const void* __restrict__ v, in
   __shared__ __attribute__((aligned(16))) uint32_t transposed[DK * PITCH];
   __shared__ float channel_inverse[DK], channel_midpoint[DK];
   [[maybe_unused]] __shared__ float partial_max[256 / DK][DK], partial_min[256 / DK][DK];
-  [[maybe_unused]] __shared__ float walked_max[PARAMS == kParamsWalk ? SLOTS : 1][DK];
+  constexpr bool WALK = PARAMS == kParamsWalk || PARAMS == kParamsWalkAffine;
+  [[maybe_unused]] __shared__ float walked_max[WALK ? SLOTS : 1][DK];
+  [[maybe_unused]] __shared__ float walked_min[PARAMS == kParamsWalkAffine ? SLOTS : 1][DK];
   const int b = bh / heads, h = bh - b * heads;
   const int tid = threadIdx.x;
   const int octet = tid % OCTETS, slot = tid / OCTETS;
@@ -264,13 +267,17 @@ __device__ __forceinline__ void value_codes_block(const void* __restrict__ v, in
       inv[i] = inverse[row0 + octet * 8 + i];
       mid[i] = midpoint[row0 + octet * 8 + i];
     }
-  } else if constexpr (PARAMS == kParamsWalk) {
+  } else if constexpr (WALK) {
     // Thread (octet, slot) takes the rows slot, slot + SLOTS, ... of the whole sequence; rows
-    // past the end read the last one again (a repeated element does not change a maximum), so
-    // the loads sit in no branch.  The maximum does not depend on the order.
-    float mx[8];
+    // past the end read the last one again (a repeated element changes neither a maximum nor
+    // a minimum), so the loads sit in no branch.  Neither depends on the order.
+    constexpr bool AFFINE = PARAMS == kParamsWalkAffine;
+    float mx[8], mn[8];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) mx[i] = 0.0f;
+    for (int i = 0; i < 8; ++i) {
+      mx[i] = AFFINE ? -FLT_MAX : 0.0f;
+      mn[i] = FLT_MAX;
+    }
     const int passes = (length + SLOTS - 1) / SLOTS;
 #pragma unroll 8
     for (int pass = 0; pass < passes; ++pass) {
@@ -278,24 +285,39 @@ __device__ __forceinline__ void value_codes_block(const void* __restrict__ v, in
       float x[8];
       load8<DT>(v, base + static_cast<int64_t>(n) * stride_n + octet * 8, x);
 #pragma unroll
-      for (int i = 0; i < 8; ++i) mx[i] = __builtin_fmaxf(mx[i], __builtin_fabsf(x[i]));
+      for (int i = 0; i < 8; ++i) {
+        if constexpr (AFFINE) {
+          mx[i] = __builtin_fmaxf(mx[i], x[i]);
+          mn[i] = __builtin_fminf(mn[i], x[i]);
+        } else {
+          mx[i] = __builtin_fmaxf(mx[i], __builtin_fabsf(x[i]));
+        }
+      }
     }
 #pragma unroll
-    for (int i = 0; i < 8; ++i) walked_max[slot][octet * 8 + i] = mx[i];
+    for (int i = 0; i < 8; ++i) {
+      walked_max[slot][octet * 8 + i] = mx[i];
+      if constexpr (AFFINE) walked_min[slot][octet * 8 + i] = mn[i];
+    }
     __syncthreads();
     if (tid < DK) {
-      float top = walked_max[0][tid];
+      float top = walked_max[0][tid], bottom = AFFINE ? walked_min[0][tid] : FLT_MAX;
 #pragma unroll
-      for (int part = 1; part < SLOTS; ++part) top = __builtin_fmaxf(top, walked_max[part][tid]);
-      const float sc = __builtin_fmaxf(top * (1.0f / 127.0f), 1e-12f);
+      for (int part = 1; part < SLOTS; ++part) {
+        top = __builtin_fmaxf(top, walked_max[part][tid]);
+        if constexpr (AFFINE) bottom = __builtin_fminf(bottom, walked_min[part][tid]);
+      }
+      const float middle = AFFINE ? 0.5f * (bottom + top) : 0.0f;
+      const float radius = AFFINE ? 0.5f * (top - bottom) : top;
+      const float sc = __builtin_fmaxf(radius * (1.0f / 127.0f), 1e-12f);
       const float reciprocal = 1.0f / sc;
       channel_inverse[tid] = reciprocal;
-      channel_midpoint[tid] = 0.0f;
+      channel_midpoint[tid] = middle;
       if (position_block == 0) {
         fused.scale[row0 + tid] = sc;
         fused.inverse[row0 + tid] = reciprocal;
-        fused.midpoint[row0 + tid] = 0.0f;
-        fused.center[row0 + tid] = 0.0f;
+        fused.midpoint[row0 + tid] = middle;
+        if constexpr (!AFFINE) fused.center[row0 + tid] = 0.0f;
       }
     }
     __syncthreads();
@@ -547,7 +569,9 @@ __global__ __launch_bounds__(512) void value_center_from_partials_kernel(
 // holds the code blocks: the parameters come from the partial ranges (the same reduction
 // and arithmetic as value_codes_block, so the same bits), and thread t plays the summation
 // threads t and t + 256 one after the other.  Warp totals land in the reference's order.
-template <int DT>
+// WALK: the ranges of the block's eight channels come from a walk over the whole sequence
+// instead of the partial ranges of an earlier launch.
+template <int DT, bool WALK = false>
 __device__ __forceinline__ void value_center_block(const void* __restrict__ v, const FusedParams& fused,
                                                    int length, int dim, int heads, int64_t stride_b,
                                                    int64_t stride_h, int64_t stride_n,
@@ -566,7 +590,20 @@ __device__ __forceinline__ void value_center_block(const void* __restrict__ v, c
     mx[i] = -FLT_MAX;
     mn[i] = FLT_MAX;
   }
-  if (lane < fused.chunks) {
+  if constexpr (WALK) {
+    // rows t, t + 256, ...; past the end the last row again (no effect on a range)
+    const int passes = (length + 255) / 256;
+#pragma unroll 4
+    for (int pass = 0; pass < passes; ++pass) {
+      float x[8];
+      load8<DT>(v, base + static_cast<int64_t>(min(pass * 256 + t, length - 1)) * stride_n + octet * 8, x);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        mx[i] = __builtin_fmaxf(mx[i], x[i]);
+        mn[i] = __builtin_fminf(mn[i], x[i]);
+      }
+    }
+  } else if (lane < fused.chunks) {
     const int64_t slot = (static_cast<int64_t>(bh) * fused.chunks + lane) * dim + octet * 8;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
@@ -580,6 +617,28 @@ __device__ __forceinline__ void value_center_block(const void* __restrict__ v, c
     for (int i = 0; i < 8; ++i) {
       mx[i] = __builtin_fmaxf(mx[i], __shfl_xor(mx[i], offset));
       mn[i] = __builtin_fminf(mn[i], __shfl_xor(mn[i], offset));
+    }
+  }
+  if constexpr (WALK) {
+    // the four wavefronts hold different rows: combine them through LDS
+    __shared__ float wave_range[2][4][8];
+    if (lane < 8) {
+      float hi = mx[0], lo = mn[0];
+#pragma unroll
+      for (int i = 1; i < 8; ++i) {
+        hi = lane == i ? mx[i] : hi;
+        lo = lane == i ? mn[i] : lo;
+      }
+      wave_range[0][t >> 6][lane] = hi;
+      wave_range[1][t >> 6][lane] = lo;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      mx[i] = __builtin_fmaxf(__builtin_fmaxf(wave_range[0][0][i], wave_range[0][1][i]),
+                              __builtin_fmaxf(wave_range[0][2][i], wave_range[0][3][i]));
+      mn[i] = __builtin_fminf(__builtin_fminf(wave_range[1][0][i], wave_range[1][1][i]),
+                              __builtin_fminf(wave_range[1][2][i], wave_range[1][3][i]));
     }
   }
 #pragma unroll
