@@ -452,12 +452,33 @@ __device__ __forceinline__ int detect_anchor_value(const void* __restrict__ k, i
   const int tid = threadIdx.x, sub = tid & 31, seg = tid >> 5;
   const bool working = tid < 128;
   const int64_t base = static_cast<int64_t>(b) * stride_b + static_cast<int64_t>(h) * stride_h;
-  for (int index = working ? tid : kSamples * dim; index < kSamples * dim; index += 128) {
-    const int s = index / dim;
-    const int c = index - s * dim;
-    int64_t row = static_cast<int64_t>(s) * (length - 1) / (kSamples - 1);
-    if (permutation != nullptr) row = permutation[(static_cast<int64_t>(b) * heads + h) * length + row];
-    samples[index] = load1<DT>(k, base + row * stride_n + c);
+  // Thread t fetches channels t and t + 128 of the nine sampled rows; every load is issued
+  // before any is stored (the detector sits in front of the K quantisation of short problems,
+  // where a loop of load-then-store round trips would be the longest chain of the launch).
+  {
+    int64_t rows[kSamples];
+#pragma unroll
+    for (int s = 0; s < kSamples; ++s) rows[s] = static_cast<int64_t>(s) * (length - 1) / (kSamples - 1);
+    if (permutation != nullptr) {
+#pragma unroll
+      for (int s = 0; s < kSamples; ++s) rows[s] = permutation[(static_cast<int64_t>(b) * heads + h) * length + rows[s]];
+    }
+    float fetched[2][kSamples];
+#pragma unroll
+    for (int part = 0; part < 2; ++part) {
+      // a channel past the head dim reads channel 0 (never stored)
+      const int channel = tid + part * 128 < dim && working ? tid + part * 128 : 0;
+#pragma unroll
+      for (int s = 0; s < kSamples; ++s) fetched[part][s] = load1<DT>(k, base + rows[s] * stride_n + channel);
+    }
+#pragma unroll
+    for (int part = 0; part < 2; ++part) {
+      const int channel = tid + part * 128;
+      if (working && channel < dim) {
+#pragma unroll
+        for (int s = 0; s < kSamples; ++s) samples[s * dim + channel] = fetched[part][s];
+      }
+    }
   }
   __syncthreads();
 

@@ -278,19 +278,27 @@ __device__ __forceinline__ void value_codes_block(const void* __restrict__ v, in
       mx[i] = AFFINE ? -FLT_MAX : 0.0f;
       mn[i] = FLT_MAX;
     }
+    // sixteen rows in flight per thread: the walk is a chain of round trips, not of bytes
+    constexpr int IN_FLIGHT = 16;
     const int passes = (length + SLOTS - 1) / SLOTS;
-#pragma unroll 8
-    for (int pass = 0; pass < passes; ++pass) {
-      const int n = min(pass * SLOTS + slot, length - 1);
-      float x[8];
-      load8<DT>(v, base + static_cast<int64_t>(n) * stride_n + octet * 8, x);
+    for (int first_pass = 0; first_pass < passes; first_pass += IN_FLIGHT) {
+      float rows_in_flight[IN_FLIGHT][8];
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        if constexpr (AFFINE) {
-          mx[i] = __builtin_fmaxf(mx[i], x[i]);
-          mn[i] = __builtin_fminf(mn[i], x[i]);
-        } else {
-          mx[i] = __builtin_fmaxf(mx[i], __builtin_fabsf(x[i]));
+      for (int j = 0; j < IN_FLIGHT; ++j) {
+        const int n = min((first_pass + j) * SLOTS + slot, length - 1);
+        load8<DT>(v, base + static_cast<int64_t>(n) * stride_n + octet * 8, rows_in_flight[j]);
+      }
+#pragma unroll
+      for (int j = 0; j < IN_FLIGHT; ++j) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          const float x = rows_in_flight[j][i];
+          if constexpr (AFFINE) {
+            mx[i] = __builtin_fmaxf(mx[i], x);
+            mn[i] = __builtin_fminf(mn[i], x);
+          } else {
+            mx[i] = __builtin_fmaxf(mx[i], __builtin_fabsf(x));
+          }
         }
       }
     }
