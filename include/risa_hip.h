@@ -244,7 +244,13 @@ int risa_prepare_key_bias(const void* mask, float* bias, int batch, int heads, i
  * 4*ceil(q_len/128) blocks of 32 queries, t over ceil(k_len/64) key tiles) has bit l set
  * when query 32*w + l%32 may attend to key 64*t + 32*rb + 8*(i/4) + 4*(l/32) + i%4; no bit
  * is set past the last query or key.  The attention kernel applies one word per score
- * from scalar registers.  risa_mask_lanes_bytes returns the size of the buffer, or 0
+ * from scalar registers.  Behind the words of all planes the buffer holds one int32 class
+ * per (b, h, w, t) (1: every bit of the 32 words set, 2: none, 0: neither) and, per
+ * (b, h, block of 128 queries), the ascending list of the key tiles in which the block sees
+ * at least one key, int32 [tiles + 1] with the length in the last entry: the attention
+ * kernel (no causal flag, no sparse pattern, no capture) walks these lists, so tiles that
+ * a block-structured mask hides from a whole query block cost nothing (they would add
+ * zeros).  risa_mask_lanes_bytes returns the size of the whole buffer, or 0
  * when the form does not apply or does not pay: the mask is not boolean, the tiles are
  * not 64 keys, the head dim is 256 (that kernel holds its scores in another layout), the
  * key stride is not 1, the query stride is 0, the launch has at most 256 workgroups of 128

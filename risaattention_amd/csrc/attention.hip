@@ -116,6 +116,7 @@ int launch_attention(const AttentionArgs& a, hipStream_t stream) {
   p.mask_stride_k = a.mask_stride_k;
   p.mask_dtype = a.mask != nullptr ? a.mask_dtype : -1;
   int mask_mode = kMaskScalar;
+  int lane_planes_b = 0, lane_planes_h = 0;  // mask planes behind the lane words
   if (a.mask != nullptr) {
     // Groups of four keys start at multiples of four, so one load per group needs
     // unit key stride, the other strides multiples of four elements and the base
@@ -141,6 +142,8 @@ int launch_attention(const AttentionArgs& a, hipStream_t stream) {
       p.mask_lanes = a.mask_lanes;
       p.mask_lanes_stride_b = a.mask_lanes_stride_b;
       p.mask_lanes_stride_h = a.mask_lanes_stride_h;
+      lane_planes_b = a.mask_lanes_stride_b != 0 ? a.batch : 1;
+      lane_planes_h = a.mask_lanes_stride_h != 0 ? a.q_heads : 1;
     }
     if (a.key_bias != nullptr) {
       if (a.mask_stride_q != 0) return fail("risa_attention: a key bias row needs a key-only mask");
@@ -178,6 +181,17 @@ int launch_attention(const AttentionArgs& a, hipStream_t stream) {
   } else if (use_key_tiles) {
     p.index_mode = 2;
     p.tile_indices = a.key_mask_tiles;
+  } else if (mask_mode == kMaskLanes && !capture && !a.is_causal) {
+    // The buffer of the lane words also lists, per mask plane and query block, the tiles in
+    // which the block sees a key at all: block-structured masks (documents, windows) skip
+    // the rest the way a sparse pattern would; skipped tiles would have added zeros.
+    p.index_mode = 3;
+    p.tile_indices = reinterpret_cast<const int32_t*>(
+        reinterpret_cast<const unsigned char*>(a.mask_lanes) +
+        mask_tile_list_offset(lane_planes_b, lane_planes_h, a.q_len, a.k_len));
+    const int64_t per_plane = static_cast<int64_t>(p.n_qb) * (p.n_kb + 1);
+    p.tile_list_stride_h = lane_planes_h > 1 ? per_plane : 0;
+    p.tile_list_stride_b = lane_planes_b > 1 ? per_plane * lane_planes_h : 0;
   }
   const bool indexed = p.index_mode != 0;
   const bool fast = a.mask == nullptr && !a.is_causal && a.sm_scale > 0.0f;

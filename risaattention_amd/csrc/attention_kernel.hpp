@@ -75,8 +75,9 @@ struct KernelParams {
   float sm2;  // sm_scale * log2(e)
   int out_dtype;
   const int32_t* row_offsets;   // sparse CSR (index_mode 1)
-  const int32_t* tile_indices;  // sparse block indices (1) or key-mask tiles (2)
+  const int32_t* tile_indices;  // sparse block indices (1), key-mask tiles (2) or mask tile lists (3)
   int index_mode;
+  int64_t tile_list_stride_b, tile_list_stride_h;  // mode 3: elements between the lists of mask planes (0: shared)
   float* workspace;  // capture
   float* lse;
   int causal;
@@ -186,7 +187,10 @@ using AttentionTileShape = TileShape<D, CTA_K, staged_mask_bytes(MASK_DT, MASK_M
 // and not a run-time branch so that the tile loop holds one unrolled mask path and
 // stays inside the instruction cache.
 template <int D, int CTA_K, bool FAST, bool INDEXED, bool CAPTURE, int MASK_DT, int MASK_MODE>
-__global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void attention_kernel(const KernelParams p) {
+__global__ __launch_bounds__(256, (D == 256 ? 1 : D == 64 && MASK_MODE == kMaskLanes ? 4 : 2)) void attention_kernel(
+    const KernelParams p) {
+  // (lane words, head dim 64: 128 registers keep four workgroups per compute unit; the variant
+  // that walks tile lists would otherwise take 130 and lose one)
   static_assert(!FAST || MASK_DT < 0, "the raw-score path takes no mask");
   static_assert(MASK_MODE == kMaskScalar || (MASK_DT >= 0 && MASK_DT != kKeyBias), "vector loads need a mask tensor");
   static_assert(MASK_MODE != kMaskStaged || CTA_K == 64, "staged masks: 64-key tiles");
@@ -213,7 +217,9 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void attention_kernel(cons
   // number of key tiles: the launch then goes through all heads of the last query
   // block first and the first query block last (longest first keeps the tail short).
   int bx, head, batch;
-  if (!FAST && p.causal) {
+  if (!FAST && (p.causal || p.index_mode == 3)) {
+    // (tile lists of a mask: a lower-triangular mask given as a tensor is the common case of
+    // lists that grow with the query block)
     const int heads = p.q_heads * p.batch;
     const int rest = blockIdx.x % heads;
     bx = p.n_qb - 1 - blockIdx.x / heads;
@@ -266,6 +272,12 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void attention_kernel(cons
       const int start = p.row_offsets[row];
       n_it = p.row_offsets[row + 1] - start;
       indices = p.tile_indices + start;
+    } else if (p.index_mode == 3) {
+      // lists of a boolean mask several heads share: per mask plane and query block, the
+      // tiles in which the block sees at least one key
+      indices = p.tile_indices + batch * p.tile_list_stride_b + head * p.tile_list_stride_h +
+                static_cast<int64_t>(bx) * (p.n_kb + 1);
+      n_it = indices[p.n_kb];
     } else {
       indices = p.tile_indices + bhq * (p.n_kb + 1);
       n_it = indices[p.n_kb];
@@ -278,11 +290,15 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void attention_kernel(cons
     }
   }
   n_it = __builtin_amdgcn_readfirstlane(n_it);
+  // Lists are ascending without repeats: one that names every tile is 0, 1, 2, ... and is
+  // walked without being read (a mask that hides no whole tile costs no list reads).
+  [[maybe_unused]] const bool whole_list = INDEXED && n_it == p.n_kb;
   // Entry `it` of the tile list through the scalar cache (the address is uniform): the first
   // entries are needed before anything else can start, and as a vector load their wait would
   // include the Q rows requested above (vector memory returns in order).
   auto tile_at = [&](int it) -> int {
     if constexpr (INDEXED) {
+      if (whole_list) return it;
       typedef const __attribute__((address_space(4))) int32_t* UniformEntries;
       return ((UniformEntries)(reinterpret_cast<uintptr_t>(indices)))[it];
     }
@@ -970,7 +986,10 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : 2)) void attention_kernel(cons
       __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
       __syncthreads();
       [[maybe_unused]] int listed_after_next = 0;
-      if constexpr (INDEXED) listed_after_next = indices[min(it + 2, n_it - 1)];
+      if constexpr (INDEXED) {
+        listed_after_next = min(it + 2, n_it - 1);
+        if (!whole_list) listed_after_next = indices[listed_after_next];
+      }
       load_k_fragments(lds + stage * Shape::kStageBytes, 0, k_first);
       if constexpr (PRELOAD) {
         load_mask_words(tile);

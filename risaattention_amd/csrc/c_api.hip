@@ -367,7 +367,7 @@ size_t risa_mask_lanes_bytes(int mask_dtype, int head_dim, int cta_k, int64_t ma
   if (batch <= 0 || q_heads <= 0 || mask_batch <= 0 || mask_heads <= 0 || q_len <= 0 || k_len <= 0) return 0;
   // The conversion reads the mask once; it pays when several heads then share the words.
   if (static_cast<int64_t>(batch) * q_heads < int64_t{8} * mask_batch * mask_heads) return 0;
-  return risa::mask_lane_words(mask_batch, mask_heads, q_len, k_len) * sizeof(uint64_t);
+  return risa::mask_lane_bytes(mask_batch, mask_heads, q_len, k_len);
 }
 
 int risa_prepare_mask_lanes(const void* mask, uint64_t* lanes, int mask_batch, int mask_heads,

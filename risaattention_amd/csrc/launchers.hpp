@@ -110,7 +110,13 @@ int launch_prepare_fused(const QkArgs& qk, const ValueArgs& v, hipStream_t strea
 
 // Lane words of a boolean mask with 64-key tiles: [batch, heads, ceil(q_len/128)*4,
 // ceil(k_len/64), 32] 64-bit words, batch and heads being the mask's own extents.
+// What the 32 lane words of one (block of 32 queries, 64-key tile) have in common: every bit
+// set (the tile needs no select), none set (the wavefront skips the tile: it would add nothing
+// to the sums and leave the running maximum where it is), or neither.
+constexpr int kLaneTileMixed = 0, kLaneTileVisible = 1, kLaneTileHidden = 2;
 size_t mask_lane_words(int batch, int heads, int q_len, int k_len);
+size_t mask_lane_bytes(int batch, int heads, int q_len, int k_len);  // words, classes and tile lists
+size_t mask_tile_list_offset(int batch, int heads, int q_len, int k_len);  // of the lists, in bytes
 int launch_mask_lanes(const void* mask, uint64_t* lanes, int batch, int heads, int q_len, int k_len,
                       int64_t stride_b, int64_t stride_h, int64_t stride_q, hipStream_t stream);
 

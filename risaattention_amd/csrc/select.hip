@@ -238,7 +238,8 @@ __device__ __forceinline__ void write_lane(uint32_t& target, uint32_t uniform_va
 }
 template <bool ALIGNED>
 __global__ __launch_bounds__(256) void mask_lanes_kernel(const uint8_t* __restrict__ mask,
-                                                         uint64_t* __restrict__ lanes, int heads,
+                                                         uint64_t* __restrict__ lanes,
+                                                         int32_t* __restrict__ classes, int heads,
                                                          int q_len, int k_len, int key_tiles,
                                                          int query_waves, int64_t stride_b,
                                                          int64_t stride_h, int64_t stride_q) {
@@ -275,6 +276,7 @@ __global__ __launch_bounds__(256) void mask_lanes_kernel(const uint8_t* __restri
     if (first_tile + t >= key_tiles) break;  // wave-uniform
     // word s of the tile goes to lane s, 32 bits at a time, straight from the scalar registers
     uint32_t mine_low = 0, mine_high = 0;
+    uint64_t every = ~uint64_t{0}, any = 0;  // what all words of the tile / at least one of them hold
 #pragma unroll
     for (int rb = 0; rb < 2; ++rb) {
 #pragma unroll
@@ -283,6 +285,8 @@ __global__ __launch_bounds__(256) void mask_lanes_kernel(const uint8_t* __restri
         for (int r = 0; r < 4; ++r) {
           const uint64_t first = __ballot(((chunk[t][rb][group * 2] >> (8 * r)) & 0xffu) != 0);
           const uint64_t second = __ballot(((chunk[t][rb][group * 2 + 1] >> (8 * r)) & 0xffu) != 0);
+          every &= first & second;
+          any |= first | second;
           const int low_slot = rb * 16 + group * 4 + r;        // b4 = b'
           const int high_slot = rb * 16 + (2 + group) * 4 + r;  // b4 = 2 + b'
           write_lane(mine_low, static_cast<uint32_t>(first), low_slot);
@@ -294,15 +298,61 @@ __global__ __launch_bounds__(256) void mask_lanes_kernel(const uint8_t* __restri
     }
     const uint64_t mine = mine_low | (static_cast<uint64_t>(mine_high) << 32);
     if (lane < 32) out[static_cast<int64_t>(first_tile + t) * 32 + lane] = mine;
+    if (lane == 0) {
+      classes[(static_cast<int64_t>(plane) * query_waves + query_wave) * key_tiles + first_tile + t] =
+          every == ~uint64_t{0} ? kLaneTileVisible : any == 0 ? kLaneTileHidden : kLaneTileMixed;
+    }
   }
 }
 
 }  // namespace
 
+// Tile lists of the mask: grid (query blocks, planes), one wavefront.  A tile is listed for a
+// block of 128 queries unless all four of its 32-query classes say "no visible key"; entry
+// [tiles] of a list holds its length (the layout the attention kernel reads for key-mask
+// tiles).  A block that sees nothing keeps an empty list: its rows come out as zeros.
+__global__ __launch_bounds__(64) void mask_tile_lists_kernel(const int32_t* __restrict__ classes,
+                                                            int32_t* __restrict__ lists, int key_tiles,
+                                                            int query_blocks) {
+  const int lane = threadIdx.x;
+  const int block = blockIdx.x, plane = blockIdx.y;
+  const int32_t* wave_classes = classes + (static_cast<int64_t>(plane) * query_blocks + block) * 4 * key_tiles;
+  int32_t* list = lists + (static_cast<int64_t>(plane) * query_blocks + block) * (key_tiles + 1);
+  int count = 0;
+  for (int first = 0; first < key_tiles; first += 64) {
+    const int tile = first + lane;
+    bool listed = false;
+    if (tile < key_tiles) {
+#pragma unroll
+      for (int w = 0; w < 4; ++w) listed = listed || wave_classes[w * key_tiles + tile] != kLaneTileHidden;
+    }
+    const uint64_t ballot = __ballot(listed);
+    if (listed) list[count + __popcll(ballot & ((uint64_t{1} << lane) - 1))] = tile;
+    count += __popcll(ballot);
+  }
+  if (lane == 0) list[key_tiles] = count;
+}
+
 size_t mask_lane_words(int batch, int heads, int q_len, int k_len) {
   const size_t query_waves = (static_cast<size_t>(q_len) + 127) / 128 * 4;
   const size_t key_tiles = (static_cast<size_t>(k_len) + 63) / 64;
   return static_cast<size_t>(batch) * heads * query_waves * key_tiles * 32;
+}
+
+// The buffer of one mask: the lane words, then one 32-bit class per 32 words (kLaneTile...),
+// then per mask plane and block of 128 queries the list of tiles with a visible key.
+size_t mask_lane_class_offset(int batch, int heads, int q_len, int k_len) {
+  return mask_lane_words(batch, heads, q_len, k_len) * sizeof(uint64_t);
+}
+size_t mask_tile_list_offset(int batch, int heads, int q_len, int k_len) {
+  const size_t classes = mask_lane_words(batch, heads, q_len, k_len) / 32;
+  return mask_lane_class_offset(batch, heads, q_len, k_len) + (classes * sizeof(int32_t) + 7) / 8 * 8;
+}
+size_t mask_lane_bytes(int batch, int heads, int q_len, int k_len) {
+  const size_t query_blocks = (static_cast<size_t>(q_len) + 127) / 128;
+  const size_t key_tiles = (static_cast<size_t>(k_len) + 63) / 64;
+  const size_t lists = static_cast<size_t>(batch) * heads * query_blocks * (key_tiles + 1);
+  return mask_tile_list_offset(batch, heads, q_len, k_len) + (lists * sizeof(int32_t) + 7) / 8 * 8;
 }
 
 int launch_mask_lanes(const void* mask, uint64_t* lanes, int batch, int heads, int q_len, int k_len,
@@ -314,8 +364,13 @@ int launch_mask_lanes(const void* mask, uint64_t* lanes, int batch, int heads, i
   const dim3 grid((key_tiles + 4 * kLaneTilesPerWave - 1) / (4 * kLaneTilesPerWave), query_waves, batch * heads);
   const bool aligned = reinterpret_cast<uintptr_t>(mask) % 16 == 0 && ((stride_b | stride_h | stride_q) & 15) == 0;
   auto kernel = aligned ? mask_lanes_kernel<true> : mask_lanes_kernel<false>;
-  kernel<<<grid, 256, 0, stream>>>(static_cast<const uint8_t*>(mask), lanes, heads, q_len, k_len,
+  unsigned char* bytes = reinterpret_cast<unsigned char*>(lanes);
+  int32_t* classes = reinterpret_cast<int32_t*>(bytes + mask_lane_class_offset(batch, heads, q_len, k_len));
+  int32_t* lists = reinterpret_cast<int32_t*>(bytes + mask_tile_list_offset(batch, heads, q_len, k_len));
+  kernel<<<grid, 256, 0, stream>>>(static_cast<const uint8_t*>(mask), lanes, classes, heads, q_len, k_len,
                                    key_tiles, query_waves, stride_b, stride_h, stride_q);
+  mask_tile_lists_kernel<<<dim3(query_waves / 4, batch * heads), 64, 0, stream>>>(classes, lists, key_tiles,
+                                                                              query_waves / 4);
   return check_launch("risa_prepare_mask_lanes");
 }
 

@@ -55,6 +55,7 @@ def prepare_mask_lanes(mask, key_block_size, head_dim):
                                      mask.stride(3), batch, q_heads, planes_b, planes_h, q_len, k_len)
     if size == 0:
         return None
+    # the lane words of every plane, then one class per tile (the library carves both)
     words = torch.empty(size // 8, device=mask.device, dtype=torch.int64)
     native.check(
         lib.risa_prepare_mask_lanes(
@@ -62,7 +63,7 @@ def prepare_mask_lanes(mask, key_block_size, head_dim):
             mask.stride(0), mask.stride(1), mask.stride(2), native.current_stream(mask.device),
         )
     )
-    plane = words.numel() // (planes_b * planes_h)
+    plane = 4 * -(-q_len // 128) * -(-k_len // 64) * 32  # words of one (batch, head) plane
     return words, (plane * planes_h if planes_b > 1 else 0), (plane if planes_h > 1 else 0)
 
 

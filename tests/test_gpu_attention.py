@@ -444,7 +444,13 @@ def test_lane_words_of_a_boolean_mask(risa, q_len, k_len, aligned):
     words, stride_b, stride_h = prepare_mask_lanes(mask.expand(2, heads, q_len, k_len), 64, 128)
     expected = expected_lane_words(planes[:, 0].numpy(), q_len, k_len)
     assert stride_h == 0 and stride_b == expected[0].size
-    assert np.array_equal(words.cpu().numpy().view(np.uint64).reshape(expected.shape), expected)
+    buffer = words.cpu().numpy().view(np.uint64)
+    assert np.array_equal(buffer[: expected.size].reshape(expected.shape), expected)
+    # behind the words: per (plane, block of 32 queries, tile) 1 = every bit set, 2 = none, 0 = neither
+    classes = buffer[expected.size:].view(np.int32)[: expected.size // 32].reshape(expected.shape[:3])
+    every = (expected == np.uint64(0xFFFFFFFFFFFFFFFF)).all(-1)
+    none = (expected == 0).all(-1)
+    assert np.array_equal(classes, np.where(every, 1, np.where(none, 2, 0)))
     # not for small launches, a plane per head, other tile sizes, head dim 256 or other dtypes
     assert prepare_mask_lanes(mask.expand(2, 8, q_len, k_len), 64, 128) is None
     assert prepare_mask_lanes(mask.expand(2, heads, q_len, k_len).contiguous(), 64, 128) is None
@@ -559,3 +565,38 @@ def test_output_rows_in_both_layouts_and_misaligned_outputs(risa, dim, heads, q_
     assert torch.equal(buffer[count:], torch.full_like(buffer[count:], 7.0))
     with pytest.raises(RuntimeError, match="16-byte aligned"):
         launch_attention(output=buffer[4 : count + 4].view(shape), **arguments)
+
+
+@pytest.mark.parametrize("dim", [64, 128])
+@pytest.mark.parametrize("pattern", ["block_diagonal", "lower_triangle", "all_true"])
+def test_structured_shared_masks_skip_and_pass_whole_tiles(risa, dim, pattern):
+    """A boolean mask that many heads share is classified per (32 queries, 64 keys): tiles
+    without a visible key are skipped and tiles without a hidden key take no select.  Both
+    must be invisible in the results: equal to the same mask given per head (which reads
+    the mask elements) bit for bit, and to the oracle on a slice."""
+    q_len, k_len, heads = 640, 700, 72
+    q = seeded((1, heads, q_len, dim), torch.bfloat16, 91)
+    k = seeded((1, 1, k_len, dim), torch.bfloat16, 92)
+    v = seeded((1, 1, k_len, dim), torch.bfloat16, 93, offset=0.5)
+    rows = torch.arange(q_len)[:, None]
+    keys = torch.arange(k_len)[None, :]
+    if pattern == "block_diagonal":
+        shared = (rows // 200) == (keys // 220)          # documents of unequal lengths
+    elif pattern == "lower_triangle":
+        shared = keys <= rows + 37
+    else:
+        shared = torch.ones(q_len, k_len, dtype=torch.bool)
+        shared[3] = False                                 # one row without any key
+    shared = shared.cuda()[None, None]
+    per_head = shared.expand(1, heads, q_len, k_len).contiguous()
+    from risaattention_amd.key_mask import prepare_mask_lanes
+    assert prepare_mask_lanes(shared.expand(1, heads, q_len, k_len), 64, dim) is not None
+    out, lse = risa.int8_attention(q, k, v, attn_mask=shared, return_lse=True)
+    out_heads, lse_heads = risa.int8_attention(q, k, v, attn_mask=per_head, return_lse=True)
+    assert torch.equal(out, out_heads)
+    assert torch.equal(lse, lse_heads)
+    checked = 2
+    prepared = oracle_prequantize(q[:, :checked], k, v, attn_mask=shared, return_lse=True)
+    expected, expected_lse, _ = oracle_pipeline.attend(prepared, return_lse=True)
+    assert relative_l2(to_numpy(out[:, :checked]), expected) < TOLERANCE
+    assert relative_l2(to_numpy(lse[:, :checked]), expected_lse) < TOLERANCE

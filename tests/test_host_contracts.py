@@ -37,9 +37,17 @@ def test_lane_word_size_query_rules():
         return lib.risa_mask_lanes_bytes(dtype, head_dim, cta_k, stride_q, stride_k, batch, heads,
                                          mask_batch, mask_heads, q_len, k_len)
 
-    # [mask batch, mask heads, blocks of 32 queries padded to 128, 64-key tiles, 32 words] x 8 bytes
-    assert size() == 2 * 1 * (4096 // 32) * (4608 // 64) * 32 * 8
-    assert size(q_len=4000, k_len=4600) == 2 * (32 * 4) * 72 * 32 * 8  # ragged extents round up
+    # [mask batch, mask heads, blocks of 32 queries padded to 128, 64-key tiles, 32 words] x 8 bytes,
+    # then one 32-bit class per (block of 32 queries, tile), then per plane and block of 128
+    # queries a tile list (tiles + 1 entries of 32 bits); every section a whole number of 8 bytes
+    def expected(planes, q_len, k_len):
+        waves, tiles = -(-q_len // 128) * 4, -(-k_len // 64)
+        round8 = lambda n: -(-n // 8) * 8
+        return planes * waves * tiles * 32 * 8 + round8(planes * waves * tiles * 4) + round8(planes * (waves // 4) * (tiles + 1) * 4)
+
+    assert size() == expected(2, 4096, 4608)
+    assert size(q_len=4000, k_len=4600) == expected(2, 4000, 4600)  # ragged extents round up
+    assert size(batch=1, heads=24, mask_batch=1, q_len=1500, k_len=100) == expected(1, 1500, 100)
     assert size(head_dim=64) == size()
     assert size(dtype=F32) == 0            # values, not decisions
     assert size(cta_k=128) == 0            # query-dependent masks run 64-key tiles
