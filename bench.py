@@ -252,8 +252,15 @@ def masked_variants(torch, batch, q_len, k_len, device):
     bias = torch.randn(batch, 1, q_len, k_len, generator=generator, device=device)  # float32
     rowmask = torch.ones(batch, 1, q_len, k_len, dtype=torch.bool, device=device)
     rowmask[0, :, :7] = False  # fully masked rows
+    # two block-structured boolean masks beside the reference's five variants: eight packed
+    # documents (block diagonal) and a causal window of 1024 keys
+    rows = torch.arange(q_len, device=device)[:, None]
+    keys = torch.arange(k_len, device=device)[None, :]
+    documents = ((rows * 8 // q_len) == (keys * 8 // k_len))[None, None].expand(batch, 1, q_len, k_len).contiguous()
+    window = ((keys <= rows) & (keys > rows - 1024))[None, None].expand(batch, 1, q_len, k_len).contiguous()
     return {"plain": dict(), "causal": dict(is_causal=True), "key_padding": dict(attn_mask=key_padding),
-            "additive_bias": dict(attn_mask=bias), "bool_mask_lse": dict(attn_mask=rowmask, return_lse=True)}
+            "additive_bias": dict(attn_mask=bias), "bool_mask_lse": dict(attn_mask=rowmask, return_lse=True),
+            "document_mask": dict(attn_mask=documents), "window_mask": dict(attn_mask=window)}
 
 
 def workload_masked(torch, risa, args, device, dims=(64, 128), seeds=None, samples=None):
