@@ -147,7 +147,7 @@ extern "C" {
 
 const char* risa_last_error(void) { return risa::last_error_storage().c_str(); }
 
-int risa_abi_version(void) { return 2; }
+int risa_abi_version(void) { return 3; }
 
 int risa_quantize_qk(const void* q, void* q_int8, float* q_scale, const void* k, void* k_int8,
                      float* k_scale, int batch, int q_heads, int q_len, int kv_heads, int k_len,

@@ -22,7 +22,7 @@ def test_library_exports_every_declared_symbol():
     library = ctypes.CDLL(str(native.library_path()))
     for name in declared:
         assert hasattr(library, name), name
-    assert native.library().risa_abi_version() == 2
+    assert native.library().risa_abi_version() == 3
     assert native.library().risa_last_error() == b""
 
 
