@@ -142,7 +142,11 @@ void risa_unpack_order(int32_t* order);
  *   dim contiguous; base 16-byte aligned, strides multiples of 8 elements: rows
  *   are written 16 bytes per lane); mask (nullable) expanded to [B,Hq,Lq,Lk] with its strides,
  *   query stride 0 selecting the key-only path; sparse_row_offsets int32
- *   [B*Hq*ceil(Lq/128)+1] and sparse_block_indices int32 (both or neither);
+ *   [B*Hq*ceil(Lq/128)+1] and sparse_block_indices int32 (both or neither; the tile
+ *   ids of every row ascending, without repeats and below the number of key tiles, as
+ *   risa_select_retained_mass writes them: a row that lists every tile is walked as
+ *   0, 1, 2, ... without being read, and only the last listed tile is treated as the
+ *   one that may be partial);
  *   block_mass (nullable) float32 workspace laid out as mass
  *   [B*Hq*ceil(Lq/128), tiles] ++ full-tile stats [B*Hq, tiles-1, Lq, 2]
  *   (u32 sum of U8 probabilities, f32 tile maximum; tile-major so that the
@@ -151,14 +155,19 @@ void risa_unpack_order(int32_t* order);
  *   total size as reference attention_int8.cuh:51-143, 871-898, whose full-tile
  *   stats are row-major); lse (nullable) float32
  *   [B,Hq,Lq]; key_mask_tiles (nullable) int32 [B,Hq,tiles+1] from
- *   risa_prepare_key_mask_tiles; key_bias (nullable) float32 [Bm,Hm,padded keys]
+ *   risa_prepare_key_mask_tiles (ascending ids, count in the last entry; same
+ *   ordering contract as the sparse lists); key_bias (nullable) float32 [Bm,Hm,padded keys]
  *   from risa_prepare_key_bias with its batch and head strides in elements (0
  *   for a broadcast extent): given together with a key-only mask (mask_stride_q
  *   0), the kernel stages this row per key tile instead of reading mask elements;
  *   mask_lanes (nullable) the lane words of a query-dependent boolean mask from
  *   risa_prepare_mask_lanes with their batch and head strides in 64-bit words (0
- *   for a broadcast extent): given together with that mask and 64-key tiles, the
- *   kernel applies the words instead of reading mask elements.
+ *   for a broadcast extent): given together with that mask (unit key stride) and 64-key
+ *   tiles, the kernel applies the words instead of reading mask elements.  The two strides
+ *   also fix the layout of the buffer: a non-zero stride means the buffer was made for
+ *   `batch` (resp. `q_heads`) planes, zero for one, and the classes and tile lists are
+ *   looked up behind the words of that many planes, for this q_len and k_len; pass the
+ *   buffer exactly as risa_prepare_mask_lanes filled it.
  */
 int risa_attention(const void* q_int8, const void* k_int8, const void* v_int8, void* out,
                    const float* q_scale, const float* k_scale, const float* v_scale,
@@ -253,8 +262,8 @@ int risa_prepare_key_bias(const void* mask, float* bias, int batch, int heads, i
  * zeros).  risa_mask_lanes_bytes returns the size of the whole buffer, or 0
  * when the form does not apply or does not pay: the mask is not boolean, the tiles are
  * not 64 keys, the head dim is 256 (that kernel holds its scores in another layout), the
- * key stride is not 1, the query stride is 0, the launch has at most 256 workgroups of 128
- * queries (it runs the sixteen-query kernel), or fewer than eight
+ * key stride is not 1, the query stride is 0, the launch has no more workgroups of 128
+ * queries than the device has compute units (it runs the sixteen-query kernel), or fewer than eight
  * (batch, head) pairs share each mask plane (the conversion reads the mask once, the
  * attention kernel would read it once per pair).  No counterpart in the reference, whose
  * kernel reads the mask per score (csrc/kernels/attention_masks.cuh:27-164); the

@@ -15,7 +15,6 @@ template <> int launch_attention_variant<128>(const KernelParams&, int, bool, bo
 int launch_attention_narrow(const KernelParams& p, int head_dim, int cta_k, hipStream_t stream);
 int launch_attention_narrow_general(const KernelParams& p, int head_dim, int cta_k, bool fast, bool indexed,
                                     bool capture, int mask_mode, hipStream_t stream);
-int narrow_attention_limit();
 
 namespace {
 
@@ -134,8 +133,17 @@ int launch_attention(const AttentionArgs& a, hipStream_t stream) {
       }
     }
     if (a.mask_lanes != nullptr && a.head_dim <= 128) {  // the sixteen-query kernel of head dim 256 reads the mask itself
-      if (a.mask_dtype != kBool || a.cta_k != 64 || a.mask_stride_q == 0)
-        return fail("risa_attention: lane words go with a query-dependent boolean mask and 64-key tiles");
+      if (a.mask_dtype != kBool || a.cta_k != 64 || a.mask_stride_q == 0 || a.mask_stride_k != 1)
+        return fail("risa_attention: lane words go with a query-dependent boolean mask of unit key stride and 64-key tiles");
+      // The strides say how many planes the buffer was made for: they are either zero or the
+      // words of one plane (times the head planes for the batch stride).
+      {
+        const int64_t plane = static_cast<int64_t>(mask_lane_words(1, 1, a.q_len, a.k_len));
+        const int64_t heads = a.mask_lanes_stride_h != 0 ? a.q_heads : 1;
+        if ((a.mask_lanes_stride_h != 0 && a.mask_lanes_stride_h != plane) ||
+            (a.mask_lanes_stride_b != 0 && a.mask_lanes_stride_b != plane * heads))
+          return fail("risa_attention: lane word strides must be 0 or the plane sizes risa_prepare_mask_lanes uses");
+      }
       if (reinterpret_cast<uintptr_t>(a.mask_lanes) % 8 != 0)
         return fail("risa_attention: lane words must be 8-byte aligned");
       mask_mode = kMaskLanes;

@@ -4,7 +4,6 @@
 
 namespace risa {
 
-int narrow_attention_limit();
 
 namespace {
 
@@ -42,15 +41,18 @@ template <int D, int CTA_K> int launch_narrow(const KernelParams& p, hipStream_t
 }  // namespace
 
 // Number of workgroups up to which the narrow kernel is the faster one: the number of
-// compute units, below which the wide kernel runs one wavefront per SIMD.
+// compute units, below which the wide kernel runs one wavefront per SIMD.  Where no device can
+// be queried (size queries made on a host without a GPU) it is the MI355X's 256.
 int narrow_attention_limit() {
+  constexpr int kMi355xComputeUnits = 256;
   static thread_local int cached_device = -1;
   static thread_local int compute_units = 0;
   int device = -1;
-  if (hipGetDevice(&device) != hipSuccess) return 0;
+  if (hipGetDevice(&device) != hipSuccess) return kMi355xComputeUnits;
   if (device != cached_device) {
     int count = 0;
-    if (hipDeviceGetAttribute(&count, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess) return 0;
+    if (hipDeviceGetAttribute(&count, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || count <= 0)
+      return kMi355xComputeUnits;
     compute_units = count;
     cached_device = device;
   }

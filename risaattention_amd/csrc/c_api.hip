@@ -19,13 +19,20 @@ namespace {
 
 constexpr int kMaxDevices = 64;
 
-// Device address of risa_static_scratch on the current device, resolved once per device.
-int static_scratch_address(void** address) {
+// Device address of risa_static_scratch on the device the stream belongs to (the current device
+// for the null stream), resolved once per device with that device current.
+int static_scratch_address(hipStream_t stream, void** address) {
   static std::mutex guard;
   static void* resolved[kMaxDevices] = {};
-  int device = -1;
-  if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= kMaxDevices)
+  int current = -1;
+  if (hipGetDevice(&current) != hipSuccess || current < 0 || current >= kMaxDevices)
     return risa::fail("risa_quantize_v_noalloc: cannot identify the current device");
+  int device = current;
+  if (stream != nullptr && hipStreamGetDevice(stream, &device) != hipSuccess)
+    return risa::fail("risa_quantize_v_noalloc: cannot identify the device of the stream");
+  if (device != current)
+    return risa::fail("risa_quantize_v_noalloc: the stream belongs to device " + std::to_string(device) +
+                      " but device " + std::to_string(current) + " is current");
   std::lock_guard<std::mutex> lock(guard);
   if (resolved[device] == nullptr) {
     void* pointer = nullptr;
@@ -196,7 +203,7 @@ int risa_quantize_v_noalloc(const void* v, void* out, float* scale, float* cente
                       std::to_string(static_cast<size_t>(RISA_STATIC_SCRATCH_BYTES)) +
                       "; use risa_quantize_v with a caller-provided workspace");
   void* scratch = nullptr;
-  int status = static_scratch_address(&scratch);
+  int status = static_scratch_address(static_cast<hipStream_t>(stream), &scratch);
   if (status != 0) return status;
   risa::ValueArgs a{};
   status = checked_v_args(a, v, out, scale, center, tile_sum, scratch, RISA_STATIC_SCRATCH_BYTES, batch,
@@ -265,8 +272,7 @@ int risa_attention(const void* q_int8, const void* k_int8, const void* v_int8, v
     return fail("risa_attention: attention mask must be bool, float16, bfloat16, or float32");
   if (batch <= 0 || q_heads <= 0 || kv_heads <= 0 || q_len <= 0 || k_len <= 0)
     return fail("risa_attention: extents must be positive");
-  if (out_stride_n % 4 != 0 || out_stride_h % 4 != 0 || out_stride_b % 4 != 0 || !aligned(out, 8))
-    return fail("risa_attention: output rows must be 8-byte aligned");
+  // (the output's alignment rule is checked once, by the launcher)
   risa::AttentionArgs a{};
   a.q = static_cast<const int8_t*>(q_int8);
   a.k = static_cast<const int8_t*>(k_int8);
@@ -358,9 +364,10 @@ size_t risa_mask_lanes_bytes(int mask_dtype, int head_dim, int cta_k, int64_t ma
                              int mask_heads, int q_len, int k_len) {
   if (mask_dtype != risa::kBool || cta_k != 64 || mask_stride_q == 0 || mask_stride_k != 1) return 0;
   if (head_dim > 128) return 0;  // the sixteen-query kernel of head dim 256 has another score layout
-  // A launch of at most one workgroup per compute unit (256 on the MI355X) runs the
-  // sixteen-query kernel, and the conversion would be a launch of its own next to a short kernel.
-  if (static_cast<int64_t>(batch) * q_heads * ((q_len + 127) / 128) <= 256) return 0;
+  // A launch of at most one workgroup per compute unit runs the sixteen-query kernel (the same
+  // limit the launcher applies), and the conversion would be a launch of its own next to a
+  // short kernel.
+  if (static_cast<int64_t>(batch) * q_heads * ((q_len + 127) / 128) <= risa::narrow_attention_limit()) return 0;
   // one conversion launch: blocks of 32 queries and mask planes are grid dimensions
   if ((static_cast<int64_t>(q_len) + 127) / 128 * 4 > 65535 || static_cast<int64_t>(mask_batch) * mask_heads > 65535)
     return 0;

@@ -134,7 +134,10 @@ __device__ __forceinline__ float load1(const void* base, int64_t offset) {
 // even code), and the low byte of its bit pattern is the two's-complement INT8 code.  One add
 // replaces round, NaN test, clamp and convert; the scales of this library keep |value| below
 // 127.5 for finite inputs (scale > max / 127), so the reference's clamp never binds, and a NaN
-// (0 * inf from a non-finite row) has a zero low byte like the reference's saturating convert.
+// (0 * inf from a row with an infinity) has a zero low byte like the reference's saturating
+// convert.  Not covered: a NaN in the *input* whose payload has a non-zero low byte travels
+// through the additions and leaves that byte as the code where the reference stores 0; the
+// scale of such a group is NaN-derived in both and the row's output meaningless either way.
 constexpr float kRoundMagic = 12582912.0f;
 __device__ __forceinline__ float round_to_code(float value) { return value + kRoundMagic; }
 __device__ __forceinline__ float code_value(float magic_sum) { return magic_sum - kRoundMagic; }

@@ -85,6 +85,9 @@ struct AttentionArgs {
   int64_t mask_lanes_stride_b, mask_lanes_stride_h;  // in words
 };
 int launch_attention(const AttentionArgs& args, hipStream_t stream);
+// Number of 128-query workgroups up to which a launch takes the sixteen-query kernel: the
+// compute units of the current device (the MI355X's 256 when no device can be queried).
+int narrow_attention_limit();
 
 struct SelectArgs {
   const float* sorted_mass;

@@ -5,8 +5,9 @@
   causal, boolean key padding, FP32 additive bias, boolean mask with fully masked rows + LSE.
   Bounds against FP32 SDPA are the reference's own (tests/cuda/test_risa_attention.py:94-149:
   atol 0.10, rtol 0.03; LSE atol 0.15), key-padding tile skipping against the same mask made
-  query dependent follows tests/cuda/test_key_mask_tiles.py:16-54, and a slice of every
-  variant is compared with the oracle to the 1e-3 relative-L2 bar.
+  query dependent follows tests/cuda/test_key_mask_tiles.py:16-54, and the whole query range
+  of the first and the last head of every variant (first, middle and last query block each
+  on its own, then all rows) is compared with the oracle to the 1e-3 relative-L2 bar.
 * Video-DiT scale: H=40, N=32760 (last query block and last key tile hold 120 rows):
   closed forms, the last block against FP32, construction + reuse, packed replay.
 * Sparse reuse on block-structured Q/K: B=1, Hq=16, Hkv=4, D=128, N=32768, 64 contiguous
@@ -124,21 +125,22 @@ def test_masked_outlier_configuration_full_size(risa, dim):
         # the call without the LSE is the same kernel launch
         assert torch.equal(risa.int8_attention(q, k, v, **kwargs), out), name
 
-        # ---- a slice against the oracle: one batch entry, two heads ----------------------
-        # causal: the first query block (positions are absolute); key padding: two query
-        # blocks of batch 1, so that the oracle also walks the list of active key tiles;
-        # otherwise one query block of batch 0 (the one with the fully masked rows).
-        entry = 1 if name == "key_padding" else 0
-        rows = slice(0, 256) if name == "key_padding" else slice(0, 128)
-        head_pair = slice(4, 6)
-        mask_slice = None
-        if mask is not None:
-            mask_slice = mask[entry:entry + 1, :, rows] if mask.shape[2] != 1 else mask[entry:entry + 1]
-        q_s, k_s, v_s = q[entry:entry + 1, head_pair, rows], k[entry:entry + 1, head_pair], v[entry:entry + 1, head_pair]
-        prepared = oracle_prequantize(q_s, k_s, v_s, attn_mask=mask_slice, is_causal=causal, return_lse=True)
-        expected, expected_lse, _ = oracle_pipeline.attend(prepared, return_lse=True)
-        assert relative_l2(to_numpy(out[entry:entry + 1, head_pair, rows]), expected) < TOLERANCE, name
-        assert relative_l2(to_numpy(lse[entry:entry + 1, head_pair, rows]), expected_lse) < TOLERANCE, name
+        # ---- against the oracle: every query block of the first and the last head -----------
+        # (all 32 query blocks, so the first, the middle and the last one; causal positions are
+        # absolute, which is why the whole query range goes to the oracle).  Key padding takes
+        # both heads from batch 1, whose tail is hidden, so that the oracle also walks the list
+        # of active key tiles; the other variants take one head from each batch entry (entry 0
+        # holds the fully masked rows of the boolean mask).
+        for head, entry in ((0, 1 if name == "key_padding" else 0), (heads - 1, 1)):
+            one = (slice(entry, entry + 1), slice(head, head + 1))
+            mask_slice = None if mask is None else mask[entry:entry + 1]
+            prepared = oracle_prequantize(q[one], k[one], v[one], attn_mask=mask_slice, is_causal=causal,
+                                          return_lse=True)
+            expected, expected_lse, _ = oracle_pipeline.attend(prepared, return_lse=True)
+            for block in (slice(0, 128), slice(q_len // 2, q_len // 2 + 128), slice(q_len - 128, q_len), slice(None)):
+                where = (name, head, entry, block)
+                assert relative_l2(to_numpy(out[one][:, :, block]), expected[:, :, block]) < TOLERANCE, where
+                assert relative_l2(to_numpy(lse[one][:, :, block]), expected_lse[:, :, block]) < TOLERANCE, where
 
     # Key padding hides whole key tiles of batch 1: skipping them through the tile list
     # equals walking every tile with the same mask made query dependent.

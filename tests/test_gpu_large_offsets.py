@@ -11,24 +11,37 @@ from risaattention_amd.attend import launch_attention
 
 pytestmark = pytest.mark.gpu
 
-REQUIRED_BYTES = 18 * 1024**3
+HEADS, DIM = 5, 64
+# 2^24 + 128 queries of 64 one-byte channels are 1 GiB + 8 KiB per head: from the fifth head on,
+# byte offsets of the codes need 33 bits, those of the fp16 output and of the capture rows more.
+QUERIES = 2**24 + 128
+MEMORY_NEEDED = 18 << 30
 
 
 @pytest.fixture(scope="module")
 def wide_buffers(risa):
-    if torch.cuda.mem_get_info()[0] < REQUIRED_BYTES:
+    """Prepared operands built by hand: all-zero Q and K codes (every score is 0), unit Q/K
+    scales, and a packed V matrix of one 64-key tile whose only non-zero column is token 0
+    (byte 0 of its 32-token group) with code 100 and scale 0.2, so a row that sees just that
+    key is exactly 20."""
+    free_bytes, _ = torch.cuda.mem_get_info()
+    if free_bytes < MEMORY_NEEDED:
         pytest.skip("large-offset checks need 18 GiB of free device memory")
-    length = (1 << 30) // 64 + 128
-    heads, dim = 5, 64
-    q = torch.zeros((1, heads, length, dim), dtype=torch.int8, device="cuda")
-    k = torch.zeros((1, 1, 1, dim), dtype=torch.int8, device="cuda")
-    v = torch.zeros((dim, 64), dtype=torch.int8, device="cuda")
-    v[:, 0] = 100  # token 0 sits at position 0 of its packed group
-    q_scale = torch.ones((1, heads, math.ceil(length / 128) * 32), device="cuda")
-    k_scale = torch.ones((1, 1, 4), device="cuda")
-    v_scale = torch.full((dim,), 0.2, device="cuda")
-    assert (heads - 1) * q.stride(1) > (1 << 32) - 1
-    yield q, k, v, q_scale, k_scale, v_scale, torch.zeros_like(v_scale)
+    device = torch.device("cuda")
+    operands = {
+        "q": torch.zeros(1, HEADS, QUERIES, DIM, dtype=torch.int8, device=device),
+        "k": torch.zeros(1, 1, 1, DIM, dtype=torch.int8, device=device),
+        "v": torch.zeros(DIM, 64, dtype=torch.int8, device=device),
+        "q_scale": torch.ones(1, HEADS, -(-QUERIES // 128) * 32, device=device),
+        "k_scale": torch.ones(1, 1, 4, device=device),
+        "v_scale": torch.full((DIM,), 0.2, device=device),
+        "v_center": torch.zeros(DIM, device=device),
+    }
+    operands["v"][:, 0] = 100
+    last_head_offset = (HEADS - 1) * operands["q"].stride(1)
+    assert last_head_offset >= 2**32
+    yield tuple(operands[name] for name in ("q", "k", "v", "q_scale", "k_scale", "v_scale", "v_center"))
+    operands.clear()
     torch.cuda.empty_cache()
 
 

@@ -275,3 +275,32 @@ def test_separate_entry_points_match_one_call_preparation(risa, dtype, dim, leng
                          (q_scale, packed.q_scale), (k_scale, packed.k_scale), (v_scale, packed.v_scale),
                          (v_center, packed.v_center), (tile_sum, packed.v_tile_sum)):
         assert torch.equal(ours, theirs)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("mode", ["absmax", "midpoint_affine"])
+def test_infinite_inputs_bit_for_bit(risa, dtype, mode):
+    """One infinite element in Q, K and V.  Its scale group's maximum is infinite, the
+    reciprocal of the scale zero, every product 0 or NaN (inf * 0), and the saturating
+    conversion of the reference turns NaN into code 0 (float_utils.cuh:23-31): the whole group
+    gets zero codes and an infinite scale, everything else is untouched.  The add-a-constant
+    conversion used here reads the low byte of the NaN that 0 * inf produces, which is zero."""
+    from risaattention_amd.layout import unpack_values
+
+    q = seeded((1, 2, 70, 128), dtype, 21)
+    k = seeded((1, 1, 300, 128), dtype, 22)
+    v = seeded((1, 1, 300, 128), dtype, 23)
+    q[0, 0, 5, 7] = float("inf")
+    k[0, 0, 130, 9] = float("-inf")
+    v[0, 0, 17, 3] = float("inf")
+    packed = risa.prequantize_int8_attention(q, k, v, v_quantization=mode)
+    with np.errstate(all="ignore"):
+        expected = oracle_prequantize(q, k, v, v_quantization=mode)
+    assert np.isinf(expected.q_scale).sum() == 1 and np.isinf(expected.k_scale).sum() == 1
+    np.testing.assert_array_equal(packed.q.cpu().numpy(), expected.q)
+    np.testing.assert_array_equal(packed.q_scale.cpu().numpy(), expected.q_scale)
+    np.testing.assert_array_equal(packed.k.cpu().numpy(), expected.k)
+    np.testing.assert_array_equal(packed.k_scale.cpu().numpy(), expected.k_scale)
+    np.testing.assert_array_equal(unpack_values(packed.v).cpu().numpy(), expected.v)
+    np.testing.assert_array_equal(packed.v_scale.cpu().numpy(), expected.v_scale)
+    np.testing.assert_array_equal(packed.v_center.cpu().numpy(), expected.v_center)  # NaN == NaN here

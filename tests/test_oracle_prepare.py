@@ -140,6 +140,49 @@ def test_anchor_decision_matches_float64_criterion():
                 assert anchor[b, h] == (rows[best] if accept else -1)
 
 
+def test_anchor_is_the_sampled_row_nearest_the_sample_centroid():
+    """sum_c (9 x_a[c] - sum_c)^2 = 81 |x_a - mean|^2, so the candidate the detector settles on
+    is the sampled row closest to the mean of the nine sampled rows (reference
+    quantize_qk_impl.cuh:442-577): a closed form that shares no expression with the oracle."""
+    r = np.random.default_rng(11)
+    for length in (9, 64, 257, 1000):
+        k = (r.standard_normal((1, 4, length, 128)) * 0.05 + r.standard_normal((1, 4, 1, 128))).astype(np.float32)
+        anchor = prepare.detect_key_anchor(k)
+        rows = [s * (length - 1) // 8 for s in range(9)]
+        for h in range(4):
+            sampled = k[0, h, rows].astype(np.float64)
+            nearest = int(np.argmin(np.linalg.norm(sampled - sampled.mean(0), axis=1)))
+            assert anchor[0, h] == rows[nearest]  # a tight cluster far from the origin always fires
+
+
+def test_anchor_accept_and_reject_rules_on_hand_built_keys():
+    """Accepted iff the shifted samples have less energy and a peak within 12.5 % of the
+    original one (reference quantize_qk_impl.cuh:430-438)."""
+    length, dim = 65, 128
+    rows = [s * (length - 1) // 8 for s in range(9)]
+    # constant offset, tiny spread: shifting removes nearly all the energy -> fires, and on
+    # the row made equal to the offset itself (distance 0 from ... the centroid is nearest to it)
+    k = np.full((1, 1, length, dim), 3.0, np.float32)
+    k[0, 0, rows] += (np.arange(9, dtype=np.float32)[:, None] - 4.0) * 1e-3  # centroid = row of sample 4
+    assert prepare.detect_key_anchor(k)[0, 0] == rows[4]
+    # zero-mean samples: +e and -e alternate, so every candidate's shift raises the energy -> no anchor
+    k = np.zeros((1, 1, length, dim), np.float32)
+    for index, row in enumerate(rows):
+        k[0, 0, row] = 1.0 if index % 2 == 0 else -1.0
+    assert prepare.detect_key_anchor(k)[0, 0] == -1
+    # energy falls but the peak grows by more than 12.5 %: eight samples at +1 and one at -0.2;
+    # the best candidate is a +1 row, which leaves a residual peak of 1.2 > 1.125
+    k = np.zeros((1, 1, length, dim), np.float32)
+    k[0, 0, rows] = 1.0
+    k[0, 0, rows[8]] = -0.2
+    assert prepare.detect_key_anchor(k)[0, 0] == -1
+    # same construction with the odd sample at +0.2 (residual peak 0.8): accepted, first +1 row wins
+    k[0, 0, rows[8]] = 0.2
+    assert prepare.detect_key_anchor(k)[0, 0] == rows[0]
+    # all samples zero: the energy does not fall strictly -> rejected
+    assert prepare.detect_key_anchor(np.zeros((1, 1, length, dim), np.float32))[0, 0] == -1
+
+
 def test_key_shift_is_softmax_invariant():
     """Subtracting the anchor changes every score of a row by the same amount."""
     r = np.random.default_rng(5)

@@ -74,6 +74,57 @@ def test_noalloc_entry_point_with_a_permutation_and_strided_values(risa):
         assert torch.equal(ours, theirs)
 
 
+@pytest.mark.parametrize("mode", ["absmax", "midpoint_affine"])
+def test_noalloc_entry_point_allocates_nothing_and_replays_from_a_graph(risa, mode):
+    """What the entry point exists for: after its first call on a device it changes nothing in
+    the device's free memory, and a call recorded into a HIP graph replays bit-equal to
+    risa_quantize_v on whatever the input buffer holds at the time of the replay."""
+    from risaattention_amd import native
+    from risaattention_amd.policy import DTYPE_CODES
+
+    lib = native.library()
+    batch, heads, length, dim, cta_k = 1, 4, 5000, 128, 128
+    padded = -(-length // cta_k) * cta_k
+    affine = int(mode == "midpoint_affine")
+    generator = torch.Generator(device="cuda").manual_seed(9)
+    v = torch.randn(batch, heads, length, dim, generator=generator, device="cuda").to(torch.bfloat16)
+    outputs = (torch.zeros(batch * heads * dim, padded, dtype=torch.int8, device="cuda"),
+               torch.zeros(batch * heads * dim, device="cuda"), torch.zeros(batch * heads * dim, device="cuda"),
+               torch.zeros(batch * heads, padded // cta_k, dim, dtype=torch.int32, device="cuda"))
+
+    def call(stream):
+        native.check(lib.risa_quantize_v_noalloc(
+            v.data_ptr(), *(t.data_ptr() for t in outputs), batch, heads, length, dim, padded, cta_k,
+            *v.stride()[:3], DTYPE_CODES[v.dtype], affine, None, stream))
+
+    call(native.current_stream(v.device))  # resolves the array's address on this device
+    torch.cuda.synchronize()
+    free_before, _ = torch.cuda.mem_get_info()
+    call(native.current_stream(v.device))
+    torch.cuda.synchronize()
+    free_after, _ = torch.cuda.mem_get_info()
+    assert free_after == free_before
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            call(side.cuda_stream)
+    for step in range(3):
+        # eager work and a synchronisation between the replays
+        v.copy_((torch.randn(v.shape, generator=generator, device="cuda") * (step + 1) - 0.5 * step).to(v.dtype))
+        for t in outputs:
+            t.fill_(3)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        _, _, expected, _ = _prepare_both(risa, v, mode, cta_k)
+        torch.cuda.synchronize()
+        for ours, theirs, name in zip(outputs, expected, ("codes", "scale", "center", "tile_sum")):
+            assert torch.equal(ours, theirs), (step, name)
+
+
 def test_noalloc_entry_point_rejects_problems_beyond_its_array(risa):
     from risaattention_amd import native
 
