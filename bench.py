@@ -16,8 +16,14 @@ The other workloads (``--workload``) follow the reference's measurement protocol
 (benchmarks/common.py:184-220): every method is warmed up, then timed in samples of
 several calls between two events, with the methods' positions rotated through every slot
 and each complete rotation reversed; seeds 0/1/2; medians of the per-seed medians.
-``--output FILE`` writes the records as JSON (schema of benchmarks/common.py:321-360) and
-``--report FILE`` prints such a file as Markdown tables.
+``--output FILE`` writes the records as JSON (schema of benchmarks/common.py:321-360),
+``--report FILE`` prints such a file as Markdown tables and ``--plot PNG`` draws its dense-
+equivalent throughput and SQNR over the sequence length (the role of reference
+benchmarks/plot_scaling.py).  ``--workload mask_tiles`` is the broadcast-mask comparison of
+reference benchmarks/masks.py (interleaved empty key tiles, optionally against a second build of
+the library given with ``--baseline-library``); ``--workload profile_ranges`` wraps warmed calls in
+named profiler ranges for ``rocprofv3 --marker-trace`` (the role of reference
+benchmarks/profile_operators.py).
 """
 
 from __future__ import annotations
@@ -57,15 +63,19 @@ def make_inputs(torch, length, seed, device):
     return q, k, v
 
 
-def fp32_reference(torch, q, k, v, chunk=2048):
-    """FP32 SDPA in query chunks (reference benchmarks/common.py:134-145)."""
+def fp32_reference(torch, q, k, v, chunk=2048, mask=None):
+    """FP32 SDPA in query chunks (reference benchmarks/common.py:134-145); ``mask`` is a
+    broadcastable boolean (True = visible) or additive mask."""
     group = q.shape[1] // k.shape[1]
     kf = k.float().repeat_interleave(group, 1).transpose(-1, -2)
     vf = v.float().repeat_interleave(group, 1)
     out = torch.empty(q.shape, dtype=torch.float32, device=q.device)
     for start in range(0, q.shape[2], chunk):
         scores = q[:, :, start : start + chunk].float() @ kf * q.shape[-1] ** -0.5
-        out[:, :, start : start + chunk] = torch.softmax(scores, dim=-1) @ vf
+        if mask is not None:
+            rows = mask if mask.shape[-2] == 1 else mask[..., start : start + chunk, :]
+            scores = scores.masked_fill(~rows, float("-inf")) if rows.dtype == torch.bool else scores + rows
+        out[:, :, start : start + chunk] = torch.softmax(scores, dim=-1).nan_to_num(nan=0.0) @ vf
     return out
 
 
@@ -231,6 +241,28 @@ def workload_sweep(torch, risa, args, device):
                          "nrmse_std": round(summary["nrmse_std"], 6), "sqnr_db": round(summary["sqnr_db"], 2),
                          "peak_incremental_mib": round(summary["peak_incremental_mib"], 1)})
     return rows
+
+
+def sweep_cells(torch, risa, device, skip=((32768, "absmax"),), seed=0):
+    """The other cells of the reference's dense table (README.md:115-123) on one seed, for the
+    default line: whole-call latency (mean of a few back-to-back calls) and NRMSE against FP32
+    SDPA per sequence length and V mode.  ``--workload sweep`` is the full protocol."""
+    batch, q_heads, kv_heads, dim = SHAPE["batch"], SHAPE["q_heads"], SHAPE["kv_heads"], SHAPE["head_dim"]
+    cells = []
+    for length in (512, 1024, 2048, 4096, 8192, 16384, 32768):
+        ops = dense_equivalent_ops(batch, q_heads, length, length, dim)
+        q, k, v = make_inputs(torch, length, seed, device)
+        reference = fp32_reference(torch, q, k, v)
+        for mode in ("absmax", "midpoint_affine"):
+            if (length, mode) in skip:
+                continue
+            call = lambda: risa.int8_attention(q, k, v, v_quantization=mode)
+            ms = time_calls(torch, call, calls_for(ops) * 2, warmup=3)
+            cells.append({"N": length, "v_quantization": mode, "ms": round(ms, 4),
+                          "tops": round(ops / (ms * 1e-3) / 1e12, 1),
+                          "nrmse": round(accuracy(torch, call(), reference)["nrmse"], 5)})
+        del reference
+    return cells
 
 
 def outlier_inputs(torch, shape_q, shape_k, seed, device):
@@ -509,6 +541,194 @@ def workload_video(torch, risa, args, device):
             "loop_speedup_vs_dense": round(10 * dense_ms / (construct_ms + sum(reuse)), 3)}
 
 
+def empty_key_tiles(tiles, fraction):
+    """Which key tiles a broadcast mask hides for a given empty fraction: the first
+    ``int(tiles * fraction)`` of the order even tiles, then odd tiles, so that hidden and
+    visible tiles interleave instead of forming a prefix (reference benchmarks/masks.py:60-66)."""
+    order = list(range(0, tiles, 2)) + list(range(1, tiles, 2))
+    return sorted(order[: int(tiles * fraction)])
+
+
+def interleaved_key_mask(torch, k_len, head_dim, fraction, mask_dtype, device):
+    """[1,1,1,Lk] key mask with whole key tiles hidden; boolean, or FP32 with -inf for hidden keys."""
+    tile = 64 if head_dim <= 64 or k_len <= 1024 else 128
+    visible = torch.ones(1, 1, 1, k_len, dtype=torch.bool, device=device)
+    for index in empty_key_tiles(-(-k_len // tile), fraction):
+        visible[..., index * tile : (index + 1) * tile] = False
+    if mask_dtype == "fp32":
+        return torch.zeros(visible.shape, dtype=torch.float32, device=device).masked_fill(~visible, float("-inf"))
+    return visible
+
+
+def workload_mask_tiles(torch, risa, args, device):
+    """Broadcast key masks that hide 0 / 25 / 50 / 75 % of the key tiles, boolean and FP32: what
+    skipping whole tiles saves.  With ``--baseline-library`` every call is also made through that
+    second build in the same process: outputs compared first, then both timed in one rotating group
+    (the protocol of reference benchmarks/masks.py:40-110 over compare_native.py:40-53)."""
+    from risaattention_amd import native
+
+    batch, q_heads, kv_heads, dim = SHAPE["batch"], SHAPE["q_heads"], SHAPE["kv_heads"], SHAPE["head_dim"]
+    length = args.length or 4096
+    fractions = args.empty_fraction or [0.0, 0.25, 0.5, 0.75]
+    if any(not 0.0 <= fraction <= 1.0 for fraction in fractions):
+        raise SystemExit("--empty-fraction must lie in [0, 1]")
+    mask_dtypes = ("bool", "fp32") if args.mask_dtype == "both" else (args.mask_dtype,)
+    modes = ("absmax", "midpoint_affine") if args.v_modes == "both" else (args.v_modes,)
+    baseline = native.load_library(args.baseline_library) if args.baseline_library else None
+    ops = dense_equivalent_ops(batch, q_heads, length, length, dim)
+    case = case_label(batch, q_heads, kv_heads, length, length, dim)
+    shape = dict(batch=batch, q_heads=q_heads, kv_heads=kv_heads, q_len=length, k_len=length, head_dim=dim)
+    first = len(RECORDS)
+    for seed in SEEDS:
+        q, k, v = make_inputs(torch, length, seed, device)
+        for mask_dtype in mask_dtypes:
+            for fraction in fractions:
+                mask = interleaved_key_mask(torch, length, dim, fraction, mask_dtype, device)
+                reference = fp32_reference(torch, q, k, v, mask=mask)
+                methods, errors, comparisons = {}, {}, {}
+                for mode in modes:
+                    call = lambda mode=mode: risa.int8_attention(q, k, v, attn_mask=mask, v_quantization=mode)
+                    after = call()
+                    errors[f"after/{mode}"] = accuracy(torch, after, reference)
+                    methods[f"after/{mode}"] = call
+                    if baseline is not None:
+                        def through_baseline(call=call):
+                            with native.using_library(baseline):
+                                return call()
+
+                        before = through_baseline()
+                        torch.testing.assert_close(before, after, atol=0.002, rtol=0.01)
+                        comparisons[mode] = {"bitwise_equal": torch.equal(before, after),
+                                             "max_abs_difference": (before.float() - after.float()).abs().max().item()}
+                        errors[f"before/{mode}"] = accuracy(torch, before, reference)
+                        methods[f"before/{mode}"] = through_baseline
+                timing = measure_methods(torch, methods, samples=args.samples, calls_per_sample=calls_for(ops),
+                                         warmup=args.method_warmup)
+                for name in methods:
+                    label, mode = name.split("/")
+                    add_record(case, shape, seed, "normal", "normal", mode, f"{label}/mask_{mask_dtype}_empty_{fraction}",
+                               timing[name], errors[name])
+                    RECORDS[-1].update(mask_empty_fraction=fraction, mask_dtype=mask_dtype, build=label,
+                                       native_comparison=comparisons.get(mode))
+                del reference
+    return mask_tile_rows(RECORDS[first:], ops)
+
+
+def mask_tile_rows(records, ops):
+    """Summary rows of the mask-tile records: per (build, mask dtype, V mode, empty fraction) the
+    median over the seeds of the per-seed medians, its ratio to the same method with nothing
+    hidden, and the mean NRMSE."""
+    rows = []
+    for summary in summarize_records(records):
+        members = [record for record in records if record["stage"] == summary["stage"]
+                   and record["v_quantization"] == summary["v_quantization"]]
+        rows.append({"build": members[0]["build"], "mask_dtype": members[0]["mask_dtype"],
+                     "v_quantization": summary["v_quantization"], "empty_fraction": members[0]["mask_empty_fraction"],
+                     "ms": round(summary["median_ms"], 4), "tops": round(ops / (summary["median_ms"] * 1e-3) / 1e12, 1),
+                     "nrmse": None if summary["nrmse"] is None else round(summary["nrmse"], 5),
+                     "bitwise_equal_to_baseline": (None if members[0]["native_comparison"] is None else
+                                                   all(member["native_comparison"]["bitwise_equal"] for member in members))})
+    for row in rows:
+        full = [other["ms"] for other in rows if other["empty_fraction"] == 0.0 and
+                all(other[key] == row[key] for key in ("build", "mask_dtype", "v_quantization"))]
+        row["vs_nothing_hidden"] = round(row["ms"] / full[0], 3) if full else None
+    return rows
+
+
+def profile_range_names(stage, modes):
+    """Names of the profiler ranges one pass of ``--workload profile_ranges`` opens, in order."""
+    return [f"risa/{stage}/{mode}" for mode in modes]
+
+
+def workload_profile_ranges(torch, risa, args, device):
+    """Warmed calls inside named profiler ranges (torch.cuda.nvtx is rocTX on PyTorch-ROCm), for
+    ``rocprofv3 --marker-trace --kernel-trace -- python3 bench.py --workload profile_ranges``.
+    No latency is reported: durations under a profiler are not benchmark figures (reference
+    benchmarks/profile_operators.py:1-66)."""
+    length = args.length or 512
+    modes = ("absmax", "midpoint_affine") if args.v_modes == "both" else (args.v_modes,)
+    q, k, v = make_inputs(torch, length, 0, device)
+    methods = {}
+    for mode in modes:
+        if args.stage == "attend":
+            packed = risa.prequantize_int8_attention(q, k, v, v_quantization=mode)
+            methods[mode] = lambda packed=packed: risa.int8_attention_from_prequantized(packed)
+        elif args.stage == "quantize":
+            methods[mode] = lambda mode=mode: risa.prequantize_int8_attention(q, k, v, v_quantization=mode)
+        else:
+            methods[mode] = lambda mode=mode: risa.int8_attention(q, k, v, v_quantization=mode)
+    for method in methods.values():
+        for _ in range(args.method_warmup):
+            method()
+    torch.cuda.synchronize()
+    names = profile_range_names(args.stage, modes)
+    for _ in range(args.calls):
+        for name, method in zip(names, methods.values()):
+            with torch.cuda.nvtx.range(name):
+                method()
+    torch.cuda.synchronize()
+    return [{"N": length, "stage": args.stage, "range": name, "calls": args.calls, "warmup": args.method_warmup}
+            for name in names]
+
+
+def scaling_series(records):
+    """What the scaling plot shows, from per-seed records: for every method (stage and V mode)
+    and sequence length, the dense-equivalent TOPS of the median over the seeds of the per-seed
+    median latencies and the mean SQNR (reference benchmarks/plot_scaling.py:66-75, 118-133:
+    4*B*Hq*Lq*Lk*D operations whatever the method skips).  Only equal Q/K lengths are plotted."""
+    series = {}
+    for row in summarize_records([r for r in records if r["shape"]["q_len"] == r["shape"]["k_len"]]):
+        shape = next(r["shape"] for r in records if r["case"] == row["case"])
+        ops = dense_equivalent_ops(shape["batch"], shape["q_heads"], shape["q_len"], shape["k_len"], shape["head_dim"])
+        label = f"{row['stage']}/{row['v_quantization']}"
+        series.setdefault(label, []).append({"length": shape["q_len"], "tops": ops / (row["median_ms"] * 1e-3) / 1e12,
+                                             "sqnr_db": row["sqnr_db"], "sqnr_db_std": None})
+    for label, points in series.items():
+        points.sort(key=lambda point: point["length"])
+    return series
+
+
+def plot_scaling(series, path, title):
+    """Grouped bars over the sequence length: SQNR against FP32 SDPA on the left (methods that
+    carry accuracy records), dense-equivalent throughput on the right."""
+    import matplotlib
+
+    matplotlib.use("Agg")
+    import matplotlib.pyplot as plt
+
+    lengths = sorted({point["length"] for points in series.values() for point in points})
+    tick = lambda n: f"{n // 1024}K" if n % 1024 == 0 else str(n)
+    figure, (left, right) = plt.subplots(1, 2, figsize=(15, 5.5))
+    panels = ((left, "sqnr_db", "SQNR vs FP32 SDPA (dB, higher is better)", "Accuracy", "{:.1f}"),
+              (right, "tops", "Dense-equivalent throughput (TOP/s)", "Speed", "{:.0f}"))
+    for axis, metric, ylabel, name, text in panels:
+        shown = {label: points for label, points in series.items() if any(p[metric] is not None for p in points)}
+        width = 0.8 / max(1, len(shown))
+        for index, (label, points) in enumerate(sorted(shown.items())):
+            by_length = {p["length"]: p[metric] for p in points}
+            heights = [by_length.get(n) or 0.0 for n in lengths]
+            places = [x + (index - (len(shown) - 1) / 2) * width for x in range(len(lengths))]
+            bars = axis.bar(places, heights, width, label=label, edgecolor="black", linewidth=0.8)
+            for bar, height in zip(bars, heights):
+                if height:
+                    axis.annotate(text.format(height), (bar.get_x() + bar.get_width() / 2, height), xytext=(0, 4),
+                                  textcoords="offset points", ha="center", va="bottom", rotation=90, fontsize=7)
+        axis.set_xticks(range(len(lengths)), [tick(n) for n in lengths])
+        axis.set_xlabel("Sequence length")
+        axis.set_ylabel(ylabel)
+        axis.set_title(name)
+        axis.grid(axis="y", linewidth=0.5, alpha=0.6)
+        axis.set_axisbelow(True)
+        axis.margins(y=0.18)
+        if shown:
+            axis.legend(fontsize=8)
+    figure.suptitle(title)
+    figure.tight_layout()
+    path.parent.mkdir(parents=True, exist_ok=True)
+    figure.savefig(path, dpi=130)
+    plt.close(figure)
+
+
 def cpu_baseline(length=1024, calls=15):
     """Oracle (numpy port of the quantised pipeline) on the host cores: the reference's own
     CPU-sized configuration (same heads and head dim as the headline, N=1024, seed 0,
@@ -568,8 +788,10 @@ def write_records(torch, risa, args, rows):
             digest.update(path.read_bytes())
     library = Path(native.library_path())
     config = {key: (str(value) if isinstance(value, Path) else value) for key, value in vars(args).items()
-              if key not in ("output", "report", "csv", "markdown")}
-    paired = args.workload in ("sweep", "masked", "sparse_blocks")
+              if key not in ("output", "report", "csv", "markdown", "plot")}
+    if args.baseline_library is not None:
+        config["baseline_library_sha256"] = hashlib.sha256(Path(args.baseline_library).read_bytes()).hexdigest()
+    paired = args.workload in ("sweep", "masked", "sparse_blocks", "mask_tiles")
     config["timing_order"] = "rotate-and-reverse" if paired else "back-to-back calls between two events"
     config["seeds"] = list(SEEDS) if paired else [0]
     payload = {
@@ -637,7 +859,9 @@ def main():
     parser.add_argument("--mode", default="absmax", choices=["absmax", "midpoint_affine"])
     parser.add_argument("--no-cpu-baseline", action="store_true")
     parser.add_argument("--no-accuracy", action="store_true")
-    parser.add_argument("--workload", default="dense", choices=["dense", "sweep", "masked", "sparse", "sparse_blocks", "video", "prepare"],
+    parser.add_argument("--workload", default="dense",
+                        choices=["dense", "sweep", "masked", "sparse", "sparse_blocks", "video", "prepare", "mask_tiles",
+                                 "profile_ranges"],
                         help="dense = headline N=32K line (default); the others are the remaining benchmark "
                              "configurations of the reference, reported as one JSON line each")
     parser.add_argument("--samples", type=int, default=10, help="event-timed samples per method and seed (--workload)")
@@ -648,11 +872,27 @@ def main():
     parser.add_argument("--report", type=Path, default=None, help="print a file written with --output as a Markdown table and exit")
     parser.add_argument("--csv", type=Path, default=None, help="with --report: also write the summary rows as CSV")
     parser.add_argument("--markdown", type=Path, default=None, help="with --report: also write the table to this file")
+    parser.add_argument("--plot", type=Path, default=None,
+                        help="with --report: also draw SQNR and dense-equivalent TOPS over the sequence length (PNG)")
+    parser.add_argument("--empty-fraction", action="append", type=float,
+                        help="mask_tiles: fraction of key tiles hidden (repeatable; default 0, 0.25, 0.5, 0.75)")
+    parser.add_argument("--mask-dtype", choices=("bool", "fp32", "both"), default="both", help="mask_tiles: mask element type")
+    parser.add_argument("--v-modes", choices=("absmax", "midpoint_affine", "both"), default="both",
+                        help="mask_tiles / profile_ranges: V quantisation modes to run")
+    parser.add_argument("--baseline-library", type=Path, default=None,
+                        help="mask_tiles: a second build of the C-ABI library to compare and time against")
+    parser.add_argument("--stage", choices=("dense", "quantize", "attend"), default="dense", help="profile_ranges: what a range wraps")
+    parser.add_argument("--calls", type=int, default=10, help="profile_ranges: ranges per V mode")
     parser.add_argument("--calibrate-copy", action="store_true",
                         help="only run a 1 GiB device copy (reference point for rocprofv3 FETCH_SIZE/WRITE_SIZE)")
     args = parser.parse_args()
     if args.report is not None:
-        table = render_report(json.loads(args.report.read_text()), args.csv)
+        payload = json.loads(args.report.read_text())
+        table = render_report(payload, args.csv)
+        if args.plot is not None:
+            environment = payload["environment"]
+            plot_scaling(scaling_series(payload.get("results") or []), args.plot,
+                         f"{payload['suite']} - {environment['gpu']} ({environment.get('arch', '')})")
         if args.markdown is not None:
             args.markdown.parent.mkdir(parents=True, exist_ok=True)
             args.markdown.write_text(table + "\n")
@@ -683,7 +923,8 @@ def main():
     if args.workload != "dense":
         runner = {"sweep": workload_sweep, "masked": workload_masked, "sparse": workload_sparse,
                   "video": workload_video, "prepare": workload_prepare,
-                  "sparse_blocks": workload_sparse_blocks}[args.workload]
+                  "sparse_blocks": workload_sparse_blocks, "mask_tiles": workload_mask_tiles,
+                  "profile_ranges": workload_profile_ranges}[args.workload]
         wall = time.perf_counter()
         rows = runner(torch, risa, args, device)
         if args.output is not None:
@@ -768,11 +1009,13 @@ def main():
     if not args.no_side_measurements:
         del out
         result["config"]["sparse_reuse"] = sparse_blocks_case(
-            torch, risa, length, args.mode, seeds=(0,), samples=6, method_warmup=3, device=device, with_quality=False)
+            torch, risa, length, args.mode, seeds=SEEDS, samples=10, method_warmup=3, device=device, with_quality=False)
         result["config"]["sparse_reuse"]["note"] = (
             "BASELINE config 4's own recipe (64 groups, centroid x 3) keeps 1.6 % of the tiles and is not this row: "
             "see --workload sparse")
         result["config"]["masked"] = workload_masked(torch, risa, args, device, dims=(128, 64), seeds=(0,), samples=4)
+        if length == 32768:
+            result["config"]["sweep"] = sweep_cells(torch, risa, device, skip=((32768, args.mode),))
         out = step()
     if not args.no_accuracy:
         reference = fp32_reference(torch, q, k, v)

@@ -171,6 +171,11 @@ def sdpa_workspace_bytes(*extents) -> int:
     return native.library().risa_sdpa_workspace_bytes(*extents)
 
 
+def forget_cached_sizes() -> None:
+    """Drop the remembered workspace sizes (they belong to the library that computed them)."""
+    sdpa_workspace_bytes.cache_clear()
+
+
 def execute_dense_attention(
     q: torch.Tensor,
     k: torch.Tensor,

@@ -9,6 +9,7 @@ pointers plus element strides, so no DLPack capsule is involved.
 
 from __future__ import annotations
 
+import contextlib
 import ctypes
 import os
 from pathlib import Path
@@ -93,20 +94,45 @@ def library_path() -> Path:
     return Path(override) if override else Path(__file__).resolve().parent / LIBRARY_NAME
 
 
+def load_library(path: Path | str) -> ctypes.CDLL:
+    """Another build of the C-ABI library (same entry points), with its signatures bound.
+    Raises OSError / AttributeError when the file cannot be loaded or lacks an entry point."""
+    loaded = ctypes.CDLL(str(path))
+    for name, (restype, argtypes) in SIGNATURES.items():
+        function = getattr(loaded, name)
+        function.restype = restype
+        function.argtypes = argtypes
+    return loaded
+
+
 def _load() -> ctypes.CDLL | None:
     global _LIBRARY, _LOAD_ERROR
     if _LIBRARY is not None or _LOAD_ERROR is not None:
         return _LIBRARY
     try:
-        library = ctypes.CDLL(str(library_path()))
-        for name, (restype, argtypes) in SIGNATURES.items():
-            function = getattr(library, name)
-            function.restype = restype
-            function.argtypes = argtypes
-        _LIBRARY = library
+        _LIBRARY = load_library(library_path())
     except (OSError, AttributeError) as error:
         _LOAD_ERROR = error
     return _LIBRARY
+
+
+@contextlib.contextmanager
+def using_library(other: ctypes.CDLL):
+    """Route every call made inside the block to *other* (from ``load_library``): the paired
+    comparison of two builds in one process that the reference's benchmark runners do by
+    swapping ``_backend._C`` (reference benchmarks/compare_native.py:40-53).  Sizes cached per
+    shape are dropped on the way in and out, since two builds may lay out workspaces differently."""
+    global _LIBRARY
+    from . import attend
+
+    previous = _load()
+    attend.forget_cached_sizes()
+    _LIBRARY = other
+    try:
+        yield other
+    finally:
+        _LIBRARY = previous
+        attend.forget_cached_sizes()
 
 
 def library() -> ctypes.CDLL:

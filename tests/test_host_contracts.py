@@ -395,3 +395,121 @@ def test_bench_paired_timing_rotates_and_reverses_positions():
         assert "| B1_Hq16_Hkv4_Lq512_Lk512_D128 | absmax | dense | 3 | 0.026 |" in report
         header, first, *_ = csv_path.read_text().splitlines()
         assert header.startswith("case,layout,qk_distribution") and "0.026" in first
+
+
+def _bench_module():
+    import importlib.util
+
+    spec = importlib.util.spec_from_file_location("bench_module", ROOT / "bench.py")
+    bench = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(bench)
+    return bench
+
+
+def _bench_record(length, seed, median_ms, stage="dense", mode="absmax", sqnr=36.0, **extra):
+    record = {"case": f"B1_Hq16_Hkv4_Lq{length}_Lk{length}_D128",
+              "shape": {"batch": 1, "q_heads": 16, "kv_heads": 4, "q_len": length, "k_len": length, "head_dim": 128},
+              "seed": seed, "layout": "hnd", "qk_distribution": "normal", "value_distribution": "normal",
+              "implementation": "risaattention_amd", "v_quantization": mode, "stage": stage,
+              "timing": {"median_ms": median_ms, "p10_ms": median_ms, "p90_ms": median_ms},
+              "accuracy": None if sqnr is None else {"nrmse": 10 ** (-sqnr / 20), "rmse": 1e-4, "sqnr_db": sqnr, "mae": 1e-4,
+                                                     "max_abs": 1e-3, "max_channel_bias": 1e-4},
+              "memory": None, "sparse": None}
+    record.update(extra)
+    return record
+
+
+def test_bench_mask_tile_benchmark_inputs_and_rows():
+    """The broadcast-mask benchmark (reference benchmarks/masks.py:40-75): hidden tiles are taken
+    from the order evens-then-odds, so they interleave with visible ones; the rows report every
+    method against the same method with nothing hidden."""
+    import torch
+
+    bench = _bench_module()
+    assert bench.empty_key_tiles(8, 0.0) == []
+    assert bench.empty_key_tiles(8, 0.25) == [0, 2]
+    assert bench.empty_key_tiles(8, 0.5) == [0, 2, 4, 6]
+    assert bench.empty_key_tiles(8, 0.75) == [0, 1, 2, 3, 4, 6]  # all evens, then odds 1 and 3
+    assert bench.empty_key_tiles(5, 1.0) == [0, 1, 2, 3, 4]
+    mask = bench.interleaved_key_mask(torch, 2048, 128, 0.25, "bool", "cpu")  # 16 tiles of 128 keys
+    assert mask.shape == (1, 1, 1, 2048) and mask.dtype == torch.bool
+    hidden = (~mask).reshape(16, 128)
+    assert hidden.all(1).tolist() == [tile in (0, 2, 4, 6) for tile in range(16)] and not hidden[1].any()
+    short = bench.interleaved_key_mask(torch, 1024, 128, 0.5, "fp32", "cpu")  # 64-key tiles up to 1024 keys
+    assert short.dtype == torch.float32 and torch.isneginf(short).sum().item() == 512
+    assert torch.isneginf(short.reshape(16, 64)).all(1).tolist() == [tile % 2 == 0 for tile in range(16)]
+    assert (short[torch.isfinite(short)] == 0).all()
+
+    records = []
+    for fraction, ms in ((0.0, 0.100), (0.5, 0.060)):
+        for seed, jitter in ((0, 0.0), (1, 0.002), (2, -0.002)):
+            for build, slower in (("after", 1.0), ("before", 1.5)):
+                records.append(_bench_record(4096, seed, (ms + jitter) * slower, stage=f"{build}/mask_bool_empty_{fraction}",
+                                             mask_empty_fraction=fraction, mask_dtype="bool", build=build,
+                                             native_comparison={"bitwise_equal": seed != 2, "max_abs_difference": 0.0}))
+    ops = bench.dense_equivalent_ops(1, 16, 4096, 4096, 128)
+    rows = {(row["build"], row["empty_fraction"]): row for row in bench.mask_tile_rows(records, ops)}
+    assert rows[("after", 0.5)]["ms"] == 0.06 and rows[("after", 0.5)]["vs_nothing_hidden"] == 0.6
+    assert rows[("before", 0.0)]["ms"] == pytest.approx(0.15) and rows[("before", 0.5)]["vs_nothing_hidden"] == 0.6
+    assert rows[("after", 0.0)]["tops"] == pytest.approx(ops / 0.1e-3 / 1e12, rel=1e-3)
+    assert rows[("after", 0.0)]["bitwise_equal_to_baseline"] is False  # one seed differed
+
+
+def test_bench_scaling_plot_inputs_and_figure(tmp_path):
+    """Dense-equivalent TOPS over N for the plot (reference benchmarks/plot_scaling.py:66-75):
+    4*B*Hq*Lq*Lk*D operations over the median of the per-seed medians, whatever a method skips."""
+    bench = _bench_module()
+    records = []
+    for length, ms in ((1024, 0.02), (4096, 0.1)):
+        for seed, jitter in ((0, 0.0), (1, 0.01), (2, -0.005)):
+            records.append(_bench_record(length, seed, ms + jitter, sqnr=36.0 + seed))
+            records.append(_bench_record(length, seed, (ms + jitter) / 2, stage="reuse", sqnr=None))
+    records.append(_bench_record(2048, 0, 1.0) | {"shape": {"batch": 1, "q_heads": 16, "kv_heads": 4, "q_len": 2048,
+                                                            "k_len": 4096, "head_dim": 128}})  # unequal lengths: left out
+    series = bench.scaling_series(records)
+    assert set(series) == {"dense/absmax", "reuse/absmax"}
+    dense = series["dense/absmax"]
+    assert [point["length"] for point in dense] == [1024, 4096]
+    assert dense[0]["tops"] == pytest.approx(4 * 16 * 1024 * 1024 * 128 / 0.02e-3 / 1e12)
+    assert dense[1]["sqnr_db"] == pytest.approx(37.0)
+    assert series["reuse/absmax"][1]["tops"] == pytest.approx(2 * dense[1]["tops"]) and series["reuse/absmax"][1]["sqnr_db"] is None
+    target = tmp_path / "figures" / "scaling.png"
+    bench.plot_scaling(series, target, "sweep - MI355X (gfx950)")
+    assert target.read_bytes()[:8] == b"\x89PNG\r\n\x1a\n" and target.stat().st_size > 10_000
+
+
+def test_bench_profile_range_names():
+    """One range per V mode and pass, named like the reference's (benchmarks/profile_operators.py:53-61)."""
+    bench = _bench_module()
+    assert bench.profile_range_names("dense", ("absmax", "midpoint_affine")) == ["risa/dense/absmax", "risa/dense/midpoint_affine"]
+    assert bench.profile_range_names("attend", ("absmax",)) == ["risa/attend/absmax"]
+
+
+def test_library_swap_routes_calls_and_restores():
+    """native.using_library: calls inside the block reach the other build, the cached workspace
+    sizes are dropped on both edges, and the in-tree library is back afterwards (also after an error)."""
+    from risaattention_amd import attend
+
+    own = native.library()
+    other = native.load_library(native.library_path())  # a second handle on the same file
+    assert other.risa_abi_version() == own.risa_abi_version()
+
+    class Recorder:
+        def __getattr__(self, name):
+            return getattr(other, name)
+
+        def risa_abi_version(self):
+            return -7
+
+    attend.sdpa_workspace_bytes(1, 2, 64, 2, 64, 128, 64, 0, -1, 0, 1, 1, 1)
+    assert attend.sdpa_workspace_bytes.cache_info().currsize >= 1
+    with native.using_library(Recorder()):
+        assert attend.sdpa_workspace_bytes.cache_info().currsize == 0
+        assert native.library().risa_abi_version() == -7
+    assert native.library() is own and attend.sdpa_workspace_bytes.cache_info().currsize == 0
+    with pytest.raises(KeyError):
+        with native.using_library(Recorder()):
+            raise KeyError("inside")
+    assert native.library() is own
+    with pytest.raises(OSError):
+        native.load_library(ROOT / "no_such_library.so")
