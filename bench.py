@@ -721,7 +721,7 @@ def plot_scaling(series, path, title):
         axis.set_axisbelow(True)
         axis.margins(y=0.18)
         if shown:
-            axis.legend(fontsize=8)
+            axis.legend(fontsize=7, loc="upper center", bbox_to_anchor=(0.5, -0.12), ncol=2 if len(shown) > 4 else len(shown))
     figure.suptitle(title)
     figure.tight_layout()
     path.parent.mkdir(parents=True, exist_ok=True)

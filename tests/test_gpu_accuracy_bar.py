@@ -3,19 +3,23 @@ B=1, Hq=16, Hkv=4, D=128, bf16 N(0,1) inputs, N = 512 ... 32K, both V modes, mea
 0/1/2 of the record of benchmarks/common.py:148-164.  The bar is the README's figure to its
 printed precision (figure + 0.00005).
 
-Eleven of the fourteen cells meet it.  Three cells at N <= 1K come out 0.2-1.2 % above it with
-this platform's device generator, and the test says why instead of widening the bar for all:
+The eight cells from N = 4K on meet it.  Up to 2K the three-seed mean sits within +-1.2 % of the
+figure with this platform's device generator (512 both modes +1.2 / +1.4 %, 1K absmax +0.6 %, 2K
+midpoint_affine +0.4 % of the figure, i.e. 0.1-0.9 % over the bar; 1K midpoint_affine and 2K
+absmax under it), with a seed-to-seed spread of up to 1.7 % at 2K.  The test says why instead of
+widening the bar for all cells:
 
 * the kernels are not the cause: on the same tensors the oracle's NRMSE equals theirs to five
   digits (asserted below);
 * the draws are: the figure moves by several per cent with the tails of the input sample (the
   V and Q/K scales are extreme-value statistics of at most a few thousand draws at these
   lengths).  The same kernels on the CPU generator's bf16 draws of the same seeds meet the
-  README's figure in all three cells (asserted below); the README's numbers come from a third
+  README's figure in every one of these cells (asserted below); the README's numbers come from a third
   generator (CUDA's) that nothing here can reproduce, and at N >= 8K this build is 0.4-1.6 %
   *below* the README with the device generator.
 
-The allowance for those three cells is 1.5 % of the figure, stated per cell in ALLOWED.
+The allowance for the cells up to 2K is 1.5 % of the figure (ALLOWED); each of them is also
+held to the two assertions above.
 """
 
 import numpy as np
@@ -31,7 +35,7 @@ README_NRMSE = {512: (0.0145, 0.0136), 1024: (0.0149, 0.0140), 2048: (0.0158, 0.
                 8192: (0.0166, 0.0155), 16384: (0.0168, 0.0156), 32768: (0.0169, 0.0157)}
 PRINTED_PRECISION = 0.00005
 MODES = ("absmax", "midpoint_affine")
-ALLOWED = {(512, "absmax"): 0.015, (1024, "absmax"): 0.015, (512, "midpoint_affine"): 0.015}
+ALLOWED = {(length, mode): 0.015 for length in (512, 1024, 2048) for mode in MODES}
 SEEDS = (0, 1, 2)
 
 
