@@ -963,14 +963,82 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : D == 64 && MASK_MODE == kMaskL
   // --- main loop: one barrier per tile -----------------------------------------
   // At the barrier of iteration t every wave has finished tile t-1 (so stage
   // (t+1)&1 may be overwritten) and has seen its own share of tile t land.
+  // Raw-score launches with head dim 128 and 128-key tiles (dense, or over a sparse pattern's
+  // tile lists) walk every tile but the last in a hand-scheduled loop, written by
+  // gen_dense_loop.py into dense_loop_d128.inc / sparse_loop_d128.inc: same arithmetic in the
+  // same order, bit-identical results.  The loop owns the whole register file, so its operands
+  // are pinned to the registers the generator chose; the last listed tile (the one that may be
+  // partial) and the epilogue stay below.
+  constexpr bool ASM_LOOP = FAST && D == 128 && CTA_K == 128 && !CAPTURE;
+  int first_tile = 0;
+  if constexpr (ASM_LOOP) {
+    if (n_it > 1) {
+      typedef __attribute__((address_space(3))) unsigned char* LdsBytes;
+      const uint32_t lds_address = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((LdsBytes)lds));
+      issue_tile(tile_at(0), 0);
+      v16i out0 = {}, out1 = {}, out2 = {}, out3 = {};
+      // this lane's fragment address per k-step (K) / key block (V): row l32 of a 32-row block
+      const uint32_t a0 = lds_address + swizzled<128>(l32, 0 + half), a1 = lds_address + swizzled<128>(l32, 2 + half);
+      const uint32_t a2 = lds_address + swizzled<128>(l32, 4 + half), a3 = lds_address + swizzled<128>(l32, 6 + half);
+      const uint32_t seed_address = lds_address + half * 16 + 2048;  // (the generator's SEED_BIAS)
+      // lane share of the copy source offsets: the rest, (wave * NC + i) KiB of K or that many
+      // groups of eight V rows, is scalar arithmetic in the loop; the share repeats with period 2 in i
+      const uint32_t kc0 = k_source_offset(0, lane) - static_cast<uint32_t>(wave * NC) * 1024u;
+      const uint32_t kc1 = k_source_offset(1, lane) - static_cast<uint32_t>(wave * NC + 1) * 1024u;
+      const uint32_t vc0 = v_source_offset(0, lane) - static_cast<uint32_t>(wave * NC) * 8u * static_cast<uint32_t>(p.padded);
+      const uint32_t vc1 = v_source_offset(1, lane) - static_cast<uint32_t>(wave * NC + 1) * 8u * static_cast<uint32_t>(p.padded);
+      // dense: sources of tile 1 (the loop advances them); sparse: bases of the head and the tile list
+      const uint64_t k_source = reinterpret_cast<uint64_t>(INDEXED ? k_base : k_base + CTA_K * D);
+      const uint64_t v_source = reinterpret_cast<uint64_t>(INDEXED ? v_base : v_base + CTA_K);
+      const uint64_t sum_source = reinterpret_cast<uint64_t>(INDEXED ? sum_base : sum_base + D);
+      const uint64_t ks_source = reinterpret_cast<uint64_t>(ks_base);
+      const int count = n_it - 1;
+      if constexpr (INDEXED) {
+        const uint64_t list = reinterpret_cast<uint64_t>(indices);
+        asm volatile(
+#include "sparse_loop_d128.inc"
+            : "+{v[128:143]}"(out0), "+{v[144:159]}"(out1), "+{v[160:175]}"(out2), "+{v[176:191]}"(out3),
+              "+{v241}"(m_run), "+{v242}"(d_part)
+            : "{v[192:195]}"(qreg[0]), "{v[196:199]}"(qreg[1]), "{v[200:203]}"(qreg[2]), "{v[204:207]}"(qreg[3]),
+              "{v244}"(q_scale), "{v246}"(a0), "{v247}"(a1), "{v248}"(a2), "{v249}"(a3), "{v250}"(seed_address),
+              "{v251}"(kc0), "{v252}"(kc1), "{v253}"(vc0), "{v254}"(vc1),
+              [kptr] "s"(k_source), [vptr] "s"(v_source), [sumptr] "s"(sum_source), [ksptr] "s"(ks_source),
+              [count] "s"(count), [wave] "s"(wave), [qs2] "s"(qs2), [padded] "s"(p.padded), [list] "s"(list)
+            :
+#include "sparse_loop_d128_clobbers.inc"
+        );
+      } else {
+        asm volatile(
+#include "dense_loop_d128.inc"
+            : "+{v[128:143]}"(out0), "+{v[144:159]}"(out1), "+{v[160:175]}"(out2), "+{v[176:191]}"(out3),
+              "+{v241}"(m_run), "+{v242}"(d_part)
+            : "{v[192:195]}"(qreg[0]), "{v[196:199]}"(qreg[1]), "{v[200:203]}"(qreg[2]), "{v[204:207]}"(qreg[3]),
+              "{v244}"(q_scale), "{v246}"(a0), "{v247}"(a1), "{v248}"(a2), "{v249}"(a3), "{v250}"(seed_address),
+              "{v251}"(kc0), "{v252}"(kc1), "{v253}"(vc0), "{v254}"(vc1),
+              [kptr] "s"(k_source), [vptr] "s"(v_source), [sumptr] "s"(sum_source), [ksptr] "s"(ks_source),
+              [count] "s"(count), [wave] "s"(wave), [qs2] "s"(qs2), [padded] "s"(p.padded)
+            :
+#include "dense_loop_d128_clobbers.inc"
+        );
+      }
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        o_acc[0][i] = __int_as_float(out0[i]);
+        o_acc[1][i] = __int_as_float(out1[i]);
+        o_acc[2][i] = __int_as_float(out2[i]);
+        o_acc[3][i] = __int_as_float(out3[i]);
+      }
+      first_tile = n_it - 1;
+    }
+  }
   if (n_it > 0) {
     v16i s[RB];
     v4i pk[RB];
     v4i k_first[RB];
     v4i v_first[2];
     v16i seed[2];
-    int tile = tile_at(0);
-    issue_tile(tile, 0);
+    int tile = tile_at(first_tile);
+    if (first_tile == 0) issue_tile(tile, 0);
     // The last listed tile reads its mask elements directly (it may be partial).
     if (n_it > 1) issue_mask_tile(tile, 0);
     load_lane_words(tile, 0);
@@ -980,7 +1048,7 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : D == 64 && MASK_MODE == kMaskL
     // needed, ahead of the copies (read where it is needed, its round trip would be
     // waited for in every tile).
     [[maybe_unused]] int listed_next = INDEXED && n_it > 1 ? tile_at(1) : 0;
-    for (int it = 0; it < n_it - 1; ++it) {
+    for (int it = first_tile; it < n_it - 1; ++it) {
       const int stage = it & 1;
       const int next_tile = INDEXED ? listed_next : it + 1;
       __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)

@@ -1,0 +1,82 @@
+"""The hand-scheduled tile loop of the raw-score kernels (head dim 128, 128-key tiles, more
+workgroups than compute units) against the loop the compiler schedules: the capturing launch of
+pattern construction keeps the compiled loop and does the same arithmetic in the same order, so
+the two outputs are equal bit for bit; tile lists are compared with the dense launch where they
+name every tile, and with the oracle walking the same lists otherwise."""
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import pipeline as oracle_pipeline
+from tests.helpers import oracle_prequantize, relative_l2, seeded, to_numpy
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("length", [2048, 2049, 2304, 4096, 4190])
+@pytest.mark.parametrize("mode", ["absmax", "midpoint_affine"])
+def test_dense_loop_equals_the_capturing_launch_bit_for_bit(risa, length, mode):
+    """Odd and even tile counts (the loop is unrolled by two and leaves from either half), a last
+    tile of one key, of half a tile, a whole one."""
+    heads = 20  # x 17..33 query blocks: above the small-launch limit of a 256-CU part
+    q = seeded((1, heads, length, 128), torch.bfloat16, length, scale=1.5)
+    k = seeded((1, 4, length, 128), torch.bfloat16, length + 1, scale=1.5)
+    v = seeded((1, 4, length, 128), torch.bfloat16, length + 2, offset=0.25)
+    dense, dense_lse = risa.int8_attention(q, k, v, v_quantization=mode, return_lse=True)
+    captured, pattern = risa.construct_sparse_int8_attention(q, k, v, theta=0.95, v_quantization=mode)
+    assert torch.equal(dense, captured)
+    checked = 2
+    prepared = oracle_prequantize(q[:, :checked], k[:, :1], v[:, :1], v_quantization=mode, return_lse=True)
+    expected, expected_lse, _ = oracle_pipeline.attend(prepared, return_lse=True)
+    assert relative_l2(to_numpy(dense[:, :checked]), expected) < 1e-3
+    assert relative_l2(to_numpy(dense_lse[:, :checked]), expected_lse) < 1e-3
+
+
+@pytest.mark.parametrize("k_len", [2304, 2300])
+def test_listed_loop_with_every_tile_equals_the_dense_launch(risa, k_len):
+    from risaattention_amd.types import RetainedMassPattern
+
+    heads, q_len = 40, 1024
+    q = seeded((1, heads, q_len, 128), torch.float16, 11)
+    k = seeded((1, 2, k_len, 128), torch.float16, 12)
+    v = seeded((1, 2, k_len, 128), torch.float16, 13, offset=-0.5)
+    packed = risa.prequantize_int8_attention(q, k, v, return_lse=True)
+    assert packed.cta_k == 128
+    tiles, rows = -(-k_len // 128), heads * (q_len // 128)
+    offsets = (np.arange(rows + 1) * tiles).astype(np.int32)
+    indices = np.tile(np.arange(tiles, dtype=np.int32), rows)
+    pattern = RetainedMassPattern(torch.from_numpy(offsets).cuda(), torch.from_numpy(indices).cuda(), 1, heads, q_len,
+                                  k_len, 128, 128, packed.attention_scale, 1.0, 1.0)
+    listed, listed_lse = risa.int8_attention_from_prequantized(packed, sparse_pattern=pattern, return_lse=True)
+    dense, dense_lse = risa.int8_attention_from_prequantized(packed, return_lse=True)
+    assert torch.equal(listed, dense)
+    assert torch.equal(listed_lse, dense_lse)
+
+
+@pytest.mark.parametrize("seed", [0, 1])
+def test_listed_loop_with_random_lists_matches_oracle(risa, seed):
+    """Lists of one to nineteen tiles, each an ascending random subset (with and without the
+    partial last tile), different for every query block."""
+    from risaattention_amd.types import RetainedMassPattern
+
+    heads, q_len, k_len = 36, 1000, 2350
+    q = seeded((1, heads, q_len, 128), torch.bfloat16, 21 + seed)
+    k = seeded((1, 1, k_len, 128), torch.bfloat16, 22 + seed)
+    v = seeded((1, 1, k_len, 128), torch.bfloat16, 23 + seed, offset=0.5)
+    packed = risa.prequantize_int8_attention(q, k, v, return_lse=True)
+    tiles, query_blocks = -(-k_len // 128), -(-q_len // 128)
+    rng = np.random.default_rng(seed)
+    lists = [np.sort(rng.choice(tiles, size=1 + (row * 7 + seed) % tiles, replace=False)) for row in range(heads * query_blocks)]
+    offsets = np.cumsum([0] + [len(entry) for entry in lists]).astype(np.int32)
+    indices = np.concatenate(lists).astype(np.int32)
+    pattern = RetainedMassPattern(torch.from_numpy(offsets).cuda(), torch.from_numpy(indices).cuda(), 1, heads, q_len,
+                                  k_len, 128, 128, packed.attention_scale, 0.5, 0.5)
+    out, lse = risa.int8_attention_from_prequantized(packed, sparse_pattern=pattern, return_lse=True)
+    checked = 3
+    rows = checked * query_blocks
+    prepared = oracle_prequantize(q[:, :checked], k, v, return_lse=True)
+    expected, expected_lse, _ = oracle_pipeline.attend(prepared, pattern=(offsets[: rows + 1], indices[: offsets[rows]]),
+                                                       return_lse=True)
+    assert relative_l2(to_numpy(out[:, :checked]), expected) < 1e-3
+    assert relative_l2(to_numpy(lse[:, :checked]), expected_lse) < 1e-3
