@@ -47,7 +47,11 @@ def v_source_offset(wave, i, lane, padded):
 
 
 def interpret(program, operands, wave, padded, memory):
-    """Runs the scalar side; returns (events, barriers).  Events: (tile, kind, payload)."""
+    """Runs the scalar side and the wait counters.  Returns (events, barriers); an event is
+    (phase, kind, payload) with phase = barriers passed so far.  Asserts on the way that no
+    instruction touches a register an LDS read or a scalar load is still to fill (LDS reads
+    complete in order, scalar loads in any order, so with a scalar load in flight only a wait
+    for zero proves anything)."""
     lines = [re.match(r'"(.*)\\n\\t"', line).group(1).split(";")[0].strip() for line in program.splitlines()]
     lines = [line for line in lines if line]
     labels = {line[:-1]: index for index, line in enumerate(lines) if line.endswith(":")}
@@ -62,6 +66,15 @@ def interpret(program, operands, wave, padded, memory):
         254: [v_source_offset(wave, 1, l, padded) - (wave * NC + 1) * 8 * padded for l in lanes],
     }
     sreg, state = {}, {"exec": (1 << 64) - 1, "scc": 0}
+    lds_pending = []      # [(first register, registers)] oldest first
+    scalar_pending = []   # [set of scalar registers]
+    fragment = {}         # first register of a 4-register group -> lane addresses of the read that filled it
+
+    def busy_vector():
+        return {r for _, registers in lds_pending for r in registers}
+
+    def busy_scalar():
+        return {r for registers in scalar_pending for r in registers}
 
     def value(token):
         token = token.strip()
@@ -72,9 +85,11 @@ def interpret(program, operands, wave, padded, memory):
         pair = re.fullmatch(r"s\[(\d+):(\d+)\]", token)
         if pair:
             low = int(pair.group(1))
+            assert not {low, low + 1} & busy_scalar(), token
             return sreg.get(low, 0) | (sreg.get(low + 1, 0) << 32)
         single = re.fullmatch(r"s(\d+)", token)
         if single:
+            assert int(single.group(1)) not in busy_scalar(), token
             return sreg.get(int(single.group(1)), 0)
         if token == "m0":
             return sreg.get("m0", 0)
@@ -94,7 +109,13 @@ def interpret(program, operands, wave, padded, memory):
             else:
                 sreg[int(token[1:])] = result & 0xFFFFFFFF
 
-    events, barriers, tile, pc, steps = [], 0, -1, 0, 0
+    def vector_registers(text):
+        registers = {int(number) for number in re.findall(r"\bv(\d+)\b", text)}
+        for low, high in re.findall(r"v\[(\d+):(\d+)\]", text):
+            registers |= set(range(int(low), int(high) + 1))
+        return registers
+
+    events, barriers, pc, steps = [], 0, 0, 0
     while pc < len(lines):
         steps += 1
         assert steps < 5_000_000, "the loop does not end"
@@ -105,9 +126,24 @@ def interpret(program, operands, wave, padded, memory):
         op, _, rest = line.partition(" ")
         args = [a.strip() for a in re.split(r",(?![^\[]*\])", rest)] if rest else []
         low32 = lambda token: value(token) & 0xFFFFFFFF
+        if op.startswith(("v_", "ds_", "global_")):
+            assert not vector_registers(rest) & busy_vector(), f"register still to be filled by an LDS read: {line}"
+            for token in re.findall(r"\bs\d+\b|s\[\d+:\d+\]", rest):
+                value(token)  # (asserts that no scalar load is still to fill it)
         if op == "s_barrier":
+            assert not lds_pending and not scalar_pending
             barriers += 1
-            tile += 1
+        elif op == "s_waitcnt":
+            counter = re.search(r"lgkmcnt\((\d+)\)", rest)
+            if counter:
+                allowed = int(counter.group(1))
+                if allowed == 0:
+                    lds_pending, scalar_pending = [], []
+                else:
+                    assert not scalar_pending, f"a partial wait with a scalar load in flight: {line}"
+                    lds_pending = lds_pending[len(lds_pending) - allowed:] if allowed < len(lds_pending) else lds_pending
+            if "vmcnt" in rest:
+                assert "vmcnt(0)" in rest
         elif op in ("s_mov_b32", "s_mov_b64"):
             assign(args[0], value(args[1]))
         elif op == "v_readfirstlane_b32":
@@ -132,49 +168,97 @@ def interpret(program, operands, wave, padded, memory):
             state["scc"] = int(low32(args[0]) == low32(args[1]))
         elif op == "s_cmp_lg_u32":
             state["scc"] = int(low32(args[0]) != low32(args[1]))
+        elif op == "s_cmp_lt_u32":
+            state["scc"] = int(low32(args[0]) < low32(args[1]))
+        elif op == "s_cselect_b32":
+            assign(args[0], value(args[1]) if state["scc"] else value(args[2]))
         elif op == "s_cbranch_scc1":
             pc = labels[args[0]] if state["scc"] else pc
         elif op == "s_cbranch_vccz":
             pass  # the rescale block touches no memory; the GPU tests take both sides
         elif op in ("s_load_dword", "s_load_dwordx2", "s_load_dwordx4"):
             address = value(args[1]) + int(args[2], 0)
-            events.append((tile, "sload", address))
+            events.append((barriers, "sload", address))
             count = {"s_load_dword": 1, "s_load_dwordx2": 2, "s_load_dwordx4": 4}[op]
             first = int(re.match(r"s\[?(\d+)", args[0]).group(1))
             for word in range(count):
                 sreg[first + word] = memory.get(address + 4 * word, 0)
+            scalar_pending.append(set(range(first, first + count)))
         elif op == "global_load_lds_dwordx4":
             assert "offset" not in args[1], "an instruction offset also moves the LDS address"
             base = value(args[1])
             register = int(args[0][1:])
             offsets = vreg[register] if register in vreg else vreg["lane16"]
             active = [l for l in lanes if (state["exec"] >> l) & 1]
-            events.append((tile, "copy", [(sreg["m0"] + 16 * l, base + offsets[l]) for l in active]))
+            events.append((barriers, "copy", [(sreg["m0"] + 16 * l, base + offsets[l]) for l in active]))
         elif op == "ds_read_b128":
             match = re.fullmatch(r"v(\d+) offset:(\d+)", args[1])
             destination = int(re.match(r"v\[(\d+):", args[0]).group(1))
-            events.append((tile, "read", (destination, [vreg[int(match.group(1))][l] + int(match.group(2)) for l in lanes])))
+            addresses = [vreg[int(match.group(1))][l] + int(match.group(2)) for l in lanes]
+            events.append((barriers, "read", (destination, addresses)))
+            lds_pending.append((destination, set(range(destination, destination + 4))))
+            fragment[destination] = tuple(addresses)
+        elif op == "v_mfma_i32_32x32x32_i8":
+            blocks = [re.match(r"v\[(\d+):", arg) for arg in args]
+            start = int(blocks[3].group(1)) if blocks[3] else None
+            events.append((barriers, "mfma", (int(blocks[0].group(1)), fragment[int(blocks[1].group(1))],
+                                                int(blocks[2].group(1)), start)))
         elif op == "v_mbcnt_lo_u32_b32":
             vreg["lane16"] = [16 * l for l in lanes]  # (followed by the shift by four)
-        elif op.startswith("v_") or op in ("s_nop", "s_waitcnt", "s_setprio"):
+        elif op.startswith("v_"):
+            for register in vector_registers(args[0]):
+                fragment.pop(register, None)  # (a vector instruction rewrote it: no longer a fragment)
+        elif op in ("s_nop", "s_setprio"):
             pass
         else:
             raise AssertionError(f"instruction the interpreter does not know: {line}")
     return events, barriers
 
 
+def lane_halves():
+    return [l // 32 for l in range(64)], [l % 32 for l in range(64)]
+
+
+def k_fragment(stage, rb, kk):
+    half, l32 = lane_halves()
+    return tuple(stage * STAGE + swizzled(rb * 32 + l32[l], kk * 2 + half[l]) for l in range(64))
+
+
+def v_fragment(stage, cb, rb):
+    half, l32 = lane_halves()
+    return tuple(stage * STAGE + 16384 + swizzled(cb * 32 + l32[l], rb * 2 + half[l]) for l in range(64))
+
+
+S_BLOCK, ACC_BLOCK, Q_BLOCK, VF_BLOCK, PK_BLOCK = [0, 16, 32, 48], [64, 80, 96, 112], [192, 196, 200, 204], [208, 212, 216, 220], [224, 228]
+
+
 def expected_reads(stage):
-    half, l32 = [l // 32 for l in range(64)], [l % 32 for l in range(64)]
+    """LDS reads of the tile in `stage`: K fragments into the accumulator registers, the
+    accumulator seeds of channel block kk over the fragments of k-step kk, V fragments."""
+    half, _ = lane_halves()
     reads = []
     for kk in range(4):
-        for rb in range(4):  # K fragments into the accumulator registers
-            reads.append((64 + kk * 16 + rb * 4, [stage * STAGE + swizzled(rb * 32 + l32[l], kk * 2 + half[l]) for l in range(64)]))
-        for b4 in range(4):  # then the accumulator seeds of channel block kk
-            reads.append((64 + kk * 16 + b4 * 4, [stage * STAGE + 32768 + (kk * 32 + b4 * 8 + half[l] * 4) * 4 for l in range(64)]))
+        for rb in range(4):
+            reads.append((ACC_BLOCK[kk] + rb * 4, list(k_fragment(stage, rb, kk))))
+        for b4 in range(4):
+            reads.append((ACC_BLOCK[kk] + b4 * 4, [stage * STAGE + 32768 + (kk * 32 + b4 * 8 + half[l] * 4) * 4 for l in range(64)]))
     for rb in range(4):
         for cb in range(4):
-            reads.append((208 + cb * 4, [stage * STAGE + 16384 + swizzled(cb * 32 + l32[l], rb * 2 + half[l]) for l in range(64)]))
+            reads.append((VF_BLOCK[cb], list(v_fragment(stage, cb, rb))))
     return reads
+
+
+def expected_matrix_instructions(stage):
+    """Per destination block, in program order: (destination, lane addresses of the A fragment,
+    first B register, first C register).  Score products start from the seed block that borrows
+    the V fragment registers; value products accumulate over the seeds read from LDS."""
+    chains = {}
+    for rb in range(4):
+        chains[S_BLOCK[rb]] = [(S_BLOCK[rb], k_fragment(stage, rb, kk), Q_BLOCK[kk], VF_BLOCK[0] if kk == 0 else S_BLOCK[rb])
+                               for kk in range(4)]
+    for cb in range(4):
+        chains[ACC_BLOCK[cb]] = [(ACC_BLOCK[cb], v_fragment(stage, cb, rb), PK_BLOCK[rb & 1], ACC_BLOCK[cb]) for rb in range(4)]
+    return chains
 
 
 @pytest.mark.parametrize("sparse", [False, True])
@@ -193,16 +277,14 @@ def test_generated_text_is_committed(sparse):
 @pytest.mark.parametrize("sparse", [False, True])
 @pytest.mark.parametrize("tiles,padded", [(2, 256), (3, 384), (6, 1024), (9, 40064), (64, 8192)])
 def test_memory_accesses_match_the_compiled_loop(sparse, tiles, padded):
-    """`tiles` listed tiles: the loop walks all but the last and copies in every one of them the next."""
+    """`tiles` listed tiles: the loop walks all but the last and copies in every one of them the
+    next; every matrix instruction multiplies the fragment the compiled loop multiplies there."""
     gen = generator()
     args = gen.parse([])
     args.sparse = sparse
     program, _ = gen.render(args)
     key_tiles = padded // CTA_K
-    if sparse:
-        listed = sorted(random.Random(tiles).sample(range(key_tiles), tiles))
-    else:
-        listed = list(range(tiles))
+    listed = sorted(random.Random(tiles).sample(range(key_tiles), tiles)) if sparse else list(range(tiles))
     memory = {LIST0 + 4 * i: tile for i, tile in enumerate(listed)}
     for wave in range(4):
         operands = {"%[kptr]": K0 if sparse else K0 + CTA_K * D, "%[vptr]": V0 if sparse else V0 + CTA_K,
@@ -210,12 +292,14 @@ def test_memory_accesses_match_the_compiled_loop(sparse, tiles, padded):
                     "%[wave]": wave, "%[qs2]": 0x3F800000, "%[padded]": padded, "%[list]": LIST0}
         events, barriers = interpret(program, operands, wave, padded, memory)
         assert barriers == tiles - 1
-        before = [event[2] for event in events if event[0] == -1 and event[1] == "sload"]
-        assert before == ([LIST0, KS0 + 16 * listed[0]] if sparse else [KS0])
+
+        def of(phase, kind):
+            return [event[2] for event in events if event[0] == phase and event[1] == kind]
+
+        assert of(0, "sload") == ([LIST0, KS0 + 16 * listed[0]] if sparse else [KS0])
+        assert not of(0, "copy") and not of(0, "read") and not of(0, "mfma")
         for index in range(tiles - 1):
-            stage, other, following = index & 1, (index & 1) ^ 1, listed[index + 1]
-            mine = [event for event in events if event[0] == index]
-            copies = sorted(pair for event in mine if event[1] == "copy" for pair in event[2])
+            phase, stage, other, following = index + 1, index & 1, (index & 1) ^ 1, listed[index + 1]
             wanted = []
             for i in range(NC):
                 for lane in range(64):
@@ -225,13 +309,16 @@ def test_memory_accesses_match_the_compiled_loop(sparse, tiles, padded):
                                    V0 + following * CTA_K + v_source_offset(wave, i, lane, padded)))
             if wave == 0:  # accumulator seeds: 512 bytes by the first 32 lanes of wavefront 0
                 wanted += [(other * STAGE + 32768 + 16 * lane, SUM0 + following * D * 4 + 16 * lane) for lane in range(32)]
-            assert copies == sorted(wanted), (wave, index)
-            assert sorted(event[2] for event in mine if event[1] == "read") == sorted(expected_reads(stage)), (wave, index)
-            loads = [event[2] for event in mine if event[1] == "sload"]
+            assert sorted(pair for copy in of(phase, "copy") for pair in copy) == sorted(wanted), (wave, index)
+            assert sorted(of(phase, "read")) == sorted(expected_reads(stage)), (wave, index)
+            issued = of(phase, "mfma")
+            assert len(issued) == 32
+            for destination, chain in expected_matrix_instructions(stage).items():
+                assert [m for m in issued if m[0] == destination] == chain, (wave, index, destination)
             if sparse:
-                assert loads == [KS0 + 16 * following, LIST0 + 4 * min(index + 2, tiles - 1)], (wave, index)
+                assert of(phase, "sload") == [KS0 + 16 * following, LIST0 + 4 * min(index + 2, tiles - 1)], (wave, index)
             else:
-                assert loads == [KS0 + 16 * following], (wave, index)
+                assert of(phase, "sload") == [KS0 + 16 * following], (wave, index)
 
 
 def test_wait_states_after_matrix_instructions():
