@@ -8,6 +8,8 @@
 
 #include "attention_dispatch.hpp"
 
+#include <cstdlib>
+
 namespace risa {
 
 template <> int launch_attention_variant<64>(const KernelParams&, int, bool, bool, bool, int, hipStream_t);
@@ -179,6 +181,11 @@ int launch_attention(const AttentionArgs& a, hipStream_t stream) {
   p.workspace = a.block_mass;
   p.lse = a.lse;
   p.causal = a.is_causal ? 1 : 0;
+  // Diagnostic switch, read at every launch: RISA_COMPILED_LOOP=1 sends the raw-score kernels of
+  // head dim 128 through the tile loop the compiler schedules instead of the hand-scheduled one
+  // (same results bit for bit; the tests compare the two).
+  const char* compiled_loop = std::getenv("RISA_COMPILED_LOOP");
+  p.compiled_loop = compiled_loop != nullptr && compiled_loop[0] != '\0' && compiled_loop[0] != '0';
 
   const bool use_key_tiles = a.key_mask_tiles != nullptr && a.mask != nullptr &&
                              a.mask_stride_q == 0 && !sparse && !capture && !a.is_causal;

@@ -81,6 +81,7 @@ struct KernelParams {
   float* workspace;  // capture
   float* lse;
   int causal;
+  int compiled_loop;  // non-zero: every tile through the loop the compiler schedules (see RISA_COMPILED_LOOP)
 };
 
 // Byte offset of 16-byte chunk `chunk` of row `row` in a swizzled LDS tile.
@@ -963,16 +964,17 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : D == 64 && MASK_MODE == kMaskL
   // --- main loop: one barrier per tile -----------------------------------------
   // At the barrier of iteration t every wave has finished tile t-1 (so stage
   // (t+1)&1 may be overwritten) and has seen its own share of tile t land.
-  // Raw-score launches with head dim 128 and 128-key tiles (dense, or over a sparse pattern's
-  // tile lists) walk every tile but the last in a hand-scheduled loop, written by
-  // gen_dense_loop.py into dense_loop_d128.inc / sparse_loop_d128.inc: same arithmetic in the
-  // same order, bit-identical results.  The loop owns the whole register file, so its operands
-  // are pinned to the registers the generator chose; the last listed tile (the one that may be
-  // partial) and the epilogue stay below.
-  constexpr bool ASM_LOOP = FAST && D == 128 && CTA_K == 128 && !CAPTURE;
+  // Raw-score launches with head dim 128 and 128-key tiles (dense, over a sparse pattern's tile
+  // lists, or capturing the statistics of pattern construction) walk every tile but the last in
+  // a hand-scheduled loop, written by gen_dense_loop.py into dense_, sparse_ and
+  // capture_loop_d128.inc: same arithmetic in the same order as the loop below, bit-identical
+  // results.  The loop owns the whole register file, so its operands are pinned to the registers
+  // the generator chose; the last listed tile (the one that may be partial) and the epilogue
+  // stay below.
+  constexpr bool ASM_LOOP = FAST && D == 128 && CTA_K == 128;
   int first_tile = 0;
   if constexpr (ASM_LOOP) {
-    if (n_it > 1) {
+    if (n_it > 1 && !p.compiled_loop) {
       typedef __attribute__((address_space(3))) unsigned char* LdsBytes;
       const uint32_t lds_address = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((LdsBytes)lds));
       issue_tile(tile_at(0), 0);
@@ -1006,6 +1008,25 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : D == 64 && MASK_MODE == kMaskL
               [count] "s"(count), [wave] "s"(wave), [qs2] "s"(qs2), [padded] "s"(p.padded), [list] "s"(list)
             :
 #include "sparse_loop_d128_clobbers.inc"
+        );
+      } else if constexpr (CAPTURE) {
+        // statistics of tile 0 for this wavefront's first query; lanes 0..31 hold the queries that store
+        const uint64_t stats_rows = reinterpret_cast<uint64_t>(
+            stats + (bhq * static_cast<uint64_t>(p.n_kb - 1) * p.q_len + (bx * kQueryBlock + wave * 32)) * 2);
+        const uint32_t tile_bytes = static_cast<uint32_t>(p.q_len) * 8u;
+        const uint64_t storing = __builtin_amdgcn_ballot_w64(half == 0 && query_ok);
+        asm volatile(
+#include "capture_loop_d128.inc"
+            : "+{v[128:143]}"(out0), "+{v[144:159]}"(out1), "+{v[160:175]}"(out2), "+{v[176:191]}"(out3),
+              "+{v241}"(m_run), "+{v242}"(d_part)
+            : "{v[192:195]}"(qreg[0]), "{v[196:199]}"(qreg[1]), "{v[200:203]}"(qreg[2]), "{v[204:207]}"(qreg[3]),
+              "{v244}"(q_scale), "{v246}"(a0), "{v247}"(a1), "{v248}"(a2), "{v249}"(a3), "{v250}"(seed_address),
+              "{v251}"(kc0), "{v252}"(kc1), "{v253}"(vc0), "{v254}"(vc1),
+              [kptr] "s"(k_source), [vptr] "s"(v_source), [sumptr] "s"(sum_source), [ksptr] "s"(ks_source),
+              [count] "s"(count), [wave] "s"(wave), [qs2] "s"(qs2), [padded] "s"(p.padded),
+              [stats] "s"(stats_rows), [qlen8] "s"(tile_bytes), [capexec] "s"(storing)
+            :
+#include "capture_loop_d128_clobbers.inc"
         );
       } else {
         asm volatile(

@@ -3,7 +3,7 @@
 128-key tiles (every listed tile but the last) as gfx950 assembly: one `asm volatile` statement
 whose operands are pinned to the registers chosen here.
 
-    python3 gen_dense_loop.py            # writes dense_loop_d128*.inc and sparse_loop_d128*.inc beside this file
+    python3 gen_dense_loop.py            # writes dense_, sparse_ and capture_loop_d128*.inc beside this file
 
 Why assembly.  The loop owns the whole register file (256 vector registers at two wavefronts
 per SIMD) and every phase reuses what the previous one has just left: the sixteen K fragments of
@@ -70,6 +70,8 @@ S_LIST = 68                    # pair: sparse: the query block's tile list
 S_TNEXT, S_TAFTER, S_INDEX, S_LAST = 70, 71, 72, 73  # sparse: next tile, the one after it, its list index, last index
 S_KWAVE, S_VWAVE = 74, 76      # pairs: sparse: this wave's share of the K and V sources
 LAST_SGPR = 77
+S_STATS, S_QLEN8, S_CAPEXEC = 78, 80, 82  # capture: pair: this wavefront's statistics rows of the tile; bytes per tile; pair: lanes that store
+LAST_SGPR_CAPTURE = 83
 
 
 class Emitter:
@@ -350,6 +352,24 @@ def tile_body(e, stage, args, label):
     for cb in range(4):
         e.wait_lds(VF[cb])
         e.mfma(ACC[cb], VF[cb], PK[1], ACC[cb])
+    if args.capture:
+        # per-tile statistics of pattern construction: the row's sum of probability bytes (both halves
+        # of the wavefront) and the tile maximum, eight bytes per query, tile-major
+        e.valu(f"v_mov_b32_e32 v{T[2]}, v{V_ROWSUM}", [T[2]])
+        e.valu(f"v_mov_b32_e32 v{T[1]}, v{V_ROWSUM}", [T[1]])
+        e.nop(2)
+        e.valu(f"v_permlane32_swap_b32_e32 v{T[2]}, v{T[1]}", [T[2], T[1]])
+        e.nop(2)
+        e.valu(f"v_add_u32_e32 v{T[2]}, v{T[2]}, v{T[1]}", [T[2]])
+        e.valu(f"v_mov_b32_e32 v{T[3]}, v{V_MX0}", [T[3]])
+        e.valu(f"v_mbcnt_lo_u32_b32 v{T[0]}, -1, 0", [T[0]])
+        e.valu(f"v_lshlrev_b32_e32 v{T[0]}, 3, v{T[0]}", [T[0]])  # lane * 8 (the lanes that store are 0..31)
+        e.ins(f"s_mov_b64 s[{S_SAVEEXEC}:{S_SAVEEXEC + 1}], exec")
+        e.ins(f"s_mov_b64 exec, s[{S_CAPEXEC}:{S_CAPEXEC + 1}]")
+        e.ins(f"global_store_dwordx2 v{T[0]}, v[{T[2]}:{T[3]}], s[{S_STATS}:{S_STATS + 1}]")
+        e.ins(f"s_mov_b64 exec, s[{S_SAVEEXEC}:{S_SAVEEXEC + 1}]")
+        e.ins(f"s_add_u32 s{S_STATS}, s{S_STATS}, s{S_QLEN8}")
+        e.ins(f"s_addc_u32 s{S_STATS + 1}, s{S_STATS + 1}, 0")
     e.valu(f"v_cvt_f32_u32_e32 v{T[0]}, v{V_ROWSUM}", [T[0]])
     e.valu(f"v_fmac_f32_e32 v{V_DPART}, v{T[0]}, v{V_TSCALE}", [V_DPART])
     # ---- K scales (and list entry) of the next tile: waited for at the next barrier ------------------
@@ -392,6 +412,10 @@ def generate(args):
     e.ins(f"s_mov_b32 s{S_VSTEP + 1}, 0")
     if args.sparse:
         e.ins(f"s_mov_b64 s[{S_LIST}:{S_LIST + 1}], %[list]")
+    if args.capture:
+        e.ins(f"s_mov_b64 s[{S_STATS}:{S_STATS + 1}], %[stats]")
+        e.ins(f"s_mov_b32 s{S_QLEN8}, %[qlen8]")
+        e.ins(f"s_mov_b64 s[{S_CAPEXEC}:{S_CAPEXEC + 1}], %[capexec]")
     # LDS base: lane 0 of the seed address register holds base + SEED_BIAS
     e.ins(f"v_readfirstlane_b32 s{S_LDS}, v{V_SEEDADDR}")
     e.ins(f"s_sub_u32 s{S_LDS}, s{S_LDS}, {SEED_BIAS}")
@@ -439,6 +463,10 @@ def generate(args):
     return e
 
 
+# (walks a tile list, stores the statistics of pattern construction, file stem)
+PROGRAMS = ((False, False, "dense_loop_d128"), (True, False, "sparse_loop_d128"), (False, True, "capture_loop_d128"))
+
+
 def render(args):
     """(program text, clobber list) as the two include files hold them."""
     e = generate(args)
@@ -446,7 +474,7 @@ def render(args):
     operands = set(range(O[0], O[0] + 64)) | set(range(Q[0], Q[0] + 16)) | {V_MRUN, V_DPART, V_QSCALE}
     operands |= set(V_A) | {V_SEEDADDR} | set(V_KC) | set(V_VC)
     clobbered = [f"v{r}" for r in range(255) if r not in operands]
-    clobbered += [f"s{r}" for r in range(36, LAST_SGPR + 1)]
+    clobbered += [f"s{r}" for r in range(36, (LAST_SGPR_CAPTURE if args.capture else LAST_SGPR) + 1)]
     clobbered += ["vcc", "scc", "m0", "memory"]
     return program, ", ".join(f'"{name}"' for name in clobbered) + "\n"
 
@@ -459,13 +487,14 @@ def parse(argv=None):
     parser.add_argument("--prios", type=lambda text: [int(x) for x in text.split(",")], default=[0, 1, 2, 0],
                         help="wave priority in the score product, the maxima/scaling pass, the exponential rounds "
                              "and the output update (measured: 0,1,2,0 beats 0,2,1,2 by 2.5 %% and no priorities by 7 %%)")
+    parser.set_defaults(sparse=False, capture=False)
     return parser.parse_args(argv)
 
 
 def main():
     args = parse()
-    for sparse, stem in ((False, "dense_loop_d128"), (True, "sparse_loop_d128")):
-        args.sparse = sparse
+    for sparse, capture, stem in PROGRAMS:
+        args.sparse, args.capture = sparse, capture
         program, clobbers = render(args)
         (args.outdir / f"{stem}.inc").write_text(program)
         (args.outdir / f"{stem}_clobbers.inc").write_text(clobbers)

@@ -188,7 +188,7 @@ def interpret(program, operands, wave, padded, memory):
             assert "offset" not in args[1], "an instruction offset also moves the LDS address"
             base = value(args[1])
             register = int(args[0][1:])
-            offsets = vreg[register] if register in vreg else vreg["lane16"]
+            offsets = vreg[register]
             active = [l for l in lanes if (state["exec"] >> l) & 1]
             events.append((barriers, "copy", [(sreg["m0"] + 16 * l, base + offsets[l]) for l in active]))
         elif op == "ds_read_b128":
@@ -203,11 +203,20 @@ def interpret(program, operands, wave, padded, memory):
             start = int(blocks[3].group(1)) if blocks[3] else None
             events.append((barriers, "mfma", (int(blocks[0].group(1)), fragment[int(blocks[1].group(1))],
                                                 int(blocks[2].group(1)), start)))
+        elif op == "global_store_dwordx2":
+            base, offsets = value(args[2]), vreg[int(args[0][1:])]
+            active = [l for l in lanes if (state["exec"] >> l) & 1]
+            events.append((barriers, "store", (int(re.match(r"v\[(\d+):", args[1]).group(1)), [base + offsets[l] for l in active])))
         elif op == "v_mbcnt_lo_u32_b32":
-            vreg["lane16"] = [16 * l for l in lanes]  # (followed by the shift by four)
+            assert args[1:] == ["-1", "0"]
+            vreg[int(args[0][1:])] = [min(l, 32) for l in lanes]  # lanes below this one among the first 32
+        elif op == "v_lshlrev_b32_e32" and int(args[2][1:]) in vreg:
+            vreg[int(args[0][1:])] = [x << int(args[1]) for x in vreg[int(args[2][1:])]]
         elif op.startswith("v_"):
             for register in vector_registers(args[0]):
                 fragment.pop(register, None)  # (a vector instruction rewrote it: no longer a fragment)
+                if register < 246:
+                    vreg.pop(register, None)  # (nor a lane index)
         elif op in ("s_nop", "s_setprio"):
             pass
         else:
@@ -261,27 +270,36 @@ def expected_matrix_instructions(stage):
     return chains
 
 
-@pytest.mark.parametrize("sparse", [False, True])
-def test_generated_text_is_committed(sparse):
+def test_generated_text_is_committed():
     gen = generator()
+    assert {stem for _, _, stem in gen.PROGRAMS} == {path.name[:-4] for path in CSRC.glob("*_loop_d128.inc")}
+    for sparse, capture, stem in gen.PROGRAMS:
+        check_committed(gen, sparse, capture, stem)
+
+
+def check_committed(gen, sparse, capture, stem):
     args = gen.parse([])
-    args.sparse = sparse
+    args.sparse, args.capture = sparse, capture
     program, clobbers = gen.render(args)
-    stem = "sparse_loop_d128" if sparse else "dense_loop_d128"
     assert (CSRC / f"{stem}.inc").read_text() == program
     assert (CSRC / f"{stem}_clobbers.inc").read_text() == clobbers
     assert '"v255"' not in clobbers and '"v254"' not in clobbers  # the compiler's own register; an operand
     assert "s_store" not in program and "s_dcache" not in program and "s_atomic" not in program
 
 
-@pytest.mark.parametrize("sparse", [False, True])
+STATS0, TILE_BYTES, STORING = 0x60000000, 40064 * 8, (1 << 20) - 1  # capture: rows of tile 0, bytes per tile, lanes that store
+
+
+@pytest.mark.parametrize("program_kind", ["dense", "sparse", "capture"])
 @pytest.mark.parametrize("tiles,padded", [(2, 256), (3, 384), (6, 1024), (9, 40064), (64, 8192)])
-def test_memory_accesses_match_the_compiled_loop(sparse, tiles, padded):
+def test_memory_accesses_match_the_compiled_loop(program_kind, tiles, padded):
     """`tiles` listed tiles: the loop walks all but the last and copies in every one of them the
-    next; every matrix instruction multiplies the fragment the compiled loop multiplies there."""
+    next; every matrix instruction multiplies the fragment the compiled loop multiplies there; the
+    capturing program stores eight bytes per storing lane and tile, tile-major."""
     gen = generator()
     args = gen.parse([])
-    args.sparse = sparse
+    sparse, capture = program_kind == "sparse", program_kind == "capture"
+    args.sparse, args.capture = sparse, capture
     program, _ = gen.render(args)
     key_tiles = padded // CTA_K
     listed = sorted(random.Random(tiles).sample(range(key_tiles), tiles)) if sparse else list(range(tiles))
@@ -289,7 +307,8 @@ def test_memory_accesses_match_the_compiled_loop(sparse, tiles, padded):
     for wave in range(4):
         operands = {"%[kptr]": K0 if sparse else K0 + CTA_K * D, "%[vptr]": V0 if sparse else V0 + CTA_K,
                     "%[sumptr]": SUM0 if sparse else SUM0 + D * 4, "%[ksptr]": KS0, "%[count]": tiles - 1,
-                    "%[wave]": wave, "%[qs2]": 0x3F800000, "%[padded]": padded, "%[list]": LIST0}
+                    "%[wave]": wave, "%[qs2]": 0x3F800000, "%[padded]": padded, "%[list]": LIST0,
+                    "%[stats]": STATS0, "%[qlen8]": TILE_BYTES, "%[capexec]": STORING}
         events, barriers = interpret(program, operands, wave, padded, memory)
         assert barriers == tiles - 1
 
@@ -319,6 +338,9 @@ def test_memory_accesses_match_the_compiled_loop(sparse, tiles, padded):
                 assert of(phase, "sload") == [KS0 + 16 * following, LIST0 + 4 * min(index + 2, tiles - 1)], (wave, index)
             else:
                 assert of(phase, "sload") == [KS0 + 16 * following], (wave, index)
+            # (row sum and tile maximum in two consecutive registers, by the storing lanes only)
+            stores = [(234, [STATS0 + index * TILE_BYTES + 8 * lane for lane in range(20)])] if capture else []
+            assert of(phase, "store") == stores, (wave, index)
 
 
 def test_wait_states_after_matrix_instructions():
@@ -326,9 +348,9 @@ def test_wait_states_after_matrix_instructions():
     (the distance gfx950 asks for after an 8-pass matrix instruction), counted as the assembler
     counts them: one per instruction, s_nop n counting n + 1."""
     gen = generator()
-    for sparse in (False, True):
+    for sparse, capture, _ in gen.PROGRAMS:
         args = gen.parse([])
-        args.sparse = sparse
+        args.sparse, args.capture = sparse, capture
         lines = [re.match(r'"(.*)\\n\\t"', line).group(1).strip() for line in gen.render(args)[0].splitlines()]
         clock, written = 0, {}
         for line in lines:

@@ -1,8 +1,12 @@
-"""The hand-scheduled tile loop of the raw-score kernels (head dim 128, 128-key tiles, more
-workgroups than compute units) against the loop the compiler schedules: the capturing launch of
-pattern construction keeps the compiled loop and does the same arithmetic in the same order, so
-the two outputs are equal bit for bit; tile lists are compared with the dense launch where they
-name every tile, and with the oracle walking the same lists otherwise."""
+"""The hand-scheduled tile loops of the raw-score kernels (head dim 128, 128-key tiles, more
+workgroups than compute units: dense, over tile lists, capturing) against the loop the compiler
+schedules, which RISA_COMPILED_LOOP=1 selects at every launch: same arithmetic in the same order,
+so outputs, log-sum-exp rows and the constructed pattern are equal bit for bit.  Tile lists are
+also compared with the dense launch where they name every tile, and with the oracle walking the
+same lists otherwise."""
+
+import os
+from contextlib import contextmanager
 
 import numpy as np
 import pytest
@@ -14,9 +18,19 @@ from tests.helpers import oracle_prequantize, relative_l2, seeded, to_numpy
 pytestmark = pytest.mark.gpu
 
 
+@contextmanager
+def compiled_loop():
+    """Launches inside go through the compiler-scheduled tile loop."""
+    os.environ["RISA_COMPILED_LOOP"] = "1"
+    try:
+        yield
+    finally:
+        del os.environ["RISA_COMPILED_LOOP"]
+
+
 @pytest.mark.parametrize("length", [2048, 2049, 2304, 4096, 4190])
 @pytest.mark.parametrize("mode", ["absmax", "midpoint_affine"])
-def test_dense_loop_equals_the_capturing_launch_bit_for_bit(risa, length, mode):
+def test_dense_and_capturing_loops_equal_the_compiled_loop_bit_for_bit(risa, length, mode):
     """Odd and even tile counts (the loop is unrolled by two and leaves from either half), a last
     tile of one key, of half a tile, a whole one."""
     heads = 20  # x 17..33 query blocks: above the small-launch limit of a 256-CU part
@@ -25,7 +39,15 @@ def test_dense_loop_equals_the_capturing_launch_bit_for_bit(risa, length, mode):
     v = seeded((1, 4, length, 128), torch.bfloat16, length + 2, offset=0.25)
     dense, dense_lse = risa.int8_attention(q, k, v, v_quantization=mode, return_lse=True)
     captured, pattern = risa.construct_sparse_int8_attention(q, k, v, theta=0.95, v_quantization=mode)
-    assert torch.equal(dense, captured)
+    with compiled_loop():
+        compiled, compiled_lse = risa.int8_attention(q, k, v, v_quantization=mode, return_lse=True)
+        compiled_captured, compiled_pattern = risa.construct_sparse_int8_attention(q, k, v, theta=0.95, v_quantization=mode)
+    assert torch.equal(dense, compiled) and torch.equal(dense_lse, compiled_lse)
+    assert torch.equal(captured, compiled_captured) and torch.equal(dense, captured)
+    # the statistics the capturing loop stores decide the pattern: same rows, same tiles, same mass
+    assert torch.equal(pattern.row_offsets, compiled_pattern.row_offsets)
+    assert torch.equal(pattern.block_indices, compiled_pattern.block_indices)
+    assert pattern.measured_retained_mass == compiled_pattern.measured_retained_mass
     checked = 2
     prepared = oracle_prequantize(q[:, :checked], k[:, :1], v[:, :1], v_quantization=mode, return_lse=True)
     expected, expected_lse, _ = oracle_pipeline.attend(prepared, return_lse=True)
@@ -73,6 +95,9 @@ def test_listed_loop_with_random_lists_matches_oracle(risa, seed):
     pattern = RetainedMassPattern(torch.from_numpy(offsets).cuda(), torch.from_numpy(indices).cuda(), 1, heads, q_len,
                                   k_len, 128, 128, packed.attention_scale, 0.5, 0.5)
     out, lse = risa.int8_attention_from_prequantized(packed, sparse_pattern=pattern, return_lse=True)
+    with compiled_loop():
+        compiled, compiled_lse = risa.int8_attention_from_prequantized(packed, sparse_pattern=pattern, return_lse=True)
+    assert torch.equal(out, compiled) and torch.equal(lse, compiled_lse)
     checked = 3
     rows = checked * query_blocks
     prepared = oracle_prequantize(q[:, :checked], k, v, return_lse=True)
