@@ -23,7 +23,8 @@ benchmarks/plot_scaling.py).  ``--workload mask_tiles`` is the broadcast-mask co
 reference benchmarks/masks.py (interleaved empty key tiles, optionally against a second build of
 the library given with ``--baseline-library``); ``--workload profile_ranges`` wraps warmed calls in
 named profiler ranges for ``rocprofv3 --marker-trace`` (the role of reference
-benchmarks/profile_operators.py).
+benchmarks/profile_operators.py); ``--workload clock`` launches the dense kernel on random and on
+all-zero operands (same cycle count, different sustained clock: for a ``--pmc GRBM_GUI_ACTIVE`` run).
 """
 
 from __future__ import annotations
@@ -41,10 +42,10 @@ sys.path.insert(0, str(ROOT))
 
 INT8_MFMA_PEAK_TOPS = 5000.0  # MI355X dense INT8, published
 # HBM/Infinity-Cache bytes of one launch of the dense attention kernel at the headline
-# shape, from rocprofv3 FETCH_SIZE (299556 KiB raw x 2.0 calibration) + WRITE_SIZE
-# (131072 KiB x 1.0); the commands and the copy calibration are in
+# shape, from rocprofv3 FETCH_SIZE (323100 KiB raw x 2.0 calibration) + WRITE_SIZE
+# (212990 KiB x 1.0); the commands and the copy calibration are in
 # profiles/attention_dense_32k_counters.md.
-ATTENTION_KERNEL_TRAFFIC_BYTES_32K = int((299556.3 * 2.0 + 131072.0) * 1024)
+ATTENTION_KERNEL_TRAFFIC_BYTES_32K = int((323100.0 * 2.0 + 212990.0) * 1024)
 SHAPE = dict(batch=1, q_heads=16, kv_heads=4, head_dim=128)
 SEEDS = (0, 1, 2)
 
@@ -729,6 +730,41 @@ def plot_scaling(series, path, title):
     plt.close(figure)
 
 
+def kernel_time(torch, risa, packed, calls, warmup=2):
+    """Milliseconds per launch of the attention kernel on prepared operands (events on the launch stream)."""
+    stream = torch.cuda.current_stream()
+    for _ in range(warmup):
+        risa.int8_attention_from_prequantized(packed)
+    begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    begin.record(stream)
+    for _ in range(calls):
+        risa.int8_attention_from_prequantized(packed)
+    end.record(stream)
+    end.synchronize()
+    return begin.elapsed_time(end) / calls
+
+
+def workload_clock(torch, risa, args, device):
+    """The dense kernel on random and on all-zero operands, `--calls` launches each, twice over.  The
+    instruction stream is the same (one data-dependent branch aside, taken in the first tiles of
+    random data only), and so is the count of GPU clock cycles per launch (run under
+    `rocprofv3 --pmc GRBM_GUI_ACTIVE --kernel-trace`); the time differs with the clock the part
+    sustains while its matrix units switch real operands."""
+    length = args.length or 32768
+    q, k, v = make_inputs(torch, length, 0, device)
+    operands = {
+        "random": risa.prequantize_int8_attention(q, k, v, v_quantization=args.mode),
+        "zeros": risa.prequantize_int8_attention(torch.zeros_like(q), torch.zeros_like(k), torch.zeros_like(v),
+                                                 v_quantization=args.mode),
+    }
+    rows = []
+    for repeat in range(2):
+        for name, packed in operands.items():
+            rows.append({"operands": name, "repeat": repeat, "N": length, "calls": args.calls,
+                         "kernel_ms": round(kernel_time(torch, risa, packed, args.calls, warmup=10), 4)})
+    return rows
+
+
 def cpu_baseline(length=1024, calls=15):
     """Oracle (numpy port of the quantised pipeline) on the host cores: the reference's own
     CPU-sized configuration (same heads and head dim as the headline, N=1024, seed 0,
@@ -861,7 +897,7 @@ def main():
     parser.add_argument("--no-accuracy", action="store_true")
     parser.add_argument("--workload", default="dense",
                         choices=["dense", "sweep", "masked", "sparse", "sparse_blocks", "video", "prepare", "mask_tiles",
-                                 "profile_ranges"],
+                                 "profile_ranges", "clock"],
                         help="dense = headline N=32K line (default); the others are the remaining benchmark "
                              "configurations of the reference, reported as one JSON line each")
     parser.add_argument("--samples", type=int, default=10, help="event-timed samples per method and seed (--workload)")
@@ -882,7 +918,7 @@ def main():
     parser.add_argument("--baseline-library", type=Path, default=None,
                         help="mask_tiles: a second build of the C-ABI library to compare and time against")
     parser.add_argument("--stage", choices=("dense", "quantize", "attend"), default="dense", help="profile_ranges: what a range wraps")
-    parser.add_argument("--calls", type=int, default=10, help="profile_ranges: ranges per V mode")
+    parser.add_argument("--calls", type=int, default=10, help="profile_ranges: ranges per V mode; clock: launches per operand set")
     parser.add_argument("--calibrate-copy", action="store_true",
                         help="only run a 1 GiB device copy (reference point for rocprofv3 FETCH_SIZE/WRITE_SIZE)")
     args = parser.parse_args()
@@ -924,7 +960,7 @@ def main():
         runner = {"sweep": workload_sweep, "masked": workload_masked, "sparse": workload_sparse,
                   "video": workload_video, "prepare": workload_prepare,
                   "sparse_blocks": workload_sparse_blocks, "mask_tiles": workload_mask_tiles,
-                  "profile_ranges": workload_profile_ranges}[args.workload]
+                  "profile_ranges": workload_profile_ranges, "clock": workload_clock}[args.workload]
         wall = time.perf_counter()
         rows = runner(torch, risa, args, device)
         if args.output is not None:
@@ -951,18 +987,17 @@ def main():
     torch.cuda.synchronize()
     ms_per_step = (time.perf_counter() - wall_start) * 1e3 / args.steps
 
-    # Attention kernel alone, timed with events on the launch stream.
+    # Attention kernel alone, timed with events on the launch stream; and once more on all-zero
+    # operands: the same instructions in the same number of clock cycles, at the clock the part
+    # holds when its multipliers switch no bits (see workload_clock).
     packed = risa.prequantize_int8_attention(q, k, v, v_quantization=args.mode)
     stream = torch.cuda.current_stream(device)
-    for _ in range(2):
-        risa.int8_attention_from_prequantized(packed)
+    kernel_ms = kernel_time(torch, risa, packed, args.steps)
+    zero_ms = None
+    if not args.no_side_measurements:
+        zero_ms = kernel_time(torch, risa, risa.prequantize_int8_attention(
+            torch.zeros_like(q), torch.zeros_like(k), torch.zeros_like(v), v_quantization=args.mode), args.steps)
     begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    begin.record(stream)
-    for _ in range(args.steps):
-        risa.int8_attention_from_prequantized(packed)
-    end.record(stream)
-    end.synchronize()
-    kernel_ms = begin.elapsed_time(end) / args.steps
     begin.record(stream)
     for _ in range(args.steps):
         risa.prequantize_int8_attention(q, k, v, v_quantization=args.mode)
@@ -994,7 +1029,11 @@ def main():
             # kernel's limiter on this hardware is the vector-instruction issue of the U8
             # softmax next to the matrix instructions (profiles/attention_dense_32k_counters.md).
             "bound": "mfma",
-            "limited_by": "VALU issue of the softmax + MFMA (they share the SIMD issue capacity)",
+            "limited_by": "VALU issue of the softmax next to the MFMAs (they share the SIMD issue capacity), at the "
+                          "clock the part sustains under this load: about 1.9 GHz against 2.4 GHz nominal "
+                          "(profiles/attention_dense_32k_clock.md); kernel_ms_zero_inputs is the same launch on "
+                          "all-zero operands, same cycle count at the full clock",
+            "kernel_ms_zero_inputs": zero_ms,
             "achieved": achieved_tops,
             "peak": INT8_MFMA_PEAK_TOPS,
             "unit": "TOP/s",

@@ -208,9 +208,11 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : D == 64 && MASK_MODE == kMaskL
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
 
   const int tid = threadIdx.x;
-  const int lane = tid & 63;
+  // (not const: the hand-scheduled tile loop owns every vector register, and the values below are
+  // formed again behind it rather than kept in scratch memory across it)
+  int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int l32 = lane & 31, half = lane >> 5;
+  int l32 = lane & 31, half = lane >> 5;
 
   // Workgroup order.  Without a causal mask the query blocks of one head are
   // neighbours, so co-resident workgroups walk the same K/V tiles and share them
@@ -245,8 +247,8 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : D == 64 && MASK_MODE == kMaskL
     bias_base = p.key_bias + batch * p.key_bias_stride_b + head * p.key_bias_stride_h;
   }
 
-  const int query = bx * kQueryBlock + wave * 32 + l32;
-  const bool query_ok = query < p.q_len;
+  int query = bx * kQueryBlock + wave * 32 + l32;
+  bool query_ok = query < p.q_len;
 
   // --- Q operand and scales ------------------------------------------------
   // Requested before the tile list is read: the list's first entries are needed at once and
@@ -313,7 +315,10 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : D == 64 && MASK_MODE == kMaskL
   // masked kernels have none to spare (a spilled offset would be reloaded through
   // the same counter the LDS copies complete on, serialising them) and recompute
   // them per tile from a lane id the compiler cannot see through.
-  constexpr bool KEEP_OFFSETS = FAST;
+  // (The hand-scheduled tile loop issues its own copies and owns every vector register: kernels
+  // that have it issue at most two tiles from here, and offsets kept for them would live in
+  // scratch memory across the loop.)
+  constexpr bool KEEP_OFFSETS = FAST && !(D == 128 && CTA_K == 128);
   auto k_source_offset = [&](int i, int lane_id) -> uint32_t {
     constexpr int CH = D / 16;
     const int slot = (wave * NC + i) * 64 + lane_id;
@@ -1042,6 +1047,12 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : D == 64 && MASK_MODE == kMaskL
 #include "dense_loop_d128_clobbers.inc"
         );
       }
+      lane = fresh_lane();
+      l32 = lane & 31;
+      half = lane >> 5;
+      query = bx * kQueryBlock + wave * 32 + l32;
+      query_ok = query < p.q_len;
+      if constexpr (CAPTURE) stat_row = static_cast<uint64_t>(bhq) * p.q_len + query;
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
         o_acc[0][i] = __int_as_float(out0[i]);
