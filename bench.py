@@ -42,10 +42,10 @@ sys.path.insert(0, str(ROOT))
 
 INT8_MFMA_PEAK_TOPS = 5000.0  # MI355X dense INT8, published
 # HBM/Infinity-Cache bytes of one launch of the dense attention kernel at the headline
-# shape, from rocprofv3 FETCH_SIZE (323100 KiB raw x 2.0 calibration) + WRITE_SIZE
-# (212990 KiB x 1.0); the commands and the copy calibration are in
+# shape, from rocprofv3 FETCH_SIZE (299610 KiB raw x 2.0 calibration) + WRITE_SIZE
+# (131070 KiB x 1.0); the commands and the copy calibration are in
 # profiles/attention_dense_32k_counters.md.
-ATTENTION_KERNEL_TRAFFIC_BYTES_32K = int((323100.0 * 2.0 + 212990.0) * 1024)
+ATTENTION_KERNEL_TRAFFIC_BYTES_32K = int((299610.0 * 2.0 + 131070.0) * 1024)
 SHAPE = dict(batch=1, q_heads=16, kv_heads=4, head_dim=128)
 SEEDS = (0, 1, 2)
 
