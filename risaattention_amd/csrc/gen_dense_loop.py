@@ -1,7 +1,9 @@
 #!/usr/bin/env python3
-"""Writes the hand-scheduled tile loop of the raw-score attention kernel for head dim 128 and
+"""Writes the hand-scheduled tile loops of the raw-score attention kernels for head dim 128 and
 128-key tiles (every listed tile but the last) as gfx950 assembly: one `asm volatile` statement
-whose operands are pinned to the registers chosen here.
+each, whose operands are pinned to the registers chosen here.  Three programs: the dense launch,
+the launch that walks a sparse pattern's tile lists, and the capturing launch of pattern
+construction (the dense loop plus one statistics store per tile).
 
     python3 gen_dense_loop.py            # writes dense_, sparse_ and capture_loop_d128*.inc beside this file
 
