@@ -122,3 +122,45 @@ def test_two_to_four_tiles_and_two_batches(risa, k_len):
     expected, expected_lse, _ = oracle_pipeline.attend(prepared, return_lse=True)
     assert relative_l2(to_numpy(out[1:, 21:]), expected) < 1e-3
     assert relative_l2(to_numpy(lse[1:, 21:]), expected_lse) < 1e-3
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_random_shapes_equal_the_compiled_loop(risa, seed):
+    """Random batch, head grouping, lengths, dtype and V mode (always more workgroups than a
+    256-CU part has compute units): dense, capturing and list-walking launches of the
+    hand-scheduled loops against the compiled loop, bit for bit."""
+    from risaattention_amd.types import RetainedMassPattern
+
+    rng = np.random.default_rng(1000 + seed)
+    batch = int(rng.integers(1, 3))
+    kv_heads = int(rng.integers(1, 5))
+    q_heads = kv_heads * int(rng.integers(1, 5))
+    q_len = int(rng.integers(129, 1500))
+    while batch * q_heads * -(-q_len // 128) <= 300:
+        q_heads += kv_heads
+    k_len = int(rng.integers(257, 3000))
+    dtype = (torch.bfloat16, torch.float16, torch.float32)[seed % 3]
+    mode = ("absmax", "midpoint_affine")[seed % 2]
+    q = seeded((batch, q_heads, q_len, 128), dtype, 3 * seed, scale=1.0 + seed % 3)
+    k = seeded((batch, kv_heads, k_len, 128), dtype, 3 * seed + 1, scale=1.0 + seed % 2)
+    v = seeded((batch, kv_heads, k_len, 128), dtype, 3 * seed + 2, offset=0.1 * seed)
+    packed = risa.prequantize_int8_attention(q, k, v, v_quantization=mode, return_lse=True)
+    # (the tile policy gives short key ranges 64-key tiles: those launches keep the compiled loop)
+    tiles, query_blocks = -(-k_len // packed.cta_k), -(-q_len // 128)
+    lists = [np.sort(rng.choice(tiles, size=int(rng.integers(1, tiles + 1)), replace=False))
+             for _ in range(batch * q_heads * query_blocks)]
+    offsets = np.cumsum([0] + [len(entry) for entry in lists]).astype(np.int32)
+    pattern = RetainedMassPattern(torch.from_numpy(offsets).cuda(), torch.from_numpy(np.concatenate(lists).astype(np.int32)).cuda(),
+                                  batch, q_heads, q_len, k_len, 128, packed.cta_k, packed.attention_scale, 0.5, 0.5)
+
+    def run():
+        dense = risa.int8_attention_from_prequantized(packed, return_lse=True)
+        listed = risa.int8_attention_from_prequantized(packed, sparse_pattern=pattern, return_lse=True)
+        captured, built = risa.construct_sparse_int8_attention(q, k, v, theta=0.9, v_quantization=mode)
+        return [*dense, *listed, captured, built.row_offsets, built.block_indices]
+
+    scheduled = run()
+    with compiled_loop():
+        compiled = run()
+    for index, (mine, theirs) in enumerate(zip(scheduled, compiled)):
+        assert torch.equal(mine, theirs), (index, batch, q_heads, kv_heads, q_len, k_len, dtype, mode)
