@@ -107,10 +107,11 @@ def test_listed_loop_with_random_lists_matches_oracle(risa, seed):
     assert relative_l2(to_numpy(lse[:, :checked]), expected_lse) < 1e-3
 
 
-@pytest.mark.parametrize("k_len", [129, 256, 257, 385])
-def test_two_to_four_tiles_and_two_batches(risa, k_len):
-    """The shortest walks of the hand-scheduled loop (one to three tiles in it, the last tile of
-    one key or whole), cross attention, two batches of grouped heads."""
+@pytest.mark.parametrize("k_len", [1025, 1152, 1153, 1280])
+def test_shortest_dense_walks_and_two_batches(risa, k_len):
+    """The shortest dense walks of the hand-scheduled loop (128-key tiles start above 1024 keys:
+    nine or ten tiles, the last of one key or whole), cross attention, two batches of grouped
+    heads."""
     q = seeded((2, 24, 1024, 128), torch.bfloat16, k_len, scale=2.0)
     k = seeded((2, 8, k_len, 128), torch.bfloat16, k_len + 1, scale=2.0)
     v = seeded((2, 8, k_len, 128), torch.bfloat16, k_len + 2, offset=-0.25)
@@ -118,6 +119,7 @@ def test_two_to_four_tiles_and_two_batches(risa, k_len):
     with compiled_loop():
         compiled, compiled_lse = risa.int8_attention(q, k, v, return_lse=True)
     assert torch.equal(out, compiled) and torch.equal(lse, compiled_lse)
+    assert risa.prequantize_int8_attention(q, k, v).cta_k == 128
     prepared = oracle_prequantize(q[1:, 21:], k[1:, 7:], v[1:, 7:], return_lse=True)
     expected, expected_lse, _ = oracle_pipeline.attend(prepared, return_lse=True)
     assert relative_l2(to_numpy(out[1:, 21:]), expected) < 1e-3
