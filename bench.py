@@ -1034,6 +1034,8 @@ def main():
                           "(profiles/attention_dense_32k_clock.md); kernel_ms_zero_inputs is the same launch on "
                           "all-zero operands, same cycle count at the full clock",
             "kernel_ms_zero_inputs": zero_ms,
+            # same cycles at 2.4 GHz over the cycles at the sustained clock: an estimate of sustained / nominal clock
+            "clock_ratio_estimate": None if zero_ms is None else zero_ms / kernel_ms,
             "achieved": achieved_tops,
             "peak": INT8_MFMA_PEAK_TOPS,
             "unit": "TOP/s",
