@@ -96,22 +96,28 @@ __global__ __launch_bounds__(256) void offsets_summary_kernel(const int32_t* __r
     }
     __syncthreads();
   }
-  for (int base = 0; base < rows; base += 256) {
-    const int row = base + tid;
-    const int value = row < rows ? counts[row] : 0;
-    scan[tid] = value;
+  // Exclusive scan of the counts: every thread owns a run of consecutive rows, the 256 run
+  // totals are scanned through LDS once, and every thread then writes its run (integer sums:
+  // any order gives the same offsets).
+  const int run = (rows + 255) / 256;
+  const int first = tid * run, last = min(first + run, rows);
+  int mine = 0;
+  for (int row = first; row < last; ++row) mine += counts[row];
+  scan[tid] = mine;
+  __syncthreads();
+  for (int offset = 1; offset < 256; offset <<= 1) {
+    const int add = tid >= offset ? scan[tid - offset] : 0;
     __syncthreads();
-    for (int offset = 1; offset < 256; offset <<= 1) {
-      const int add = tid >= offset ? scan[tid - offset] : 0;
-      __syncthreads();
-      scan[tid] += add;
-      __syncthreads();
-    }
-    if (row < rows) row_offsets[row] = carry + scan[tid] - value;
-    __syncthreads();
-    if (tid == 255) carry += scan[255];
+    scan[tid] += add;
     __syncthreads();
   }
+  int running = scan[tid] - mine;
+  for (int row = first; row < last; ++row) {
+    row_offsets[row] = running;
+    running += counts[row];
+  }
+  if (tid == 255) carry = scan[255];
+  __syncthreads();
   if (tid == 0) {
     row_offsets[rows] = carry;
     summary[0] = selected_sums[0];
