@@ -993,8 +993,15 @@ def main():
     packed = risa.prequantize_int8_attention(q, k, v, v_quantization=args.mode)
     stream = torch.cuda.current_stream(device)
     kernel_ms = kernel_time(torch, risa, packed, args.steps)
-    zero_ms = None
+    zero_ms = compiled_ms = None
     if not args.no_side_measurements:
+        # the same launch through the compiler-scheduled tile loop (diagnostic switch of the library,
+        # read at every launch): what the hand-scheduled loop is worth on this machine
+        os.environ["RISA_COMPILED_LOOP"] = "1"
+        try:
+            compiled_ms = kernel_time(torch, risa, packed, args.steps)
+        finally:
+            del os.environ["RISA_COMPILED_LOOP"]
         zero_ms = kernel_time(torch, risa, risa.prequantize_int8_attention(
             torch.zeros_like(q), torch.zeros_like(k), torch.zeros_like(v), v_quantization=args.mode), args.steps)
     begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -1033,6 +1040,11 @@ def main():
                           "clock the part sustains under this load: about 1.9 GHz against 2.4 GHz nominal "
                           "(profiles/attention_dense_32k_clock.md); kernel_ms_zero_inputs is the same launch on "
                           "all-zero operands, same cycle count at the full clock",
+            "kernel_ms_compiled_loop": compiled_ms,
+            "kernel_ms_compiled_loop_note": "RISA_COMPILED_LOOP=1: every tile through the compiler-scheduled loop of this "
+                                            "build, which forms its copy offsets per tile and runs about 2.5 % behind the "
+                                            "previous library's loop (an A/B of the two libraries on one machine: 5.44 "
+                                            "against 5.15 ms)",
             "kernel_ms_zero_inputs": zero_ms,
             # same cycles at 2.4 GHz over the cycles at the sustained clock: an estimate of sustained / nominal clock
             "clock_ratio_estimate": None if zero_ms is None else zero_ms / kernel_ms,
