@@ -632,7 +632,21 @@ __global__ __launch_bounds__(256, (D == 256 ? 1 : D == 64 && MASK_MODE == kMaskL
       const bool on_diagonal = p.causal && tile * CTA_K + CTA_K - 1 > first_query;
       const bool partial = LAST && (tile + 1) * CTA_K > p.k_len;
       float mx = kRowFloor;
-      if (!has_mask && !on_diagonal && !partial) {
+      // A key-only mask whose additive row is zero over this whole tile (a padding mask leaves
+      // every tile but the one at its edge like that) changes nothing in it: x + 0 = x bit for
+      // bit (a zero of either sign; only the sign of a zero sum can differ, which neither the
+      // maximum nor the exponential sees).  One LDS read per wavefront and tile decides.
+      [[maybe_unused]] bool zero_row = false;
+      if constexpr (MASK_DT == kKeyBias) {
+        if (!on_diagonal && !partial) {
+          const float* bias_row = reinterpret_cast<const float*>(
+              lds + (it & 1) * Shape::kStageBytes + 2 * Shape::kTileBytes + Shape::kSeedBytes);
+          const v4i probe = *reinterpret_cast<const v4i*>(bias_row + (lane & (CTA_K / 4 - 1)) * 4);
+          const bool nonzero = (static_cast<uint32_t>(probe[0] | probe[1] | probe[2] | probe[3]) << 1) != 0;
+          zero_row = __builtin_amdgcn_ballot_w64(nonzero) == 0;
+        }
+      }
+      if ((!has_mask || zero_row) && !on_diagonal && !partial) {
 #pragma unroll
         for (int rb = 0; rb < RB; ++rb)
 #pragma unroll

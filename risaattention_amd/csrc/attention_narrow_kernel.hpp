@@ -350,7 +350,18 @@ __global__ __launch_bounds__(64 * WAVES * KSPLIT) void attention_narrow_kernel(c
       const bool partial = LAST && (tile + 1) * CTA_K > p.k_len;
       const int key0 = tile * CTA_K + 32 * (grp >> 1) + 4 * (grp & 1);
       float mx = kRowFloor;
-      if (MASK_DT < 0 && !on_diagonal && !partial) {
+      // (a key-only mask whose additive row is zero over this whole tile changes nothing in it:
+      // as in the wide kernel, one LDS read per wavefront and tile decides)
+      [[maybe_unused]] bool zero_row = false;
+      if constexpr (MASK_DT == kKeyBias) {
+        if (!on_diagonal && !partial) {
+          const int* whole_row = reinterpret_cast<const int*>(lds + (it & 1) * Shape::kStageBytes + Shape::kMaskOffset);
+          const v4i probe = *reinterpret_cast<const v4i*>(whole_row + (lane & (CTA_K / 4 - 1)) * 4);
+          const bool nonzero = (static_cast<uint32_t>(probe[0] | probe[1] | probe[2] | probe[3]) << 1) != 0;
+          zero_row = __builtin_amdgcn_ballot_w64(nonzero) == 0;
+        }
+      }
+      if ((MASK_DT < 0 || zero_row) && !on_diagonal && !partial) {
 #pragma unroll
         for (int kb = 0; kb < KB; ++kb)
 #pragma unroll

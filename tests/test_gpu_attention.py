@@ -209,6 +209,34 @@ def test_key_bias_large_tile_and_lse(risa):
         torch.testing.assert_close(lse, mask.logsumexp(-1).expand(1, 2, 17), atol=0.01, rtol=0)
 
 
+@pytest.mark.parametrize("dim,heads,q_len,k_len", [(128, 40, 1024, 1500), (128, 2, 200, 1500), (64, 48, 900, 700),
+                                                   (256, 4, 300, 1500), (64, 2, 100, 330)])
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("kind", ["padding", "bias"])
+def test_key_only_masks_with_untouched_tiles(risa, dim, heads, q_len, k_len, causal, kind):
+    """A key-only mask that leaves whole key tiles untouched (an additive row of zeros there: the
+    kernels skip the addition for such a tile) beside tiles with hidden keys, with finite terms,
+    and a hidden tail; 32-query and 16-query kernels, 64- and 128-key tiles, every head dim."""
+    q = seeded((1, heads, q_len, dim), torch.bfloat16, 41, scale=1.5)
+    k = seeded((1, 2, k_len, dim), torch.bfloat16, 42, scale=1.5)
+    v = seeded((1, 2, k_len, dim), torch.bfloat16, 43, offset=0.5)
+    if kind == "padding":
+        mask = torch.ones(1, 1, 1, k_len, dtype=torch.bool, device="cuda")
+        mask[..., k_len - k_len // 7:] = False
+        mask[..., 70:75] = False
+    else:
+        mask = torch.zeros(1, 1, 1, k_len, device="cuda")
+        mask[..., 130:190] = seeded((60,), torch.float32, 44)
+        mask[..., 3] = -0.0
+        mask[..., k_len - 77:] = float("-inf")
+    out, lse = risa.int8_attention(q, k, v, attn_mask=mask, is_causal=causal, return_lse=True)
+    checked = slice(heads - 1, heads)
+    prepared = oracle_prequantize(q[:, checked], k[:, 1:], v[:, 1:], attn_mask=mask, is_causal=causal, return_lse=True)
+    expected, expected_lse, _ = oracle_pipeline.attend(prepared, return_lse=True)
+    assert relative_l2(to_numpy(out[:, checked]), expected) < TOLERANCE
+    assert relative_l2(to_numpy(lse[:, checked]), expected_lse) < TOLERANCE
+
+
 def test_lse_restores_shifted_keys_and_empty_rows(risa):
     """reference tests/cuda/test_risa_attention.py:181-193."""
     from risaattention_amd.policy import apply_score_mask
