@@ -73,7 +73,8 @@ S_TNEXT, S_TAFTER, S_INDEX, S_LAST = 70, 71, 72, 73  # sparse: next tile, the on
 S_KWAVE, S_VWAVE = 74, 76      # pairs: sparse: this wave's share of the K and V sources
 LAST_SGPR = 77
 S_STATS, S_QLEN8, S_CAPEXEC = 78, 80, 82  # capture: pair: this wavefront's statistics rows of the tile; bytes per tile; pair: lanes that store
-LAST_SGPR_CAPTURE = 83
+S_CAPNOW = 84                  # capture: pair: the lanes that store at the next statistics store (none before the first tile)
+LAST_SGPR_CAPTURE = 85
 
 
 class Emitter:
@@ -157,6 +158,31 @@ def add64(e, pair, amount):
     e.ins(f"s_addc_u32 s{pair + 1}, s{pair + 1}, 0")
 
 
+def statistics_store(e):
+    """Capturing launch: the statistics of the tile walked last — the row's sum of probability
+    bytes (both halves of the wavefront) and the tile maximum, eight bytes per query, tile-major.
+    Issued at the top of the next tile (and once behind the loop), where the row sum and the tile
+    maximum are still in their registers: a store issued at the end of its own tile would be
+    waited for at the next barrier, a few hundred cycles later, with the copies (stores and loads
+    share the counter); issued here it has a whole tile to complete.  Before the first tile the
+    lanes that store are none."""
+    e.valu(f"v_mov_b32_e32 v{T[2]}, v{V_ROWSUM}", [T[2]])
+    e.valu(f"v_mov_b32_e32 v{T[1]}, v{V_ROWSUM}", [T[1]])
+    e.nop(2)
+    e.valu(f"v_permlane32_swap_b32_e32 v{T[2]}, v{T[1]}", [T[2], T[1]])
+    e.nop(2)
+    e.valu(f"v_add_u32_e32 v{T[2]}, v{T[2]}, v{T[1]}", [T[2]])
+    e.valu(f"v_mov_b32_e32 v{T[3]}, v{V_MX0}", [T[3]])
+    e.valu(f"v_mbcnt_lo_u32_b32 v{T[0]}, -1, 0", [T[0]])
+    e.valu(f"v_lshlrev_b32_e32 v{T[0]}, 3, v{T[0]}", [T[0]])  # lane * 8 (the lanes that store are 0..31)
+    e.ins(f"s_mov_b64 s[{S_SAVEEXEC}:{S_SAVEEXEC + 1}], exec")
+    e.ins(f"s_mov_b64 exec, s[{S_CAPNOW}:{S_CAPNOW + 1}]")
+    e.ins(f"global_store_dwordx2 v{T[0]}, v[{T[2]}:{T[3]}], s[{S_STATS}:{S_STATS + 1}]")
+    e.ins(f"s_mov_b64 exec, s[{S_SAVEEXEC}:{S_SAVEEXEC + 1}]")
+    e.ins(f"s_add_u32 s{S_STATS}, s{S_STATS}, s{S_QLEN8}")
+    e.ins(f"s_addc_u32 s{S_STATS + 1}, s{S_STATS + 1}, 0")
+
+
 def tile_body(e, stage, args, label):
     """One tile held in LDS stage `stage`; its copies fill the other stage with the next tile."""
     other = stage ^ 1
@@ -169,6 +195,8 @@ def tile_body(e, stage, args, label):
     for kk in range(4):
         for rb in range(4):
             e.ds_read(ACC[kk] + rb * 4, V_A[kk], base + rb * 4096)
+    if args.capture:
+        statistics_store(e)
     if args.sparse:
         # sources of the next listed tile: bases of the head (with this wave's share) + tile * stride
         e.ins(f"s_mov_b32 s{S_TNEXT}, s{S_TAFTER}")
@@ -354,24 +382,6 @@ def tile_body(e, stage, args, label):
     for cb in range(4):
         e.wait_lds(VF[cb])
         e.mfma(ACC[cb], VF[cb], PK[1], ACC[cb])
-    if args.capture:
-        # per-tile statistics of pattern construction: the row's sum of probability bytes (both halves
-        # of the wavefront) and the tile maximum, eight bytes per query, tile-major
-        e.valu(f"v_mov_b32_e32 v{T[2]}, v{V_ROWSUM}", [T[2]])
-        e.valu(f"v_mov_b32_e32 v{T[1]}, v{V_ROWSUM}", [T[1]])
-        e.nop(2)
-        e.valu(f"v_permlane32_swap_b32_e32 v{T[2]}, v{T[1]}", [T[2], T[1]])
-        e.nop(2)
-        e.valu(f"v_add_u32_e32 v{T[2]}, v{T[2]}, v{T[1]}", [T[2]])
-        e.valu(f"v_mov_b32_e32 v{T[3]}, v{V_MX0}", [T[3]])
-        e.valu(f"v_mbcnt_lo_u32_b32 v{T[0]}, -1, 0", [T[0]])
-        e.valu(f"v_lshlrev_b32_e32 v{T[0]}, 3, v{T[0]}", [T[0]])  # lane * 8 (the lanes that store are 0..31)
-        e.ins(f"s_mov_b64 s[{S_SAVEEXEC}:{S_SAVEEXEC + 1}], exec")
-        e.ins(f"s_mov_b64 exec, s[{S_CAPEXEC}:{S_CAPEXEC + 1}]")
-        e.ins(f"global_store_dwordx2 v{T[0]}, v[{T[2]}:{T[3]}], s[{S_STATS}:{S_STATS + 1}]")
-        e.ins(f"s_mov_b64 exec, s[{S_SAVEEXEC}:{S_SAVEEXEC + 1}]")
-        e.ins(f"s_add_u32 s{S_STATS}, s{S_STATS}, s{S_QLEN8}")
-        e.ins(f"s_addc_u32 s{S_STATS + 1}, s{S_STATS + 1}, 0")
     e.valu(f"v_cvt_f32_u32_e32 v{T[0]}, v{V_ROWSUM}", [T[0]])
     e.valu(f"v_fmac_f32_e32 v{V_DPART}, v{T[0]}, v{V_TSCALE}", [V_DPART])
     # ---- K scales (and list entry) of the next tile: waited for at the next barrier ------------------
@@ -398,6 +408,8 @@ def tile_body(e, stage, args, label):
                 e.valu(f"v_sub_f32_e32 v{T[j]}, v{ACC[cb] + i + j}, v{V_SEEDVAL}", [T[j]])
             for j in range(4):
                 e.valu(f"v_fmac_f32_e32 v{O[cb] + i + j}, v{T[j]}, v{V_TSCALE}", [O[cb] + i + j])
+    if args.capture:
+        e.ins(f"s_mov_b64 s[{S_CAPNOW}:{S_CAPNOW + 1}], s[{S_CAPEXEC}:{S_CAPEXEC + 1}]")
 
 
 def generate(args):
@@ -418,6 +430,10 @@ def generate(args):
         e.ins(f"s_mov_b64 s[{S_STATS}:{S_STATS + 1}], %[stats]")
         e.ins(f"s_mov_b32 s{S_QLEN8}, %[qlen8]")
         e.ins(f"s_mov_b64 s[{S_CAPEXEC}:{S_CAPEXEC + 1}], %[capexec]")
+        # the store at the top of the first tile has no lanes and moves the pointer to tile 0
+        e.ins(f"s_mov_b64 s[{S_CAPNOW}:{S_CAPNOW + 1}], 0")
+        e.ins(f"s_sub_u32 s{S_STATS}, s{S_STATS}, s{S_QLEN8}")
+        e.ins(f"s_subb_u32 s{S_STATS + 1}, s{S_STATS + 1}, 0")
     # LDS base: lane 0 of the seed address register holds base + SEED_BIAS
     e.ins(f"v_readfirstlane_b32 s{S_LDS}, v{V_SEEDADDR}")
     e.ins(f"s_sub_u32 s{S_LDS}, s{S_LDS}, {SEED_BIAS}")
@@ -462,6 +478,8 @@ def generate(args):
     e.raw("Lrisa_done_%=:")
     e.ins("s_waitcnt lgkmcnt(0)")
     e.ins("s_setprio 0")
+    if args.capture:
+        statistics_store(e)  # of the last tile walked here
     return e
 
 

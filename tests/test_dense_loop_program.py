@@ -154,8 +154,8 @@ def interpret(program, operands, wave, padded, memory):
             total = low32(args[1]) + low32(args[2]) + (state["scc"] if op == "s_addc_u32" else 0)
             state["scc"] = total >> 32
             assign(args[0], total)
-        elif op == "s_sub_u32":
-            total = low32(args[1]) - low32(args[2])
+        elif op in ("s_sub_u32", "s_subb_u32"):
+            total = low32(args[1]) - low32(args[2]) - (state["scc"] if op == "s_subb_u32" else 0)
             state["scc"] = int(total < 0)
             assign(args[0], total)
         elif op == "s_min_u32":
@@ -338,9 +338,17 @@ def test_memory_accesses_match_the_compiled_loop(program_kind, tiles, padded):
                 assert of(phase, "sload") == [KS0 + 16 * following, LIST0 + 4 * min(index + 2, tiles - 1)], (wave, index)
             else:
                 assert of(phase, "sload") == [KS0 + 16 * following], (wave, index)
-            # (row sum and tile maximum in two consecutive registers, by the storing lanes only)
-            stores = [(234, [STATS0 + index * TILE_BYTES + 8 * lane for lane in range(20)])] if capture else []
-            assert of(phase, "store") == stores, (wave, index)
+        # statistics stores (row sum and tile maximum in two consecutive registers, by the storing
+        # lanes only): the one of tile t at the top of tile t+1, none of the lanes before the first
+        # tile, the last one behind the loop
+        stores = [event[2] for event in events if event[1] == "store"]
+        if capture:
+            assert stores == [(234, [])] + [(234, [STATS0 + index * TILE_BYTES + 8 * lane for lane in range(20)])
+                                            for index in range(tiles - 1)], wave
+            phases = [event[0] for event in events if event[1] == "store"]
+            assert phases == list(range(1, tiles)) + [tiles - 1]
+        else:
+            assert not stores
 
 
 def test_wait_states_after_matrix_instructions():
