@@ -166,15 +166,15 @@ def statistics_store(e):
     waited for at the next barrier, a few hundred cycles later, with the copies (stores and loads
     share the counter); issued here it has a whole tile to complete.  Before the first tile the
     lanes that store are none."""
-    e.valu(f"v_mov_b32_e32 v{T[2]}, v{V_ROWSUM}", [T[2]])
+    # (the row sum register is free by now: the swap may exchange halves in place; other
+    # instructions stand where the lane swap needs wait states before and after it)
     e.valu(f"v_mov_b32_e32 v{T[1]}, v{V_ROWSUM}", [T[1]])
-    e.nop(2)
-    e.valu(f"v_permlane32_swap_b32_e32 v{T[2]}, v{T[1]}", [T[2], T[1]])
-    e.nop(2)
-    e.valu(f"v_add_u32_e32 v{T[2]}, v{T[2]}, v{T[1]}", [T[2]])
-    e.valu(f"v_mov_b32_e32 v{T[3]}, v{V_MX0}", [T[3]])
     e.valu(f"v_mbcnt_lo_u32_b32 v{T[0]}, -1, 0", [T[0]])
     e.valu(f"v_lshlrev_b32_e32 v{T[0]}, 3, v{T[0]}", [T[0]])  # lane * 8 (the lanes that store are 0..31)
+    e.valu(f"v_permlane32_swap_b32_e32 v{V_ROWSUM}, v{T[1]}", [V_ROWSUM, T[1]])
+    e.valu(f"v_mov_b32_e32 v{T[3]}, v{V_MX0}", [T[3]])
+    e.nop(1)
+    e.valu(f"v_add_u32_e32 v{T[2]}, v{V_ROWSUM}, v{T[1]}", [T[2]])
     e.ins(f"s_mov_b64 s[{S_SAVEEXEC}:{S_SAVEEXEC + 1}], exec")
     e.ins(f"s_mov_b64 exec, s[{S_CAPNOW}:{S_CAPNOW + 1}]")
     e.ins(f"global_store_dwordx2 v{T[0]}, v[{T[2]}:{T[3]}], s[{S_STATS}:{S_STATS + 1}]")
