@@ -997,11 +997,15 @@ def main():
     if not args.no_side_measurements:
         # the same launch through the compiler-scheduled tile loop (diagnostic switch of the library,
         # read at every launch): what the hand-scheduled loop is worth on this machine
+        before = os.environ.get("RISA_COMPILED_LOOP")
         os.environ["RISA_COMPILED_LOOP"] = "1"
         try:
             compiled_ms = kernel_time(torch, risa, packed, args.steps)
         finally:
-            del os.environ["RISA_COMPILED_LOOP"]
+            if before is None:
+                del os.environ["RISA_COMPILED_LOOP"]
+            else:
+                os.environ["RISA_COMPILED_LOOP"] = before
         zero_ms = kernel_time(torch, risa, risa.prequantize_int8_attention(
             torch.zeros_like(q), torch.zeros_like(k), torch.zeros_like(v), v_quantization=args.mode), args.steps)
     begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)

@@ -21,11 +21,15 @@ pytestmark = pytest.mark.gpu
 @contextmanager
 def compiled_loop():
     """Launches inside go through the compiler-scheduled tile loop."""
+    before = os.environ.get("RISA_COMPILED_LOOP")
     os.environ["RISA_COMPILED_LOOP"] = "1"
     try:
         yield
     finally:
-        del os.environ["RISA_COMPILED_LOOP"]
+        if before is None:
+            del os.environ["RISA_COMPILED_LOOP"]
+        else:
+            os.environ["RISA_COMPILED_LOOP"] = before
 
 
 @pytest.mark.parametrize("length", [2048, 2049, 2304, 4096, 4190])
