@@ -227,6 +227,21 @@ int risa_select_retained_mass(const float* sorted_mass, const int64_t* descendin
                               int row_count, int key_blocks, double theta, void* stream);
 
 /*
+ * The same selection over unsorted masses: sorts every row in the library first
+ * (descending, ties by ascending tile id, i.e. the order of a stable descending sort; the
+ * reference sorts with torch.sort in Python, src/risa_attention/sparse.py:24, and leaves ties
+ * open), then selects as risa_select_retained_mass does.  sorted_mass float32 and
+ * descending_indices int64, both [row_count, key_blocks], are outputs the caller provides.
+ * Rows of up to risa_sortable_key_blocks() tiles; longer rows are rejected (sort outside and
+ * call risa_select_retained_mass).
+ */
+int risa_sortable_key_blocks(void);
+int risa_sort_select_retained_mass(const float* masses, float* sorted_mass, int64_t* descending_indices,
+                                   int32_t* counts, uint8_t* support, double* row_totals,
+                                   int32_t* row_offsets, int32_t* block_indices, double* summary,
+                                   int row_count, int key_blocks, double theta, void* stream);
+
+/*
  * Active key tiles of a broadcast key mask.  Replaces
  * launch_prepare_key_mask_tiles (reference csrc/launchers.h:39-43,
  * csrc/kernels/key_mask_tiles.cu:45-61).

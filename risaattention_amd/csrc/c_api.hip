@@ -335,6 +335,27 @@ int risa_select_retained_mass(const float* sorted_mass, const int64_t* descendin
   return risa::launch_select_retained_mass(a, static_cast<hipStream_t>(stream));
 }
 
+int risa_sort_select_retained_mass(const float* masses, float* sorted_mass, int64_t* descending_indices,
+                                   int32_t* counts, uint8_t* support, double* row_totals,
+                                   int32_t* row_offsets, int32_t* block_indices, double* summary,
+                                   int row_count, int key_blocks, double theta, void* stream) {
+  if (row_count <= 0 || key_blocks <= 0)
+    return risa::fail("risa_sort_select_retained_mass: invalid shape, dtype, or stride");
+  if (static_cast<int64_t>(row_count) * key_blocks > INT32_MAX)
+    return risa::fail("risa_sort_select_retained_mass: matrix is too large");
+  if (key_blocks > risa::kSortableTiles)
+    return risa::fail("risa_sort_select_retained_mass: more than " + std::to_string(risa::kSortableTiles) +
+                      " key tiles per row: sort outside and call risa_select_retained_mass");
+  const int status = risa::launch_sort_rows(masses, sorted_mass, descending_indices, row_count, key_blocks,
+                                            static_cast<hipStream_t>(stream));
+  if (status != 0) return status;
+  risa::SelectArgs a{sorted_mass, descending_indices, counts,   support,    row_totals, row_offsets,
+                     block_indices, summary,          row_count, key_blocks, theta};
+  return risa::launch_select_retained_mass(a, static_cast<hipStream_t>(stream));
+}
+
+int risa_sortable_key_blocks(void) { return risa::kSortableTiles; }
+
 int risa_prepare_key_mask_tiles(const void* mask, int32_t* tiles, int batch, int q_heads,
                                 int key_length, int tile_size, int64_t stride_b, int64_t stride_h,
                                 int64_t stride_k, int mask_dtype, void* stream) {

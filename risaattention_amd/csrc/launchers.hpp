@@ -102,6 +102,10 @@ struct SelectArgs {
   double theta;
 };
 int launch_select_retained_mass(const SelectArgs& args, hipStream_t stream);
+// Most key tiles a row may have for the in-library sort (one workgroup, 32 KB of LDS).
+constexpr int kSortableTiles = 4096;
+int launch_sort_rows(const float* masses, float* sorted_mass, int64_t* order, int rows, int tiles,
+                     hipStream_t stream);
 
 int launch_key_mask_tiles(const void* mask, int32_t* tiles, int batch, int heads, int length,
                           int tile_size, int64_t stride_b, int64_t stride_h, int64_t stride_k,

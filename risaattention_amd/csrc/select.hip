@@ -69,6 +69,50 @@ __global__ __launch_bounds__(64) void select_rows_kernel(const float* __restrict
   }
 }
 
+// Descending order of every row's masses with ties by ascending tile id (what a stable
+// descending sort gives; the contract sorts with torch.sort in Python, reference
+// src/risa_attention/sparse.py:24, and documents ties as free): one workgroup per row, a bitonic
+// network over the row padded to a power of two in LDS.  Padding entries (-inf, ids past the row)
+// end up last and are not written.
+// THREADS: 64 for rows of up to 1024 entries (a single wavefront's barriers cost next to nothing
+// and sixteen such workgroups share a compute unit), 256 beyond.
+template <int THREADS>
+__global__ __launch_bounds__(THREADS) void sort_rows_kernel(const float* __restrict__ masses,
+                                                            float* __restrict__ sorted_mass,
+                                                            int64_t* __restrict__ order, int tiles, int padded) {
+  extern __shared__ unsigned char sort_lds[];
+  float* key = reinterpret_cast<float*>(sort_lds);
+  int* id = reinterpret_cast<int*>(key + padded);
+  const int tid = threadIdx.x;
+  const int64_t base = static_cast<int64_t>(blockIdx.x) * tiles;
+  for (int i = tid; i < padded; i += THREADS) {
+    key[i] = i < tiles ? masses[base + i] : -__builtin_inff();
+    id[i] = i;
+  }
+  __syncthreads();
+  for (int k = 2; k <= padded; k <<= 1) {
+    for (int j = k >> 1; j > 0; j >>= 1) {
+      for (int t = tid; t < padded / 2; t += THREADS) {
+        const int low = (t / j) * 2 * j + (t % j), high = low + j;
+        const float a = key[low], b = key[high];
+        const int ia = id[low], ib = id[high];
+        const bool b_first = b > a || (b == a && ib < ia);  // b belongs in front of a
+        const bool a_first = a > b || (a == b && ia < ib);
+        // the first half of every 2k block ends up in order, the second half reversed
+        if (((low & k) == 0) ? b_first : a_first) {
+          key[low] = b, key[high] = a;
+          id[low] = ib, id[high] = ia;
+        }
+      }
+      __syncthreads();
+    }
+  }
+  for (int i = tid; i < tiles; i += THREADS) {
+    sorted_mass[base + i] = key[i];
+    order[base + i] = id[i];
+  }
+}
+
 // Single workgroup: exclusive scan of the per-row counts and the FP64 summary
 // (pairwise tree over 256 partial sums, as in the contract).
 __global__ __launch_bounds__(256) void offsets_summary_kernel(const int32_t* __restrict__ counts,
@@ -387,6 +431,19 @@ int launch_key_bias(const void* mask, float* bias, int batch, int heads, int len
   key_bias_kernel<<<grid, 256, 0, stream>>>(mask, bias, length, padded, stride_b, stride_h, stride_k,
                                             dtype);
   return check_launch("risa_prepare_key_bias");
+}
+
+int launch_sort_rows(const float* masses, float* sorted_mass, int64_t* order, int rows, int tiles,
+                     hipStream_t stream) {
+  int padded = 2;
+  while (padded < tiles) padded <<= 1;
+  if (padded > kSortableTiles) return fail("risa_sort_select_retained_mass: more key tiles than one workgroup sorts");
+  if (padded <= 1024) {
+    sort_rows_kernel<64><<<rows, 64, static_cast<size_t>(padded) * 8, stream>>>(masses, sorted_mass, order, tiles, padded);
+  } else {
+    sort_rows_kernel<256><<<rows, 256, static_cast<size_t>(padded) * 8, stream>>>(masses, sorted_mass, order, tiles, padded);
+  }
+  return check_launch("risa_sort_select_retained_mass");
 }
 
 int launch_select_retained_mass(const SelectArgs& a, hipStream_t stream) {

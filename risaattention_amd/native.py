@@ -75,6 +75,8 @@ SIGNATURES = {
     ),
     "risa_selector_workspace_size": (_c_size, [_c_int]),
     "risa_select_retained_mass": (_c_int, [_c_ptr] * 8 + [_c_int, _c_int, _c_f64, _c_ptr]),
+    "risa_sortable_key_blocks": (_c_int, []),
+    "risa_sort_select_retained_mass": (_c_int, [_c_ptr] * 9 + [_c_int, _c_int, _c_f64, _c_ptr]),
     "risa_prepare_key_mask_tiles": (
         _c_int,
         [_c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_i64, _c_i64, _c_i64, _c_int, _c_ptr],

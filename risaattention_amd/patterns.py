@@ -24,20 +24,28 @@ def select_retained_mass_csr(masses: torch.Tensor, theta: float):
     """
     rows, tiles = masses.shape
     device = masses.device
-    sorted_mass, order = masses.sort(dim=-1, descending=True)
+    library = native.library()
+    # Rows that fit one workgroup are sorted inside the library (one launch; ties by ascending
+    # tile id); longer ones with torch.sort, as the reference does (sparse.py:24).
+    in_library = tiles <= library.risa_sortable_key_blocks() and masses.is_contiguous()
+    if in_library:
+        sorted_mass = torch.empty_like(masses)
+        order = torch.empty((rows, tiles), dtype=torch.int64, device=device)
+    else:
+        sorted_mass, order = masses.sort(dim=-1, descending=True)
     counts = torch.empty(rows, dtype=torch.int32, device=device)
     support = torch.empty((rows, tiles), dtype=torch.uint8, device=device)
     row_totals = torch.empty((rows, 2), dtype=torch.float64, device=device)
     row_offsets = torch.empty(rows + 1, dtype=torch.int32, device=device)
     storage = torch.empty(rows * tiles, dtype=torch.int32, device=device)
     summary = torch.empty(3, dtype=torch.float64, device=device)
-    native.check(
-        native.library().risa_select_retained_mass(
-            sorted_mass.data_ptr(), order.data_ptr(), counts.data_ptr(), support.data_ptr(),
-            row_totals.data_ptr(), row_offsets.data_ptr(), storage.data_ptr(), summary.data_ptr(),
-            rows, tiles, float(theta), native.current_stream(device),
-        )
-    )
+    outputs = (sorted_mass.data_ptr(), order.data_ptr(), counts.data_ptr(), support.data_ptr(),
+               row_totals.data_ptr(), row_offsets.data_ptr(), storage.data_ptr(), summary.data_ptr(),
+               rows, tiles, float(theta), native.current_stream(device))
+    if in_library:
+        native.check(library.risa_sort_select_retained_mass(masses.data_ptr(), *outputs))
+    else:
+        native.check(library.risa_select_retained_mass(*outputs))
     selected_mass, total_mass, selected_blocks = summary.tolist()
     return row_offsets, storage[: int(selected_blocks)], selected_mass / max(total_mass, 1e-20)
 

@@ -84,12 +84,34 @@ def test_block_mass_values_match_oracle(risa):
 
 
 @pytest.mark.parametrize("theta", [0.5, 0.99, 1.0])
-def test_selector_kernel_matches_oracle_exactly(risa, theta):
+@pytest.mark.parametrize("rows,tiles", [(531, 257), (40, 1), (9, 2), (77, 64), (33, 1000), (5, 4096)])
+def test_selector_kernel_matches_oracle_exactly(risa, theta, rows, tiles):
+    """Rows of up to 4096 tiles are sorted inside the library, ties by ascending tile id: the
+    order of the oracle's stable descending sort, so the CSR is equal entry for entry even with
+    repeated masses (a row of zeros, a row of one value, masses drawn from eight levels)."""
     from risaattention_amd.patterns import select_retained_mass_csr
 
     g = torch.Generator().manual_seed(1)
-    masses = (torch.rand(531, 257, generator=g) ** 6).cuda()
-    masses[7] = 0
+    masses = (torch.rand(rows, tiles, generator=g) ** 6)
+    masses[rows // 2] = 0
+    masses[rows // 3] = 0.25
+    masses[1] = (masses[1] * 8).floor() / 8
+    masses = masses.cuda()
+    row_offsets, block_indices, measured = select_retained_mass_csr(masses, theta)
+    ro, bi, expected_measured, _ = oracle_selection.select_retained_mass(masses.cpu().numpy(), theta)
+    np.testing.assert_array_equal(row_offsets.cpu().numpy(), ro)
+    np.testing.assert_array_equal(block_indices.cpu().numpy(), bi)
+    assert measured == pytest.approx(expected_measured, rel=1e-12)
+
+
+@pytest.mark.parametrize("theta", [0.5, 0.99])
+def test_selector_kernel_over_an_outside_sort(risa, theta):
+    """Rows longer than the library sorts take torch.sort, as in the reference: the CSR equals the
+    oracle's for that permutation."""
+    from risaattention_amd.patterns import select_retained_mass_csr
+
+    g = torch.Generator().manual_seed(2)
+    masses = (torch.rand(6, 4100, generator=g) ** 6).cuda()
     row_offsets, block_indices, measured = select_retained_mass_csr(masses, theta)
     order = masses.sort(dim=-1, descending=True).indices.cpu().numpy()
     ro, bi, expected_measured, _ = oracle_selection.select_retained_mass(masses.cpu().numpy(), theta, order=order)
